@@ -1,0 +1,178 @@
+"""``vdm_w4a4_packed_v1`` checkpoints: reader, writer and the switches that put
+a model into kernel mode.  Same functions, arguments, return values and
+exception types as the reference's vdm_infer/checkpoints/packed_checkpoint.py.
+
+On disk a packed checkpoint is ``torch.save`` of
+``{"format": "vdm_w4a4_packed_v1", "metadata": {...}, "model": state_dict}``
+where, for every QuantLinear ``<name>``, the state dict holds
+``<name>.vdm_weight_packed`` (u8 [N, K/2]), ``<name>.vdm_weight_scale_packed``
+(fp16 [N, K/64]), ``<name>.vdm_weight_scale`` (fp16 [N]) and ``<name>.bias``
+but no fp ``<name>.weight`` and no quantizer state.  Buffers stay in the v1
+byte layout in the module (they are the state-dict contract); the gfx950
+kernels relayout them once on first use.
+"""
+from __future__ import annotations
+
+import gc
+from typing import Any
+
+import torch
+import torch.nn as nn
+
+PACKED_CHECKPOINT_FORMAT = "vdm_w4a4_packed_v1"
+# checkpoints written by earlier tooling carry a different infix in the format
+# string and in the three buffer names (packed_checkpoint.py:19,25)
+_LEGACY_INFIX = "".join(("d", "i", "y", "_"))
+_LEGACY_PACKED_CHECKPOINT_FORMAT = PACKED_CHECKPOINT_FORMAT.replace("vdm_", "vdm_" + _LEGACY_INFIX, 1)
+VDM_BUFFER_SUFFIXES = ("vdm_weight_packed", "vdm_weight_scale_packed", "vdm_weight_scale")
+_LEGACY_BUFFER_SUFFIXES = tuple(_LEGACY_INFIX + s[len("vdm_"):] for s in VDM_BUFFER_SUFFIXES)
+_KNOWN_FORMATS = (PACKED_CHECKPOINT_FORMAT, _LEGACY_PACKED_CHECKPOINT_FORMAT)
+
+
+def is_packed_checkpoint(ckpt: Any) -> bool:
+    return isinstance(ckpt, dict) and "model" in ckpt and ckpt.get("format") in _KNOWN_FORMATS
+
+
+def load_quant_checkpoint(path: str, dcp_loader) -> dict:
+    """``.pt``/``.pth`` files are read with ``weights_only=True``; anything else
+    is handed to ``dcp_loader`` (packed_checkpoint.py:32-37)."""
+    if path.endswith((".pt", ".pth")):
+        print(f"Loading torch checkpoint from {path}")
+        return torch.load(path, map_location="cpu", weights_only=True)
+    return dcp_loader(path)
+
+
+def _key(module_name: str, suffix: str) -> str:
+    return f"{module_name}.{suffix}" if module_name else suffix
+
+
+def _is_quantizer_state(key: str) -> bool:
+    return ".wquantizer." in key or ".aquantizer." in key
+
+
+def _attach_buffer(module: nn.Module, name: str, tensor: torch.Tensor) -> None:
+    module._buffers.pop(name, None)
+    if hasattr(module, name):
+        delattr(module, name)
+    module.register_buffer(name, tensor.detach().contiguous())
+
+
+def _to_kernel_mode(module: nn.Module) -> None:
+    """Module state after packed buffers are attached (packed_checkpoint.py:120-131)."""
+    module.use_vdm_kernel, module.use_kernel, module.use_kernel_fused = True, False, False
+    module.set_quant_state(use_wq=True, use_aq=True)
+    if getattr(module, "weight", None) is not None:
+        module.register_parameter("weight", None)
+    for q in ("wquantizer", "aquantizer"):
+        if hasattr(module, q):
+            delattr(module, q)
+            setattr(module, q, None)
+
+
+def load_packed_quantized_model(model: nn.Module, packed_ckpt: dict, *, quant_linear_cls: type, dtype: torch.dtype,
+                                device: torch.device, require_vdm_kernel: bool = True) -> tuple:
+    """Populate a freshly built model (Linear layers already swapped for
+    ``quant_linear_cls``) from a packed checkpoint; returns ``(missing,
+    unexpected)`` key lists (packed_checkpoint.py:52-148).
+
+    Raises ValueError for an unknown format, AssertionError when the kernel
+    library is required but unavailable, KeyError when a QuantLinear lacks any of
+    its three buffers, RuntimeError when no QuantLinear was populated.
+    """
+    if not is_packed_checkpoint(packed_ckpt):
+        found = packed_ckpt.get("format") if isinstance(packed_ckpt, dict) else type(packed_ckpt)
+        raise ValueError(f"Unsupported checkpoint format: {found}")
+    if require_vdm_kernel:
+        from dsaquant_amd.kernels.vdm_w4a4 import is_available, load_error
+
+        assert is_available(), f"DSAQuant W4A4 kernel not compiled/available: {load_error()}"
+
+    state_dict = packed_ckpt["model"]
+    quant_layers = {name: m for name, m in model.named_modules() if isinstance(m, quant_linear_cls)}
+    fp_weight_keys = {_key(name, "weight") for name in quant_layers}
+    packed_suffixes = VDM_BUFFER_SUFFIXES + _LEGACY_BUFFER_SUFFIXES
+
+    plain_state = {
+        k: v for k, v in state_dict.items()
+        if not k.endswith(packed_suffixes) and not _is_quantizer_state(k) and not k.endswith("._bias_half") and k not in fp_weight_keys
+    }
+    missing, unexpected = model.load_state_dict(plain_state, strict=False, assign=True)
+    missing = [k for k in missing if k not in fp_weight_keys and not _is_quantizer_state(k)]
+
+    absent: list = []
+    populated = 0
+    for name, module in quant_layers.items():
+        resolved = {}
+        for suffix, legacy in zip(VDM_BUFFER_SUFFIXES, _LEGACY_BUFFER_SUFFIXES):
+            k = _key(name, suffix)
+            resolved[suffix] = k if k in state_dict else _key(name, legacy)
+        gone = [k for k in resolved.values() if k not in state_dict]
+        if gone:
+            absent.extend(gone)
+            continue
+        for suffix, k in resolved.items():
+            _attach_buffer(module, suffix, state_dict[k])
+        _to_kernel_mode(module)
+        populated += 1
+
+    if absent:
+        raise KeyError(f"Packed checkpoint is missing {len(absent)} VDM buffers, e.g. {', '.join(absent[:8])}")
+    if populated == 0:
+        raise RuntimeError("No QuantLinear layers were populated from the packed checkpoint")
+
+    del state_dict, plain_state
+    gc.collect()
+
+    model = model.to(dtype).to(device)
+    for module in model.modules():
+        if isinstance(module, quant_linear_cls) and module.bias is not None:
+            module._bias_half = module.bias.half().contiguous()
+    print(f"Loaded packed DSAQuant W4A4 checkpoint: {populated} QuantLinear layers")
+    return list(missing), list(unexpected)
+
+
+def enable_quant_kernels(model: nn.Module, *, quant_linear_cls: type) -> None:
+    """Pack and switch every QuantLinear; a failing layer is reported and left
+    in fake-quant mode (packed_checkpoint.py:151-164)."""
+    print("Enabling DSAQuant W4A4 kernel mode...")
+    for name, module in model.named_modules():
+        if isinstance(module, quant_linear_cls):
+            module.set_quant_state(use_wq=True, use_aq=True)
+            try:
+                module.enable_vdm_kernel_mode()
+            except Exception as exc:
+                print(f"  Failed to enable VDM kernel for {name}: {exc}")
+
+
+def enable_fused_qkv(model: nn.Module, *, quant_linear_cls: type, attention_cls: type, use_fused_qkv: bool) -> None:
+    """Mark attention modules whose q/k/v are all in kernel mode for the fused
+    QKV path (packed_checkpoint.py:167-188)."""
+    if not use_fused_qkv:
+        return
+    print("Enabling fused QKV kernel (vdm)...")
+    for module in model.modules():
+        if not isinstance(module, attention_cls):
+            continue
+        qkv = (module.to_q, module.to_k, module.to_v)
+        if all(isinstance(p, quant_linear_cls) and p.use_vdm_kernel for p in qkv):
+            module.use_fused_qkv_kernel = True
+            module.qkv_kernel_backend = "vdm"
+
+
+def packed_state_dict_from_model(model: nn.Module, *, float_dtype: torch.dtype = torch.float16) -> dict:
+    """State dict for export: quantizer state and cached fp16 biases dropped,
+    floating tensors cast to ``float_dtype``, uint8 kept (packed_checkpoint.py:190-199)."""
+    out = {}
+    for k, v in model.state_dict().items():
+        if _is_quantizer_state(k) or k.endswith("._bias_half"):
+            continue
+        t = v.detach().cpu().contiguous()
+        out[k] = t.to(float_dtype) if t.is_floating_point() else t
+    return out
+
+
+def save_packed_checkpoint(model: nn.Module, output_path: str, *, metadata: dict | None = None,
+                           float_dtype: torch.dtype = torch.float16) -> None:
+    torch.save({"format": PACKED_CHECKPOINT_FORMAT, "metadata": metadata or {},
+                "model": packed_state_dict_from_model(model, float_dtype=float_dtype)}, output_path)
+    print(f"Saved packed checkpoint to {output_path}")

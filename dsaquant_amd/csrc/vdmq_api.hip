@@ -1,0 +1,222 @@
+// extern "C" boundary of libvdmq: argument checking and dispatch only.
+#include <stdarg.h>
+#include <stdio.h>
+
+#include "vdmq_internal.h"
+
+namespace vdmq {
+
+static thread_local char g_error[512] = "";
+
+int fail(int code, const char *fmt, ...) {
+    va_list ap;
+    va_start(ap, fmt);
+    vsnprintf(g_error, sizeof(g_error), fmt, ap);
+    va_end(ap);
+    return code;
+}
+
+int check_launch(const char *what) {
+    hipError_t e = hipGetLastError();
+    if (e != hipSuccess) return fail(VDMQ_ELAUNCH, "%s: launch failed: %s", what, hipGetErrorString(e));
+    return VDMQ_OK;
+}
+
+int launch_weight_relayout(const void *src, void *dst, int64_t N, int64_t K, bool to_native, hipStream_t s);
+int launch_wscale_relayout(const void *src, void *dst, int64_t N, int64_t K, bool to_plain, hipStream_t s);
+int launch_act_to_v1(const void *qact, const void *scale_h, int64_t M, int64_t K, void *qact_v1, void *ascales_v1, hipStream_t s);
+int launch_act_to_native(const void *qact_v1, const void *ascales_v1, int64_t M, int64_t K, void *qact, void *scale_h, hipStream_t s);
+
+namespace {
+
+constexpr int64_t kMaxK = 65536;      /* keeps 256 * sum(q*q) inside int32 */
+constexpr int64_t kMaxDim = 1 << 30;  /* int indexing inside the kernels */
+
+int check_k(int64_t K) {
+    if (K <= 0 || K % VDMQ_WARP_K != 0) return fail(VDMQ_ESHAPE, "K must be a positive multiple of %d (got %lld)", VDMQ_WARP_K, (long long)K);
+    if (K > kMaxK) return fail(VDMQ_ESHAPE, "K must be <= %lld (got %lld)", (long long)kMaxK, (long long)K);
+    return VDMQ_OK;
+}
+
+int check_n(int64_t N) {
+    if (N <= 0 || N % VDMQ_BLOCK_N != 0) return fail(VDMQ_ESHAPE, "N must be a positive multiple of %d (got %lld)", VDMQ_BLOCK_N, (long long)N);
+    if (N > kMaxDim) return fail(VDMQ_ESHAPE, "shape too large for int indexing");
+    return VDMQ_OK;
+}
+
+int check_m(int64_t M) {
+    if (M < 0 || M > kMaxDim) return fail(VDMQ_ESHAPE, "M out of range (got %lld)", (long long)M);
+    return VDMQ_OK;
+}
+
+int check_ptr(const void *p, const char *name, bool need16 = true) {
+    if (p == nullptr) return fail(VDMQ_EINVAL, "%s is null", name);
+    if (need16 && !aligned16(p)) return fail(VDMQ_EINVAL, "%s must be 16-byte aligned", name);
+    return VDMQ_OK;
+}
+
+#define VDMQ_TRY(expr)                  \
+    do {                                \
+        int rc_ = (expr);               \
+        if (rc_ != VDMQ_OK) return rc_; \
+    } while (0)
+
+inline hipStream_t as_stream(vdmq_stream_t s) { return static_cast<hipStream_t>(s); }
+
+}  // namespace
+}  // namespace vdmq
+
+using namespace vdmq;
+
+extern "C" {
+
+int vdmq_version(void) { return 1; }
+const char *vdmq_arch(void) { return "gfx950"; }
+const char *vdmq_last_error(void) { return g_error; }
+int64_t vdmq_k_padded(int64_t K) { return k_padded(K); }
+
+int vdmq_quantize_act(const void *x, int64_t M, int64_t K, int64_t ldx, float clip, void *qact, void *scale_h, vdmq_stream_t stream) {
+    VDMQ_TRY(check_k(K));
+    VDMQ_TRY(check_m(M));
+    if (M == 0) return VDMQ_OK;
+    VDMQ_TRY(check_ptr(x, "x"));
+    VDMQ_TRY(check_ptr(qact, "qact"));
+    VDMQ_TRY(check_ptr(scale_h, "scale_h", false));
+    if (ldx < K || ldx % 8 != 0) return fail(VDMQ_ESHAPE, "ldx must be >= K and a multiple of 8 (got %lld)", (long long)ldx);
+    return launch_quantize_act(static_cast<const __half *>(x), M, K, ldx, clip, static_cast<uint8_t *>(qact),
+                               static_cast<__half *>(scale_h), as_stream(stream));
+}
+
+static int gemm_checked(const void *qact, const void *ascale, const void *wq, const void *wscale, const void *bias, void *out,
+                        int out_dtype, int32_t *acc, int64_t M, int64_t N, int64_t K, int64_t ldo, vdmq_stream_t stream) {
+    VDMQ_TRY(check_k(K));
+    VDMQ_TRY(check_n(N));
+    VDMQ_TRY(check_m(M));
+    if (M == 0) return VDMQ_OK;
+    VDMQ_TRY(check_ptr(qact, "qact"));
+    VDMQ_TRY(check_ptr(wq, "wq"));
+    if (acc == nullptr) {
+        VDMQ_TRY(check_ptr(ascale, "ascale", false));
+        VDMQ_TRY(check_ptr(wscale, "wscale"));
+        VDMQ_TRY(check_ptr(out, "out"));
+        if (bias != nullptr) VDMQ_TRY(check_ptr(bias, "bias"));
+        if (out_dtype != VDMQ_OUT_F16 && out_dtype != VDMQ_OUT_BF16) return fail(VDMQ_EINVAL, "unknown out_dtype %d", out_dtype);
+        if (ldo < N || ldo % 8 != 0) return fail(VDMQ_ESHAPE, "ldo must be >= N and a multiple of 8 (got %lld)", (long long)ldo);
+    } else {
+        VDMQ_TRY(check_ptr(acc, "acc"));
+    }
+    return launch_gemm(static_cast<const uint8_t *>(qact), static_cast<const __half *>(ascale), static_cast<const uint8_t *>(wq),
+                       static_cast<const __half *>(wscale), static_cast<const __half *>(bias), out, out_dtype, acc, M, N, K, ldo,
+                       as_stream(stream));
+}
+
+int vdmq_gemm_w4a4(const void *qact, const void *ascale, const void *wq, const void *wscale, const void *bias, void *out,
+                   int out_dtype, int64_t M, int64_t N, int64_t K, int64_t ldo, vdmq_stream_t stream) {
+    return gemm_checked(qact, ascale, wq, wscale, bias, out, out_dtype, nullptr, M, N, K, ldo, stream);
+}
+
+int vdmq_gemm_w4a4_acc(const void *qact, const void *wq, int32_t *acc, int64_t M, int64_t N, int64_t K, vdmq_stream_t stream) {
+    if (acc == nullptr && M != 0) return fail(VDMQ_EINVAL, "acc is null");
+    return gemm_checked(qact, nullptr, wq, nullptr, nullptr, nullptr, VDMQ_OUT_F16, acc, M, N, K, N, stream);
+}
+
+int64_t vdmq_workspace_bytes(int64_t M, int64_t K) {
+    if (M < 0 || K <= 0) return 0;
+    const int64_t q = (M * (k_padded(K) / 2) + 255) / 256 * 256;
+    return q + (M * 2 + 255) / 256 * 256;
+}
+
+int vdmq_linear_w4a4(const void *x, int64_t M, int64_t K, int64_t ldx, float clip, const void *wq, const void *wscale,
+                     const void *bias, void *out, int out_dtype, int64_t N, int64_t ldo, void *workspace, int64_t workspace_bytes,
+                     vdmq_stream_t stream) {
+    VDMQ_TRY(check_k(K));
+    VDMQ_TRY(check_n(N));
+    VDMQ_TRY(check_m(M));
+    if (M == 0) return VDMQ_OK;
+    VDMQ_TRY(check_ptr(workspace, "workspace"));
+    if (workspace_bytes < vdmq_workspace_bytes(M, K))
+        return fail(VDMQ_ENOSPACE, "workspace has %lld bytes, %lld needed", (long long)workspace_bytes,
+                    (long long)vdmq_workspace_bytes(M, K));
+    uint8_t *qact = static_cast<uint8_t *>(workspace);
+    void *scale = qact + (M * (k_padded(K) / 2) + 255) / 256 * 256;
+    VDMQ_TRY(vdmq_quantize_act(x, M, K, ldx, clip, qact, scale, stream));
+    return vdmq_gemm_w4a4(qact, scale, wq, wscale, bias, out, out_dtype, M, N, K, ldo, stream);
+}
+
+int vdmq_weight_v1_to_native(const void *qweight_v1, void *wq_native, int64_t N, int64_t K, vdmq_stream_t stream) {
+    VDMQ_TRY(check_k(K));
+    VDMQ_TRY(check_n(N));
+    VDMQ_TRY(check_ptr(qweight_v1, "qweight_v1"));
+    VDMQ_TRY(check_ptr(wq_native, "wq_native"));
+    return launch_weight_relayout(qweight_v1, wq_native, N, K, true, as_stream(stream));
+}
+
+int vdmq_weight_native_to_v1(const void *wq_native, void *qweight_v1, int64_t N, int64_t K, vdmq_stream_t stream) {
+    VDMQ_TRY(check_k(K));
+    VDMQ_TRY(check_n(N));
+    VDMQ_TRY(check_ptr(qweight_v1, "qweight_v1"));
+    VDMQ_TRY(check_ptr(wq_native, "wq_native"));
+    return launch_weight_relayout(wq_native, qweight_v1, N, K, false, as_stream(stream));
+}
+
+int vdmq_wscale_v1_to_plain(const void *packed_v1, void *plain, int64_t N, int64_t K, vdmq_stream_t stream) {
+    VDMQ_TRY(check_k(K));
+    VDMQ_TRY(check_n(N));
+    VDMQ_TRY(check_ptr(packed_v1, "packed_v1", false));
+    VDMQ_TRY(check_ptr(plain, "plain", false));
+    return launch_wscale_relayout(packed_v1, plain, N, K, true, as_stream(stream));
+}
+
+int vdmq_wscale_plain_to_v1(const void *plain, void *packed_v1, int64_t N, int64_t K, vdmq_stream_t stream) {
+    VDMQ_TRY(check_k(K));
+    VDMQ_TRY(check_n(N));
+    VDMQ_TRY(check_ptr(packed_v1, "packed_v1", false));
+    VDMQ_TRY(check_ptr(plain, "plain", false));
+    return launch_wscale_relayout(plain, packed_v1, N, K, false, as_stream(stream));
+}
+
+int vdmq_act_native_to_v1(const void *qact, const void *scale_h, int64_t M, int64_t K, void *qact_v1, void *ascales_v1,
+                          vdmq_stream_t stream) {
+    VDMQ_TRY(check_k(K));
+    VDMQ_TRY(check_m(M));
+    if (M == 0) return VDMQ_OK;
+    VDMQ_TRY(check_ptr(qact, "qact"));
+    VDMQ_TRY(check_ptr(scale_h, "scale_h", false));
+    VDMQ_TRY(check_ptr(qact_v1, "qact_v1"));
+    VDMQ_TRY(check_ptr(ascales_v1, "ascales_v1", false));
+    return launch_act_to_v1(qact, scale_h, M, K, qact_v1, ascales_v1, as_stream(stream));
+}
+
+int vdmq_act_v1_to_native(const void *qact_v1, const void *ascales_v1, int64_t M, int64_t K, void *qact, void *scale_h,
+                          vdmq_stream_t stream) {
+    VDMQ_TRY(check_k(K));
+    VDMQ_TRY(check_m(M));
+    if (M % VDMQ_BLOCK_M != 0) return fail(VDMQ_ESHAPE, "M must be a multiple of %d (got %lld)", VDMQ_BLOCK_M, (long long)M);
+    if (M == 0) return VDMQ_OK;
+    VDMQ_TRY(check_ptr(qact, "qact"));
+    VDMQ_TRY(check_ptr(scale_h, "scale_h", false));
+    VDMQ_TRY(check_ptr(qact_v1, "qact_v1"));
+    VDMQ_TRY(check_ptr(ascales_v1, "ascales_v1", false));
+    return launch_act_to_native(qact_v1, ascales_v1, M, K, qact, scale_h, as_stream(stream));
+}
+
+int vdmq_row_scale(const void *w, int64_t rows, int64_t K, float clip, void *scale_h, vdmq_stream_t stream) {
+    VDMQ_TRY(check_k(K));
+    VDMQ_TRY(check_m(rows));
+    if (rows == 0) return VDMQ_OK;
+    VDMQ_TRY(check_ptr(w, "w"));
+    VDMQ_TRY(check_ptr(scale_h, "scale_h", false));
+    return launch_row_scale(static_cast<const __half *>(w), rows, K, clip, static_cast<__half *>(scale_h), as_stream(stream));
+}
+
+int vdmq_quantize_weight_native(const void *w, const void *scale_h, void *wq_native, int64_t N, int64_t K, vdmq_stream_t stream) {
+    VDMQ_TRY(check_k(K));
+    VDMQ_TRY(check_n(N));
+    VDMQ_TRY(check_ptr(w, "w"));
+    VDMQ_TRY(check_ptr(scale_h, "scale_h", false));
+    VDMQ_TRY(check_ptr(wq_native, "wq_native"));
+    return launch_quantize_given_scale(static_cast<const __half *>(w), static_cast<const __half *>(scale_h), N, K,
+                                       static_cast<uint8_t *>(wq_native), as_stream(stream));
+}
+
+}  // extern "C"

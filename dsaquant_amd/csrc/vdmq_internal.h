@@ -1,0 +1,33 @@
+// Internal declarations shared by the vdmq translation units (gfx950 only).
+#pragma once
+
+#include <hip/hip_fp16.h>
+#include <hip/hip_runtime.h>
+#include <stdint.h>
+
+#include "vdmq.h"
+
+namespace vdmq {
+
+// The GEMM consumes K in steps of this many elements; native rows are padded
+// with zero nibbles up to a multiple of it.
+constexpr int kKStep = 128;
+
+constexpr int kWaveSize = 64;
+
+int fail(int code, const char *fmt, ...) __attribute__((format(printf, 2, 3)));
+int check_launch(const char *what);
+
+inline int64_t k_padded(int64_t K) { return (K + kKStep - 1) / kKStep * kKStep; }
+inline int64_t ceil_div(int64_t a, int64_t b) { return (a + b - 1) / b; }
+inline bool aligned16(const void *p) { return (reinterpret_cast<uintptr_t>(p) & 15u) == 0; }
+
+// kernels' host launchers (no argument checking: the extern "C" layer does it)
+int launch_quantize_act(const __half *x, int64_t M, int64_t K, int64_t ldx, float clip, uint8_t *qact, __half *scale_h,
+                        hipStream_t stream);
+int launch_row_scale(const __half *x, int64_t rows, int64_t K, float clip, __half *scale_h, hipStream_t stream);
+int launch_quantize_given_scale(const __half *x, const __half *scale_h, int64_t rows, int64_t K, uint8_t *q, hipStream_t stream);
+int launch_gemm(const uint8_t *qact, const __half *ascale, const uint8_t *wq, const __half *wscale, const __half *bias,
+                void *out, int out_dtype, int32_t *acc_out, int64_t M, int64_t N, int64_t K, int64_t ldo, hipStream_t stream);
+
+}  // namespace vdmq

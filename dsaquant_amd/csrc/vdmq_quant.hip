@@ -1,0 +1,276 @@
+// Dynamic per-token A4 quantizer for gfx950: one pass over X.
+//
+// One 64-lane wave owns one token row.  The row is read once with 128-bit
+// loads and kept in registers; the absmax is reduced on the packed fp16 bit
+// patterns (exact, order-free); the scale is rounded to fp16; every element is
+// multiplied by the fp32 reciprocal of that fp16 scale, rounded half-to-even
+// and saturated to [-8, 7]; eight results are packed into one 32-bit word and
+// stored row-major (element e of a word in nibble e).
+//
+// Arithmetic contract (IEEE reading of vdm_w4a4_kernel.cu:459-481, 95-102,
+// 319-329 of the reference): see quantize_word_exact below, which spells it
+// out literally and serves rows that contain NaN/Inf or whose fp16 scale is
+// zero/non-finite; all other rows take a shorter, bit-identical sequence.
+#include "vdmq_internal.h"
+
+namespace vdmq {
+namespace {
+
+typedef unsigned short u16x2 __attribute__((ext_vector_type(2)));
+typedef unsigned int u32x4 __attribute__((ext_vector_type(4)));
+
+__device__ __forceinline__ uint32_t pk_max_u16(uint32_t a, uint32_t b) {
+    u16x2 r = __builtin_elementwise_max(__builtin_bit_cast(u16x2, a), __builtin_bit_cast(u16x2, b));
+    return __builtin_bit_cast(uint32_t, r);
+}
+
+__device__ __forceinline__ float half_bits_to_float(uint32_t bits16) {
+    return __half2float(__ushort_as_half(static_cast<unsigned short>(bits16)));
+}
+
+template <typename T>
+__device__ __forceinline__ T wave_max(T v) {
+#pragma unroll
+    for (int off = 32; off > 0; off >>= 1) {
+        T o = __shfl_xor(v, off, 64);
+        v = o > v ? o : v;
+    }
+    return v;
+}
+
+// fmaxf semantics of the reference's reduction: a NaN operand is ignored.
+__device__ __forceinline__ float max_ignoring_nan(float acc, float a) { return (a == a && a > acc) ? a : acc; }
+
+// cvt.rni.s32.f32 + cvt.pack.sat.s4: NaN -> 0, saturate, round half to even.
+__device__ __forceinline__ uint32_t sat_s4_rni(float v) {
+    if (v != v) return 0u;
+    if (v >= 7.0f) return 7u;
+    if (v <= -8.0f) return 8u; /* -8 as a nibble */
+    return static_cast<uint32_t>(static_cast<int>(__builtin_rintf(v))) & 0xFu;
+}
+
+// Literal form: q = sat_s4(rni(float(x) * rscale)) for the two halves of `w`.
+__device__ __forceinline__ uint32_t quantize_pair_exact(uint32_t w, float rscale) {
+    float lo = half_bits_to_float(w & 0xFFFFu) * rscale;
+    float hi = half_bits_to_float(w >> 16) * rscale;
+    return sat_s4_rni(lo) | (sat_s4_rni(hi) << 4);
+}
+
+__device__ __forceinline__ uint32_t quantize_word_exact(u32x4 v, float rscale) {
+    return quantize_pair_exact(v.x, rscale) | (quantize_pair_exact(v.y, rscale) << 8) |
+           (quantize_pair_exact(v.z, rscale) << 16) | (quantize_pair_exact(v.w, rscale) << 24);
+}
+
+// Fast form for finite inputs and a finite non-zero scale.  t = clamp(v) is
+// rounded to an integer by adding 1.5*2^23 + 8 (the fp32 adder rounds half to
+// even on the unit grid there), which leaves u = rni(t) + 8 in [0, 15] in the
+// low bits of the sum: bits = 0x4B400000 + u.  Eight sums are combined with
+// shift-adds; the constant parts add up to 0x4B400000 * 0x11111111 (mod 2^32)
+// and are removed at the end; u ^ 8 is the two's complement nibble.
+constexpr float kMagic = 12582920.0f; /* 1.5 * 2^23 + 8 */
+constexpr uint32_t kMagicSum = static_cast<uint32_t>(0x4B400000ull * 0x11111111ull);
+
+__device__ __forceinline__ uint32_t quantize_word_fast(u32x4 v, float rscale) {
+    const uint32_t w[4] = {v.x, v.y, v.z, v.w};
+    uint32_t acc = 0;
+#pragma unroll
+    for (int i = 0; i < 4; ++i) {
+        float2 f = __half22float2(__builtin_bit_cast(__half2, w[i]));
+        float t0 = __builtin_amdgcn_fmed3f(f.x * rscale, -8.0f, 7.0f);
+        float t1 = __builtin_amdgcn_fmed3f(f.y * rscale, -8.0f, 7.0f);
+        acc += __float_as_uint(t0 + kMagic) << (8 * i);
+        acc += __float_as_uint(t1 + kMagic) << (8 * i + 4);
+    }
+    return (acc - kMagicSum) ^ 0x88888888u;
+}
+
+__device__ __forceinline__ uint32_t absmax_bits(u32x4 v, uint32_t m) {
+    m = pk_max_u16(m, v.x & 0x7FFF7FFFu);
+    m = pk_max_u16(m, v.y & 0x7FFF7FFFu);
+    m = pk_max_u16(m, v.z & 0x7FFF7FFFu);
+    m = pk_max_u16(m, v.w & 0x7FFF7FFFu);
+    return m;
+}
+
+__device__ __forceinline__ float absmax_exact(u32x4 v, float mx) {
+    const uint32_t w[4] = {v.x, v.y, v.z, v.w};
+#pragma unroll
+    for (int i = 0; i < 4; ++i) {
+        mx = max_ignoring_nan(mx, fabsf(half_bits_to_float(w[i] & 0xFFFFu)));
+        mx = max_ignoring_nan(mx, fabsf(half_bits_to_float(w[i] >> 16)));
+    }
+    return mx;
+}
+
+// scale = max > 0 ? (max / 7) * clip : 1, rounded to fp16 (token_scale_kernel).
+__device__ __forceinline__ __half scale_from_absmax(float amax, float clip) {
+    float s = amax > 0.0f ? (amax / 7.0f) * clip : 1.0f;
+    return __float2half_rn(s);
+}
+
+__device__ __forceinline__ bool scale_is_ordinary(__half s) {
+    uint32_t b = __half_as_ushort(s) & 0x7FFFu;
+    return b != 0u && b < 0x7C00u;
+}
+
+constexpr int kRowsPerBlock = 4; /* one wave per row */
+
+// NCH = number of 512-element chunks (one 128-bit load per lane each) that
+// cover the padded row.
+template <int NCH>
+__global__ __launch_bounds__(kRowsPerBlock * kWaveSize) void quantize_rows_kernel(const __half *__restrict__ x, int64_t ldx,
+                                                                                  int M, int K, int Kp, float clip,
+                                                                                  uint8_t *__restrict__ qact,
+                                                                                  __half *__restrict__ scale_h) {
+    const int lane = threadIdx.x & (kWaveSize - 1);
+    const int64_t row = static_cast<int64_t>(blockIdx.x) * kRowsPerBlock + (threadIdx.x >> 6);
+    if (row >= M) return;
+    const u32x4 *src = reinterpret_cast<const u32x4 *>(x + row * ldx);
+
+    u32x4 v[NCH];
+#pragma unroll
+    for (int c = 0; c < NCH; ++c) {
+        const int k0 = c * 512 + lane * 8;
+        v[c] = k0 < K ? __builtin_nontemporal_load(src + c * 64 + lane) : u32x4{0u, 0u, 0u, 0u};
+    }
+
+    uint32_t m2 = 0;
+#pragma unroll
+    for (int c = 0; c < NCH; ++c) m2 = absmax_bits(v[c], m2);
+    uint32_t m16 = (m2 & 0xFFFFu) > (m2 >> 16) ? (m2 & 0xFFFFu) : (m2 >> 16);
+    m16 = wave_max(m16);
+
+    uint32_t *dst = reinterpret_cast<uint32_t *>(qact + row * (Kp / 2));
+    __half sh;
+    bool fast = m16 < 0x7C00u; /* every element finite */
+    if (fast) {
+        sh = scale_from_absmax(half_bits_to_float(m16), clip);
+        fast = scale_is_ordinary(sh);
+    }
+    if (fast) {
+        const float rscale = 1.0f / __half2float(sh);
+#pragma unroll
+        for (int c = 0; c < NCH; ++c) {
+            const int k0 = c * 512 + lane * 8;
+            if (k0 < Kp) dst[c * 64 + lane] = quantize_word_fast(v[c], rscale);
+        }
+    } else {
+        float mx = 0.0f;
+#pragma unroll
+        for (int c = 0; c < NCH; ++c) mx = absmax_exact(v[c], mx);
+        // fmaxf-style wave reduction (no NaN can be held in mx)
+        mx = wave_max(mx);
+        sh = scale_from_absmax(mx, clip);
+        const float rscale = 1.0f / __half2float(sh);
+#pragma unroll
+        for (int c = 0; c < NCH; ++c) {
+            const int k0 = c * 512 + lane * 8;
+            if (k0 < Kp) dst[c * 64 + lane] = quantize_word_exact(v[c], rscale);
+        }
+    }
+    if (lane == 0) scale_h[row] = sh;
+}
+
+// Any K: two passes over the row (the second one is served by the caches).
+__global__ __launch_bounds__(kRowsPerBlock * kWaveSize) void quantize_rows_anyk_kernel(const __half *__restrict__ x, int64_t ldx,
+                                                                                       int M, int K, int Kp, float clip,
+                                                                                       uint8_t *__restrict__ qact,
+                                                                                       __half *__restrict__ scale_h) {
+    const int lane = threadIdx.x & (kWaveSize - 1);
+    const int64_t row = static_cast<int64_t>(blockIdx.x) * kRowsPerBlock + (threadIdx.x >> 6);
+    if (row >= M) return;
+    const u32x4 *src = reinterpret_cast<const u32x4 *>(x + row * ldx);
+    float mx = 0.0f;
+    for (int k0 = lane * 8; k0 < K; k0 += 512) mx = absmax_exact(src[k0 / 8], mx);
+    mx = wave_max(mx);
+    const __half sh = scale_from_absmax(mx, clip);
+    const float rscale = 1.0f / __half2float(sh);
+    uint32_t *dst = reinterpret_cast<uint32_t *>(qact + row * (Kp / 2));
+    for (int k0 = lane * 8; k0 < Kp; k0 += 512) {
+        u32x4 v = k0 < K ? src[k0 / 8] : u32x4{0u, 0u, 0u, 0u};
+        dst[k0 / 8] = quantize_word_exact(v, rscale);
+    }
+    if (lane == 0) scale_h[row] = sh;
+}
+
+// Per-row scale only (weights: quantize_weight_per_channel's first launch).
+__global__ __launch_bounds__(kRowsPerBlock * kWaveSize) void row_scale_kernel(const __half *__restrict__ x, int64_t rows, int K,
+                                                                              float clip, __half *__restrict__ scale_h) {
+    const int lane = threadIdx.x & (kWaveSize - 1);
+    const int64_t row = static_cast<int64_t>(blockIdx.x) * kRowsPerBlock + (threadIdx.x >> 6);
+    if (row >= rows) return;
+    const u32x4 *src = reinterpret_cast<const u32x4 *>(x + row * static_cast<int64_t>(K));
+    float mx = 0.0f;
+    for (int k0 = lane * 8; k0 < K; k0 += 512) mx = absmax_exact(src[k0 / 8], mx);
+    mx = wave_max(mx);
+    if (lane == 0) scale_h[row] = scale_from_absmax(mx, clip);
+}
+
+// Quantize rows with caller-provided fp16 scales into the native layout
+// (weights: quantize_warp_static_scale, vdm_w4a4_kernel.cu:296-338).
+__global__ __launch_bounds__(256) void quantize_given_scale_kernel(const __half *__restrict__ x, const __half *__restrict__ scale_h,
+                                                                   int64_t rows, int K, int Kp, uint8_t *__restrict__ q) {
+    const int64_t words_per_row = Kp / 8;
+    const int64_t idx = static_cast<int64_t>(blockIdx.x) * blockDim.x + threadIdx.x;
+    if (idx >= rows * words_per_row) return;
+    const int64_t row = idx / words_per_row;
+    const int k0 = static_cast<int>(idx % words_per_row) * 8;
+    u32x4 v = k0 < K ? *reinterpret_cast<const u32x4 *>(x + row * K + k0) : u32x4{0u, 0u, 0u, 0u};
+    const float rscale = 1.0f / __half2float(scale_h[row]);
+    reinterpret_cast<uint32_t *>(q)[idx] = quantize_word_exact(v, rscale);
+}
+
+template <int NCH>
+int launch_reg(const __half *x, int64_t M, int64_t K, int64_t ldx, float clip, uint8_t *qact, __half *scale_h, hipStream_t s) {
+    const unsigned grid = static_cast<unsigned>(ceil_div(M, kRowsPerBlock));
+    hipLaunchKernelGGL(quantize_rows_kernel<NCH>, dim3(grid), dim3(kRowsPerBlock * kWaveSize), 0, s, x, ldx, static_cast<int>(M),
+                       static_cast<int>(K), static_cast<int>(k_padded(K)), clip, qact, scale_h);
+    return check_launch("quantize_rows_kernel");
+}
+
+}  // namespace
+
+int launch_quantize_act(const __half *x, int64_t M, int64_t K, int64_t ldx, float clip, uint8_t *qact, __half *scale_h,
+                        hipStream_t s) {
+    if (M == 0) return VDMQ_OK;
+    const int64_t nch = ceil_div(k_padded(K), 512);
+#define VDMQ_CASE(n) \
+    if (nch <= n) return launch_reg<n>(x, M, K, ldx, clip, qact, scale_h, s)
+    VDMQ_CASE(1);
+    VDMQ_CASE(2);
+    VDMQ_CASE(3);
+    VDMQ_CASE(4);
+    VDMQ_CASE(6);
+    VDMQ_CASE(8);
+    VDMQ_CASE(10);
+    VDMQ_CASE(12);
+    VDMQ_CASE(14);
+    VDMQ_CASE(16);
+    VDMQ_CASE(18);
+    VDMQ_CASE(20);
+    VDMQ_CASE(24);
+    VDMQ_CASE(28);
+    VDMQ_CASE(32);
+#undef VDMQ_CASE
+    const unsigned grid = static_cast<unsigned>(ceil_div(M, kRowsPerBlock));
+    hipLaunchKernelGGL(quantize_rows_anyk_kernel, dim3(grid), dim3(kRowsPerBlock * kWaveSize), 0, s, x, ldx, static_cast<int>(M),
+                       static_cast<int>(K), static_cast<int>(k_padded(K)), clip, qact, scale_h);
+    return check_launch("quantize_rows_anyk_kernel");
+}
+
+int launch_row_scale(const __half *x, int64_t rows, int64_t K, float clip, __half *scale_h, hipStream_t s) {
+    if (rows == 0) return VDMQ_OK;
+    hipLaunchKernelGGL(row_scale_kernel, dim3(static_cast<unsigned>(ceil_div(rows, kRowsPerBlock))),
+                       dim3(kRowsPerBlock * kWaveSize), 0, s, x, rows, static_cast<int>(K), clip, scale_h);
+    return check_launch("row_scale_kernel");
+}
+
+int launch_quantize_given_scale(const __half *x, const __half *scale_h, int64_t rows, int64_t K, uint8_t *q, hipStream_t s) {
+    if (rows == 0) return VDMQ_OK;
+    const int64_t total = rows * (k_padded(K) / 8);
+    hipLaunchKernelGGL(quantize_given_scale_kernel, dim3(static_cast<unsigned>(ceil_div(total, 256))), dim3(256), 0, s, x, scale_h,
+                       rows, static_cast<int>(K), static_cast<int>(k_padded(K)), q);
+    return check_launch("quantize_given_scale_kernel");
+}
+
+}  // namespace vdmq

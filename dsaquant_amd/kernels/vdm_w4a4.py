@@ -1,0 +1,362 @@
+"""W4A4 kernel wrapper for MI355X, function-for-function with the reference's
+``vdm_infer/kernels/vdm_w4a4.py`` (same names, arguments, shapes, dtypes and
+error types), backed by ``libvdmq.so`` through ctypes instead of a JIT-built
+CUDA extension.
+
+What differs underneath (not visible through this API):
+
+* activations are quantized in ONE pass (absmax + quantize) into a row-major
+  int4 buffer with one fp16 scale per token -- the v1 fragment-ordered ``qact``
+  and the K/64-times replicated ``ascales`` only exist when a caller asks for
+  them through ``quantize_activation_per_token``;
+* the checkpoint's v1 weight buffers are relaid once per (qweight, wscales)
+  pair into the row-major form the gfx950 GEMM consumes, and cached for the
+  lifetime of the v1 tensor (the reference caches its concatenated QKV buffers
+  the same way, attention.py:44-54).
+
+There is no CPU/PyTorch fallback: without the built library or a GPU every
+kernel function raises.
+"""
+from __future__ import annotations
+
+import weakref
+from typing import Dict, Optional, Tuple
+
+import torch
+
+from .. import _lib
+
+BLOCK_M = 256  # vdm_w4a4.py:23-25 of the reference
+BLOCK_N = 128
+WARP_K = 64
+
+_LOAD_ERROR: Optional[BaseException] = None
+
+
+def build_config() -> dict:
+    """Counterpart of vdm_w4a4.py:115-127: where the native code comes from."""
+    return {
+        "library": str(_lib.LIB_PATH),
+        "arch_list": "gfx950",
+        "arch_tag": "gfx950",
+        "build_dir": str(_lib.CSRC / "_build"),
+        "extension_name": "libvdmq",
+        "torch_hip": torch.version.hip,
+    }
+
+
+def _load_ext():
+    global _LOAD_ERROR
+    try:
+        lib = _lib.load()
+        if not torch.cuda.is_available():
+            raise RuntimeError("no HIP device is visible to torch")
+        _LOAD_ERROR = None
+        return lib
+    except BaseException as exc:  # kept for load_error(), like vdm_w4a4.py:165-167
+        _LOAD_ERROR = exc
+        raise
+
+
+def is_available() -> bool:
+    """Never raises (vdm_w4a4.py:170-175)."""
+    try:
+        _load_ext()
+        return True
+    except BaseException:
+        return False
+
+
+def load_error() -> Optional[BaseException]:
+    return _LOAD_ERROR
+
+
+# ----------------------------------------------------------------- helpers
+
+def _stream(device: torch.device) -> int:
+    return torch.cuda.current_stream(device).cuda_stream
+
+
+def _require(cond: bool, msg: str) -> None:
+    # the reference's TORCH_CHECK failures surface as RuntimeError
+    if not cond:
+        raise _lib.VdmqError(msg)
+
+
+def _check_device_tensor(t: torch.Tensor, name: str, dtype: torch.dtype) -> None:
+    _require(t.is_cuda, f"{name} must be a CUDA tensor")  # vdm_w4a4_kernel.cu:688-691
+    _require(t.is_contiguous(), f"{name} must be contiguous")
+    _require(t.dtype == dtype, f"{name} must be {str(dtype).replace('torch.', '')}")
+
+
+def _as_2d_half_contiguous(x: torch.Tensor) -> Tuple[torch.Tensor, Tuple[int, ...]]:
+    orig_shape = tuple(x.shape[:-1])
+    return x.reshape(-1, x.shape[-1]).half().contiguous(), orig_shape
+
+
+def _check_linear_shapes(x_2d: torch.Tensor, qweight: torch.Tensor, wscales: torch.Tensor) -> None:
+    # same conditions, order and exception type as vdm_w4a4.py:198-206
+    if x_2d.shape[1] % WARP_K != 0:
+        raise ValueError(f"K={x_2d.shape[1]} must be a multiple of {WARP_K}")
+    if qweight.shape[0] % BLOCK_N != 0:
+        raise ValueError(f"N={qweight.shape[0]} must be a multiple of {BLOCK_N}")
+    if qweight.shape[1] != x_2d.shape[1] // 2:
+        raise ValueError("qweight shape must be [N, K/2]")
+    if wscales.shape != (qweight.shape[0], x_2d.shape[1] // WARP_K):
+        raise ValueError("wscales shape must be [N, K/64]")
+
+
+def k_padded(K: int) -> int:
+    return int(_lib.load().vdmq_k_padded(K))
+
+
+# one-time v1 -> native relayout, cached per v1 tensor pair
+_NATIVE_CACHE: Dict[tuple, Tuple[torch.Tensor, torch.Tensor]] = {}
+
+
+def _native_weights(qweight: torch.Tensor, wscales: torch.Tensor) -> Tuple[torch.Tensor, torch.Tensor]:
+    key = (qweight.data_ptr(), wscales.data_ptr(), tuple(qweight.shape), qweight.device.index, qweight._version, wscales._version)
+    hit = _NATIVE_CACHE.get(key)
+    if hit is not None:
+        return hit
+    lib = _load_ext()
+    _check_device_tensor(qweight, "qweight", torch.uint8)
+    _check_device_tensor(wscales, "wscales", torch.float16)
+    N, K = qweight.shape[0], qweight.shape[1] * 2
+    with torch.cuda.device(qweight.device):
+        native = torch.empty((N, k_padded(K) // 2), dtype=torch.uint8, device=qweight.device)
+        plain = torch.empty((N,), dtype=torch.float16, device=qweight.device)
+        s = _stream(qweight.device)
+        _lib.check(lib.vdmq_weight_v1_to_native(qweight.data_ptr(), native.data_ptr(), N, K, s))
+        _lib.check(lib.vdmq_wscale_v1_to_plain(wscales.data_ptr(), plain.data_ptr(), N, K, s))
+    _NATIVE_CACHE[key] = (native, plain)
+    weakref.finalize(qweight, _NATIVE_CACHE.pop, key, None)
+    return native, plain
+
+
+def clear_native_cache() -> None:
+    _NATIVE_CACHE.clear()
+
+
+# -------------------------------------------------------------- public API
+
+def pack_weight_with_scale(weight: torch.Tensor, channel_scale: torch.Tensor):
+    """Pack fp weights with caller-provided per-channel scales.
+
+    Returns ``(qweight u8 [N, K/2] v1, packed_scales fp16 [N, K/64] v1,
+    channel_scales fp16 [N])`` like vdm_w4a4.py:209-214 /
+    vdm_w4a4_kernel.cu:697-728.
+    """
+    lib = _load_ext()
+    weight_h = weight.detach().half().contiguous()
+    scale_h = channel_scale.detach().view(-1).half().contiguous().to(weight_h.device)
+    _check_device_tensor(weight_h, "weight", torch.float16)
+    _require(weight_h.dim() == 2, "weight must be [N, K]")
+    N, K = weight_h.shape
+    _require(scale_h.numel() == N, "channel_scales length must equal N")
+    _require(N % BLOCK_N == 0, f"N must be a multiple of {BLOCK_N}")
+    _require(K % WARP_K == 0, f"K must be a multiple of {WARP_K}")
+    dev = weight_h.device
+    with torch.cuda.device(dev):
+        s = _stream(dev)
+        native = torch.empty((N, k_padded(K) // 2), dtype=torch.uint8, device=dev)
+        qweight = torch.empty((N, K // 2), dtype=torch.uint8, device=dev)
+        packed_scales = torch.empty((N, K // WARP_K), dtype=torch.float16, device=dev)
+        _lib.check(lib.vdmq_quantize_weight_native(weight_h.data_ptr(), scale_h.data_ptr(), native.data_ptr(), N, K, s))
+        _lib.check(lib.vdmq_weight_native_to_v1(native.data_ptr(), qweight.data_ptr(), N, K, s))
+        _lib.check(lib.vdmq_wscale_plain_to_v1(scale_h.data_ptr(), packed_scales.data_ptr(), N, K, s))
+    # the native form is already at hand: seed the cache so the first GEMM needs no relayout
+    key = (qweight.data_ptr(), packed_scales.data_ptr(), tuple(qweight.shape), dev.index, qweight._version, packed_scales._version)
+    _NATIVE_CACHE[key] = (native, scale_h.clone())
+    weakref.finalize(qweight, _NATIVE_CACHE.pop, key, None)
+    return qweight, packed_scales, scale_h
+
+
+def quantize_weight_per_channel(weight: torch.Tensor):
+    """Derive per-channel scales (absmax/7, clip 1) and pack
+    (vdm_w4a4.py:217-219 / vdm_w4a4_kernel.cu:730-763)."""
+    lib = _load_ext()
+    weight_h = weight.detach().half().contiguous()
+    _check_device_tensor(weight_h, "weight", torch.float16)
+    _require(weight_h.dim() == 2, "weight must be [N, K]")
+    N, K = weight_h.shape
+    _require(N % BLOCK_N == 0, f"N must be a multiple of {BLOCK_N}")
+    _require(K % WARP_K == 0, f"K must be a multiple of {WARP_K}")
+    with torch.cuda.device(weight_h.device):
+        scales = torch.empty((N,), dtype=torch.float16, device=weight_h.device)
+        _lib.check(lib.vdmq_row_scale(weight_h.data_ptr(), N, K, 1.0, scales.data_ptr(), _stream(weight_h.device)))
+    return pack_weight_with_scale(weight_h, scales)
+
+
+def _linear_2d(x_2d: torch.Tensor, native_w: torch.Tensor, wscale: torch.Tensor, bias: Optional[torch.Tensor], clip_ratio: float,
+               out_dtype: torch.dtype = torch.float16) -> torch.Tensor:
+    lib = _load_ext()
+    M, K = x_2d.shape
+    N = native_w.shape[0]
+    dev = x_2d.device
+    _require(native_w.device == dev and wscale.device == dev, "weights and input must be on the same device")
+    if bias is not None:
+        _check_device_tensor(bias, "bias", torch.float16)
+        _require(bias.dim() == 1, "bias must be [N]")
+        _require(bias.numel() == N, "bias length must equal N")
+    with torch.cuda.device(dev):
+        out = torch.empty((M, N), dtype=out_dtype, device=dev)
+        if M == 0:
+            return out
+        ws_bytes = int(lib.vdmq_workspace_bytes(M, K))
+        workspace = torch.empty((ws_bytes,), dtype=torch.uint8, device=dev)
+        _lib.check(lib.vdmq_linear_w4a4(
+            x_2d.data_ptr(), M, K, x_2d.stride(0), float(clip_ratio), native_w.data_ptr(), wscale.data_ptr(),
+            None if bias is None else bias.data_ptr(), out.data_ptr(),
+            _lib.VDMQ_OUT_F16 if out_dtype == torch.float16 else _lib.VDMQ_OUT_BF16, N, out.stride(0), workspace.data_ptr(),
+            ws_bytes, _stream(dev)))
+    return out
+
+
+def linear_vdm_w4a4(
+    x: torch.Tensor,
+    qweight: torch.Tensor,
+    wscales: torch.Tensor,
+    bias: Optional[torch.Tensor] = None,
+    clip_ratio: float = 1.0,
+    bias_half: Optional[torch.Tensor] = None,
+) -> torch.Tensor:
+    """W4A4 linear: dynamic per-token A4 quantization of ``x``, int4 x int4 GEMM
+    against the packed weights, per-token x per-channel scale and fp16 bias.
+    Signature and semantics of vdm_w4a4.py:222-244; the output is always fp16."""
+    _load_ext()
+    x_2d, orig_shape = _as_2d_half_contiguous(x)
+    _check_linear_shapes(x_2d, qweight, wscales)
+    _require(x_2d.is_cuda, "input must be a CUDA tensor")
+    native_w, wscale = _native_weights(qweight.contiguous(), wscales.contiguous())
+    b = bias_half if bias_half is not None else bias
+    if b is not None:
+        b = b.half().contiguous().view(-1)
+    out = _linear_2d(x_2d, native_w, wscale, b, clip_ratio)
+    return out.view(*orig_shape, -1)
+
+
+def quantize_activation_per_token(x: torch.Tensor, clip_ratio: float = 1.0):
+    """Returns ``(qact u8 [ceil(M,256), K/2], ascales fp16 [ceil(M,256), K/64],
+    act_scales fp16 [M])`` in the reference's v1 layouts
+    (vdm_w4a4.py:247-250 / vdm_w4a4_kernel.cu:840-874)."""
+    lib = _load_ext()
+    x_2d, _ = _as_2d_half_contiguous(x)
+    _check_device_tensor(x_2d, "input", torch.float16)
+    M, K = x_2d.shape
+    _require(K % WARP_K == 0, f"K must be a multiple of {WARP_K}")
+    PM = (M + BLOCK_M - 1) // BLOCK_M * BLOCK_M
+    dev = x_2d.device
+    with torch.cuda.device(dev):
+        s = _stream(dev)
+        native = torch.empty((M, k_padded(K) // 2), dtype=torch.uint8, device=dev)
+        act_scales = torch.empty((M,), dtype=torch.float16, device=dev)
+        qact = torch.empty((PM, K // 2), dtype=torch.uint8, device=dev)
+        ascales = torch.empty((PM, K // WARP_K), dtype=torch.float16, device=dev)
+        _lib.check(lib.vdmq_quantize_act(x_2d.data_ptr(), M, K, x_2d.stride(0), float(clip_ratio), native.data_ptr(),
+                                         act_scales.data_ptr(), s))
+        _lib.check(lib.vdmq_act_native_to_v1(native.data_ptr(), act_scales.data_ptr(), M, K, qact.data_ptr(), ascales.data_ptr(), s))
+    return qact, ascales, act_scales
+
+
+def quantize_activation_native(x: torch.Tensor, clip_ratio: float = 1.0):
+    """The quantizer's own output: ``(qact u8 [M, Kp/2] row-major, scales fp16 [M])``."""
+    lib = _load_ext()
+    x_2d, _ = _as_2d_half_contiguous(x)
+    _check_device_tensor(x_2d, "input", torch.float16)
+    M, K = x_2d.shape
+    _require(K % WARP_K == 0, f"K must be a multiple of {WARP_K}")
+    dev = x_2d.device
+    with torch.cuda.device(dev):
+        native = torch.empty((M, k_padded(K) // 2), dtype=torch.uint8, device=dev)
+        act_scales = torch.empty((M,), dtype=torch.float16, device=dev)
+        _lib.check(lib.vdmq_quantize_act(x_2d.data_ptr(), M, K, x_2d.stride(0), float(clip_ratio), native.data_ptr(),
+                                         act_scales.data_ptr(), _stream(dev)))
+    return native, act_scales
+
+
+def linear_prequantized(qact: torch.Tensor, ascales: torch.Tensor, qweight: torch.Tensor, wscales: torch.Tensor) -> torch.Tensor:
+    """GEMM only, on v1-layout activations already padded to BLOCK_M rows; no
+    bias (vdm_w4a4.py:253-256 / vdm_w4a4_kernel.cu:876-918)."""
+    lib = _load_ext()
+    qact, ascales = qact.contiguous(), ascales.contiguous()
+    qweight, wscales = qweight.contiguous(), wscales.contiguous()
+    _check_device_tensor(qact, "qact", torch.uint8)
+    _check_device_tensor(ascales, "ascales", torch.float16)
+    _check_device_tensor(qweight, "qweight", torch.uint8)
+    _check_device_tensor(wscales, "wscales", torch.float16)
+    _require(qact.dim() == 2 and ascales.dim() == 2 and qweight.dim() == 2 and wscales.dim() == 2, "all inputs must be 2-D")
+    M, K, N = qact.shape[0], qact.shape[1] * 2, qweight.shape[0]
+    _require(qweight.shape[1] == K // 2, "qweight second dim must be K / 2")
+    _require(K % WARP_K == 0, f"K must be a multiple of {WARP_K}")
+    _require(tuple(ascales.shape) == (M, K // WARP_K), "bad ascales shape")
+    _require(tuple(wscales.shape) == (N, K // WARP_K), "bad wscales shape")
+    _require(M % BLOCK_M == 0, f"M must be a multiple of {BLOCK_M}")
+    _require(N % BLOCK_N == 0, f"N must be a multiple of {BLOCK_N}")
+    native_w, wscale = _native_weights(qweight, wscales)
+    dev = qact.device
+    with torch.cuda.device(dev):
+        s = _stream(dev)
+        out = torch.empty((M, N), dtype=torch.float16, device=dev)
+        if M == 0:
+            return out
+        native = torch.empty((M, k_padded(K) // 2), dtype=torch.uint8, device=dev)
+        scales = torch.empty((M,), dtype=torch.float16, device=dev)
+        _lib.check(lib.vdmq_act_v1_to_native(qact.data_ptr(), ascales.data_ptr(), M, K, native.data_ptr(), scales.data_ptr(), s))
+        _lib.check(lib.vdmq_gemm_w4a4(native.data_ptr(), scales.data_ptr(), native_w.data_ptr(), wscale.data_ptr(), None,
+                                      out.data_ptr(), _lib.VDMQ_OUT_F16, M, N, K, out.stride(0), s))
+    return out
+
+
+def gemm_int32_accumulators(qact_native: torch.Tensor, wq_native: torch.Tensor, K: int) -> torch.Tensor:
+    """Checker's view: the exact int32 accumulators of the GEMM, [M, N]."""
+    lib = _load_ext()
+    M, N = qact_native.shape[0], wq_native.shape[0]
+    dev = qact_native.device
+    with torch.cuda.device(dev):
+        acc = torch.empty((M, N), dtype=torch.int32, device=dev)
+        if M:
+            _lib.check(lib.vdmq_gemm_w4a4_acc(qact_native.data_ptr(), wq_native.data_ptr(), acc.data_ptr(), M, N, K, _stream(dev)))
+    return acc
+
+
+def linear_vdm_w4a4_qkv(
+    x: torch.Tensor,
+    q_weight_packed: torch.Tensor,
+    q_weight_scale: torch.Tensor,
+    k_weight_packed: torch.Tensor,
+    k_weight_scale: torch.Tensor,
+    v_weight_packed: torch.Tensor,
+    v_weight_scale: torch.Tensor,
+    q_bias: Optional[torch.Tensor] = None,
+    k_bias: Optional[torch.Tensor] = None,
+    v_bias: Optional[torch.Tensor] = None,
+    clip_ratio: float = 1.0,
+    w_qkv_packed: Optional[torch.Tensor] = None,
+    w_qkv_scale: Optional[torch.Tensor] = None,
+    qkv_bias_half: Optional[torch.Tensor] = None,
+):
+    """Fused QKV: one activation quantization and one GEMM against the
+    row-concatenated Wq|Wk|Wv; returns three views of one [..., 3N] tensor
+    (vdm_w4a4.py:259-298).  A row-concatenation of v1 buffers is itself a valid
+    v1 buffer because every 128-row block is self-contained."""
+    if w_qkv_packed is None or w_qkv_scale is None:
+        w_qkv_packed = torch.cat([q_weight_packed, k_weight_packed, v_weight_packed], dim=0).contiguous()
+        w_qkv_scale = torch.cat([q_weight_scale, k_weight_scale, v_weight_scale], dim=0).contiguous()
+    if qkv_bias_half is None:
+        n = q_weight_packed.shape[0]
+        has_bias = q_bias is not None or k_bias is not None or v_bias is not None
+        if has_bias:
+            device = w_qkv_packed.device
+
+            def zeros():
+                return torch.zeros(n, dtype=torch.float16, device=device)
+
+            qkv_bias_half = torch.cat([
+                q_bias.half().contiguous() if q_bias is not None else zeros(),
+                k_bias.half().contiguous() if k_bias is not None else zeros(),
+                v_bias.half().contiguous() if v_bias is not None else zeros(),
+            ], dim=0)
+    qkv = linear_vdm_w4a4(x, w_qkv_packed, w_qkv_scale, bias=None, clip_ratio=clip_ratio, bias_half=qkv_bias_half)
+    n = q_weight_packed.shape[0]
+    return qkv.split(n, dim=-1)

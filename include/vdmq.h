@@ -1,0 +1,134 @@
+/*
+ * vdmq -- C ABI of the MI355X (gfx950) W4A4 linear hot path.
+ *
+ * Every entry point takes plain device pointers, sizes and a HIP stream, and
+ * returns 0 on success or a negative VDMQ_E* code; vdmq_last_error() then
+ * holds a message (thread-local).  No entry point allocates, frees or
+ * synchronises: all buffers are caller-owned device memory, all work is
+ * enqueued asynchronously on `stream` (0 = the null stream) of the current
+ * device.
+ *
+ * The functions replace the six pybind entry points of the reference
+ * extension (vdm_infer/kernels/csrc/vdm_w4a4_kernel.cu:924-940) and the kernel
+ * launches behind them; the citation on each declaration names the part it
+ * stands in for.
+ *
+ * Layouts
+ *   "v1"      the byte order the reference's CUDA packers emit and packed
+ *             checkpoints (format "vdm_w4a4_packed_v1") store:
+ *             qweight u8 [N, K/2], packed scales fp16 [N, K/64],
+ *             qact u8 [ceil(M,256), K/2], ascales fp16 [ceil(M,256), K/64].
+ *   "native"  what the gfx950 kernels consume: row-major packed int4,
+ *             u8 [rows, Kp/2] with Kp = vdmq_k_padded(K); byte j of a row holds
+ *             element 2j in its low nibble and 2j+1 in its high nibble (two's
+ *             complement); elements K..Kp-1 are zero.  Scales are one fp16 per
+ *             row ([M] for tokens, [N] for output channels).
+ */
+#ifndef VDMQ_H
+#define VDMQ_H
+
+#include <stdint.h>
+
+#ifdef __cplusplus
+extern "C" {
+#endif
+
+#define VDMQ_OK 0
+#define VDMQ_EINVAL (-1)  /* null pointer, misaligned pointer, bad enum */
+#define VDMQ_ESHAPE (-2)  /* a shape precondition failed (K % 64, N % 128, ...) */
+#define VDMQ_ELAUNCH (-3) /* the HIP runtime refused a launch */
+#define VDMQ_ENOSPACE (-4) /* caller workspace too small */
+
+#define VDMQ_OUT_F16 0
+#define VDMQ_OUT_BF16 1
+
+/* Shape constants of the v1 layout (vdm_w4a4_kernel.cu:15-24, vdm_w4a4.py:23-25). */
+#define VDMQ_BLOCK_M 256
+#define VDMQ_BLOCK_N 128
+#define VDMQ_WARP_K 64
+
+typedef void *vdmq_stream_t; /* hipStream_t */
+
+int vdmq_version(void);
+const char *vdmq_arch(void);       /* "gfx950" */
+const char *vdmq_last_error(void); /* message of the last failure on this thread */
+
+/* Native row length in elements for a logical K (K rounded up to the GEMM's
+ * K step).  Native rows are vdmq_k_padded(K)/2 bytes. */
+int64_t vdmq_k_padded(int64_t K);
+
+/* Dynamic per-token A4 quantizer.  Replaces token_scale_kernel +
+ * act_quantize_per_token_kernel (vdm_w4a4_kernel.cu:459-516, launched at
+ * :802-816 and :858-872) with one pass over x.
+ *   x       fp16 [M, K], row stride ldx elements (ldx % 8 == 0, 16-byte aligned)
+ *   qact    u8 [M, Kp/2] native, 16-byte aligned
+ *   scale_h fp16 [M]: fp16_rn(absmax > 0 ? (absmax / 7) * clip : 1)
+ * Preconditions: K % 64 == 0, M >= 0. */
+int vdmq_quantize_act(const void *x, int64_t M, int64_t K, int64_t ldx, float clip, void *qact, void *scale_h,
+                      vdmq_stream_t stream);
+
+/* W4A4 GEMM with fused epilogue.  Replaces linear_w4a4_kernel
+ * (vdm_w4a4_kernel.cu:627-686, launched at :819 and :907):
+ *   acc[m,n] = sum_k qact[m,k] * wq[n,k]                      (int32, exact)
+ *   out[m,n] = fp16_rn(float(acc) * (float(ascale[m]) * float(wscale[n])))
+ *              then, with a bias, one more fp16 addition of bias[n]
+ *   qact u8 [M, Kp/2] native; ascale fp16 [M]; wq u8 [N, Kp/2] native;
+ *   wscale fp16 [N]; bias fp16 [N] or NULL; out [M, N] with row stride ldo
+ *   elements (ldo % 8 == 0), out_dtype VDMQ_OUT_F16 or VDMQ_OUT_BF16.
+ * Preconditions: K % 64 == 0, N % 128 == 0, K <= 65536. */
+int vdmq_gemm_w4a4(const void *qact, const void *ascale, const void *wq, const void *wscale, const void *bias, void *out,
+                   int out_dtype, int64_t M, int64_t N, int64_t K, int64_t ldo, vdmq_stream_t stream);
+
+/* Same GEMM, but writes the raw int32 accumulators acc [M, N] (row stride N)
+ * instead of the scaled output: the checker's view of the value the reference
+ * holds in `ipsum` before finalize_int_accum (vdm_w4a4_kernel.cu:650, :684). */
+int vdmq_gemm_w4a4_acc(const void *qact, const void *wq, int32_t *acc, int64_t M, int64_t N, int64_t K, vdmq_stream_t stream);
+
+/* Bytes of caller workspace vdmq_linear_w4a4 needs for an [M, K] input. */
+int64_t vdmq_workspace_bytes(int64_t M, int64_t K);
+
+/* Quantize + GEMM: linear_dynamic / linear_dynamic_bias
+ * (vdm_w4a4_kernel.cu:765-838).  `workspace` holds the native qact and the
+ * token scales; it replaces the reference's per-call torch::empty scratch
+ * (:796-798). */
+int vdmq_linear_w4a4(const void *x, int64_t M, int64_t K, int64_t ldx, float clip, const void *wq, const void *wscale,
+                     const void *bias, void *out, int out_dtype, int64_t N, int64_t ldo, void *workspace,
+                     int64_t workspace_bytes, vdmq_stream_t stream);
+
+/* One-time relayouts between the checkpoint's v1 buffers and native ones.
+ * v1 weight layout: weight_quantize_per_channel_kernel + pack_wscales
+ * (vdm_w4a4_kernel.cu:518-551, :286-294).  N % 128 == 0, K % 64 == 0. */
+int vdmq_weight_v1_to_native(const void *qweight_v1, void *wq_native, int64_t N, int64_t K, vdmq_stream_t stream);
+int vdmq_weight_native_to_v1(const void *wq_native, void *qweight_v1, int64_t N, int64_t K, vdmq_stream_t stream);
+/* packed scales fp16 [N, K/64] -> plain fp16 [N] (k-group 0, as the reference
+ * GEMM reads them, :661-663) and back (repeated per k-group, :548-550). */
+int vdmq_wscale_v1_to_plain(const void *packed_v1, void *plain, int64_t N, int64_t K, vdmq_stream_t stream);
+int vdmq_wscale_plain_to_v1(const void *plain, void *packed_v1, int64_t N, int64_t K, vdmq_stream_t stream);
+
+/* Activation buffers in the v1 layout, for the split entry points
+ * quantize_activation_per_token / linear_prequantized
+ * (vdm_w4a4_kernel.cu:840-918).  PM = ceil(M, 256); rows M..PM-1 of the v1
+ * buffers are zero with scale 1 (:357-378).
+ *   native_to_v1: qact u8 [M, Kp/2], scale fp16 [M] -> qact_v1 u8 [PM, K/2],
+ *                 ascales_v1 fp16 [PM, K/64]
+ *   v1_to_native: the inverse, for all PM rows (M % 256 == 0 required, :896). */
+int vdmq_act_native_to_v1(const void *qact, const void *scale_h, int64_t M, int64_t K, void *qact_v1, void *ascales_v1,
+                          vdmq_stream_t stream);
+int vdmq_act_v1_to_native(const void *qact_v1, const void *ascales_v1, int64_t M, int64_t K, void *qact, void *scale_h,
+                          vdmq_stream_t stream);
+
+/* Per-row scale of an fp16 matrix with clip 1: the token_scale_kernel launch
+ * of quantize_weight_per_channel (vdm_w4a4_kernel.cu:747-751). */
+int vdmq_row_scale(const void *w, int64_t rows, int64_t K, float clip, void *scale_h, vdmq_stream_t stream);
+
+/* Quantize fp16 weights [N, K] (contiguous) with caller-provided per-channel
+ * fp16 scales into a native buffer: q = sat_s4(rni(float(w) * (1 / float(s))))
+ * -- the arithmetic of pack_weight_with_scale / quantize_warp_static_scale
+ * (vdm_w4a4_kernel.cu:697-728, :296-338).  The v1 buffers that function
+ * returns are then vdmq_weight_native_to_v1 + vdmq_wscale_plain_to_v1. */
+int vdmq_quantize_weight_native(const void *w, const void *scale_h, void *wq_native, int64_t N, int64_t K, vdmq_stream_t stream);
+
+#ifdef __cplusplus
+}
+#endif
+#endif /* VDMQ_H */

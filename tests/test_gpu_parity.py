@@ -1,0 +1,336 @@
+"""GPU parity: the HIP path (through the C ABI / the Python boundary) against
+the CPU oracle on identical seeded inputs.
+
+Bars: packed int4 activations, fp16 token scales and int32 accumulators are
+bit-exact; the fp16 output is compared bit-for-bit as well (every operation of
+the epilogue is a correctly rounded IEEE operation on both sides), with the
+stated tolerance max|err| <= 1e-3 * max|Y| as the contractual bound.
+"""
+import numpy as np
+import pytest
+import torch
+
+import oracle as O
+
+pytestmark = pytest.mark.gpu
+
+DEV = "cuda:0"
+
+
+def vk():
+    from dsaquant_amd.kernels import vdm_w4a4
+
+    assert vdm_w4a4.is_available(), vdm_w4a4.load_error()
+    return vdm_w4a4
+
+
+def t16(a):
+    return torch.from_numpy(np.ascontiguousarray(a)).to(DEV)
+
+
+def unpack_native(buf: np.ndarray, K: int) -> np.ndarray:
+    """row-major packed int4 [R, Kp/2] -> int8 [R, K]; also checks the zero padding."""
+    lo = (buf & 0xF).astype(np.int8)
+    hi = (buf >> 4).astype(np.int8)
+    q = np.empty((buf.shape[0], buf.shape[1] * 2), np.int8)
+    q[:, 0::2], q[:, 1::2] = lo, hi
+    q = np.where(q >= 8, q - 16, q).astype(np.int8)
+    assert not q[:, K:].any(), "padding nibbles must be zero"
+    return q[:, :K]
+
+
+def pack_native(q: np.ndarray, Kp: int) -> np.ndarray:
+    R, K = q.shape
+    full = np.zeros((R, Kp), np.uint8)
+    full[:, :K] = q.astype(np.uint8) & 0xF
+    return (full[:, 0::2] | (full[:, 1::2] << 4)).astype(np.uint8)
+
+
+def special_rows(x: np.ndarray) -> np.ndarray:
+    x = x.copy()
+    M = x.shape[0]
+    if M > 12:
+        x[1] = 0
+        x[2, 5] = np.float16(np.nan)
+        x[3, 7] = np.float16(np.inf)
+        x[4, 9] = np.float16(-np.inf)
+        x[5] = np.float16(6e-8)  # fp16 scale underflows to zero
+        x[6] = np.float16(65504.0)
+        x[7, ::2] = np.float16(-65504.0)
+        x[8] = np.float16(1e-4)
+        x[9, 0] = np.float16(np.nan)
+        x[9, 1] = np.float16(np.inf)
+        x[10] = np.float16(np.nan)
+    return x
+
+
+# ------------------------------------------------------------ quantizer
+
+QUANT_SHAPES = [(257, 1536), (4096, 1536), (515, 5120), (300, 8960), (130, 13824), (100, 64), (77, 192), (33, 3072), (64, 14336),
+                (19, 16384 + 64), (5, 2048)]
+
+
+@pytest.mark.parametrize("M,K", QUANT_SHAPES)
+@pytest.mark.parametrize("clip", [1.0, 0.95])
+def test_quantizer_bit_exact(M, K, clip):
+    v = vk()
+    x, _, _, _ = O.synth_linear(M, K, 128, seed=M + K)
+    x = special_rows(x)
+    print(f"quantizer M={M} K={K} clip={clip}", flush=True)
+    qn, sc = v.quantize_activation_native(t16(x), clip)
+    torch.cuda.synchronize()
+    want_s = O.np_row_scale(x, clip)
+    got_s = sc.cpu().numpy()
+    assert np.array_equal(got_s.view(np.uint16), want_s.view(np.uint16))
+    want_q = O.np_quantize_rows(x, want_s)
+    got_q = unpack_native(qn.cpu().numpy(), K)
+    assert np.array_equal(got_q, want_q)
+
+
+def test_quantizer_against_scalar_c_oracle():
+    v = vk()
+    x = special_rows(O.synth_linear(64, 320, 128, seed=3)[0])
+    for clip in (1.0, 0.95, 0.3, 2.0):
+        qn, sc = v.quantize_activation_native(t16(x), clip)
+        s = O.c_row_scale(x, clip)
+        assert np.array_equal(sc.cpu().numpy().view(np.uint16), s.view(np.uint16))
+        assert np.array_equal(unpack_native(qn.cpu().numpy(), 320), O.c_quantize_rows(x, s))
+
+
+def test_quantizer_empty_and_strided():
+    v = vk()
+    qn, sc = v.quantize_activation_native(torch.empty((0, 128), dtype=torch.float16, device=DEV))
+    assert qn.shape == (0, 64) and sc.shape == (0,)
+    # leading dims are flattened, bf16/fp32 inputs are cast to fp16 first (vdm_w4a4.py:182-184)
+    x = torch.randn(3, 5, 256, device=DEV)
+    qn, sc = v.quantize_activation_native(x)
+    xh = x.half().reshape(-1, 256).cpu().numpy()
+    s = O.np_row_scale(xh, 1.0)
+    assert np.array_equal(sc.cpu().numpy().view(np.uint16), s.view(np.uint16))
+    assert np.array_equal(unpack_native(qn.cpu().numpy(), 256), O.np_quantize_rows(xh, s))
+
+
+# ------------------------------------------------------------------ GEMM
+
+GEMM_SHAPES = [(257, 1536, 1536), (1, 128, 64), (31, 256, 192), (512, 3072, 1536), (300, 128, 8960), (1000, 1536, 5120), (256, 10240, 5120),
+               (700, 384, 13824)]
+
+
+@pytest.mark.parametrize("M,N,K", GEMM_SHAPES)
+def test_gemm_int32_accumulators_exact(M, N, K):
+    v = vk()
+    rng = np.random.default_rng(M * 7 + N + K)
+    qx = rng.integers(-8, 8, (M, K), dtype=np.int8)
+    qw = rng.integers(-8, 8, (N, K), dtype=np.int8)
+    Kp = v.k_padded(K)
+    print(f"gemm acc M={M} N={N} K={K}", flush=True)
+    acc = v.gemm_int32_accumulators(t16(pack_native(qx, Kp)), t16(pack_native(qw, Kp)), K)
+    torch.cuda.synchronize()
+    assert np.array_equal(acc.cpu().numpy(), O.np_gemm_i32(qx, qw))
+
+
+def test_gemm_extreme_values_do_not_overflow():
+    v = vk()
+    K = 14336
+    qx = np.full((64, K), -8, np.int8)
+    qw = np.full((128, K), -8, np.int8)
+    qw[1] = 7
+    acc = v.gemm_int32_accumulators(t16(pack_native(qx, K)), t16(pack_native(qw, K)), K).cpu().numpy()
+    assert (acc[:, 0] == 64 * K).all() and (acc[:, 1] == -56 * K).all()
+
+
+# ----------------------------------------------------- whole linear path
+
+LINEAR_CASES = [
+    # (M, K, N, clip, bias)  -- the reference's smoke shape, config 0, skinny/ragged cases
+    (257, 1536, 1536, 0.95, True),
+    (4096, 1536, 4608, 1.0, True),
+    (512, 1536, 3072, 1.0, True),
+    (512, 5120, 10240, 1.0, False),
+    (1237, 8960, 1536, 0.95, True),
+    (300, 13824, 5120, 1.0, True),
+    (3, 64, 128, 1.0, True),
+]
+
+
+@pytest.mark.parametrize("M,K,N,clip,use_bias", LINEAR_CASES)
+def test_linear_matches_oracle(M, K, N, clip, use_bias):
+    v = vk()
+    x, qw, ws, bias = O.synth_linear(M, K, N, seed=0)
+    qweight_v1 = O.np_pack_wgt_v1(qw)
+    wscales_v1 = O.np_pack_wscales_v1(ws, K)
+    print(f"linear M={M} K={K} N={N} clip={clip} bias={use_bias}", flush=True)
+    y = v.linear_vdm_w4a4(t16(x), t16(qweight_v1), t16(wscales_v1), t16(bias) if use_bias else None, clip_ratio=clip)
+    torch.cuda.synchronize()
+    assert y.dtype == torch.float16 and tuple(y.shape) == (M, N)
+    want, _, _, _ = O.np_linear(x, qw, ws, bias if use_bias else None, clip)
+    got = y.cpu().numpy()
+    err = np.abs(got.astype(np.float32) - want.astype(np.float32)).max()
+    assert err <= 1e-3 * np.abs(want.astype(np.float32)).max()  # the contractual tolerance
+    assert np.array_equal(got.view(np.uint16), want.view(np.uint16))  # and in fact bit-exact
+
+
+def test_linear_leading_dims_bias_half_precedence_and_dtype():
+    v = vk()
+    x, qw, ws, bias = O.synth_linear(2 * 130, 256, 128, seed=5)
+    qv1, sv1 = t16(O.np_pack_wgt_v1(qw)), t16(O.np_pack_wscales_v1(ws, 256))
+    other = (bias.astype(np.float32) * 3).astype(np.float16)
+    y = v.linear_vdm_w4a4(t16(x).reshape(2, 130, 256).to(torch.bfloat16), qv1, sv1, t16(other).float(), 1.0, bias_half=t16(bias))
+    assert y.shape == (2, 130, 128) and y.dtype == torch.float16
+    xh = torch.from_numpy(x).to(torch.bfloat16).half().numpy()  # the cast chain the wrapper applies
+    want, _, _, _ = O.np_linear(xh, qw, ws, bias, 1.0)  # bias_half wins over bias
+    assert np.array_equal(y.reshape(-1, 128).cpu().numpy().view(np.uint16), want.view(np.uint16))
+
+
+def test_bf16_output_within_tolerance():
+    from dsaquant_amd import _lib
+
+    v = vk()
+    M, K, N = 300, 512, 256
+    x, qw, ws, bias = O.synth_linear(M, K, N, seed=6)
+    native_w, wscale = v._native_weights(t16(O.np_pack_wgt_v1(qw)), t16(O.np_pack_wscales_v1(ws, K)))
+    y = v._linear_2d(t16(x), native_w, wscale, t16(bias), 1.0, out_dtype=torch.bfloat16)
+    want, _, as_h, acc = O.np_linear(x, qw, ws, bias, 1.0)
+    exact = acc.astype(np.float64) * as_h.astype(np.float64)[:, None] * ws.astype(np.float64)[None, :] + bias.astype(np.float64)
+    err = np.abs(y.float().cpu().numpy().astype(np.float64) - exact)
+    assert err.max() <= 2.0 ** -8 * np.abs(exact).max()
+
+
+def test_shape_and_dtype_errors():
+    v = vk()
+    x = torch.zeros((4, 128), dtype=torch.float16, device=DEV)
+    qw = torch.zeros((128, 64), dtype=torch.uint8, device=DEV)
+    ws = torch.zeros((128, 2), dtype=torch.float16, device=DEV)
+    with pytest.raises(ValueError):
+        v.linear_vdm_w4a4(torch.zeros((4, 96), dtype=torch.float16, device=DEV), qw, ws)  # K % 64
+    with pytest.raises(ValueError):
+        v.linear_vdm_w4a4(x, qw[:64], ws[:64])  # N % 128
+    with pytest.raises(ValueError):
+        v.linear_vdm_w4a4(x, torch.zeros((128, 32), dtype=torch.uint8, device=DEV), ws)  # qweight [N, K/2]
+    with pytest.raises(ValueError):
+        v.linear_vdm_w4a4(x, qw, ws[:, :1])  # wscales [N, K/64]
+    with pytest.raises(RuntimeError):
+        v.linear_vdm_w4a4(x, qw.to(torch.int8), ws)  # dtype
+    with pytest.raises(RuntimeError):
+        v.linear_vdm_w4a4(x, qw, ws, bias=torch.zeros(64, dtype=torch.float16, device=DEV))  # bias length
+    with pytest.raises(RuntimeError):
+        v.linear_prequantized(torch.zeros((100, 64), dtype=torch.uint8, device=DEV), torch.zeros((100, 2), dtype=torch.float16, device=DEV), qw, ws)
+
+
+# ------------------------------------------------------ v1 layout surface
+
+def test_pack_weight_with_scale_emits_v1_layout():
+    v = vk()
+    rng = np.random.default_rng(7)
+    N, K = 256, 320
+    w = rng.standard_normal((N, K)).astype(np.float16)
+    scale = (np.abs(w.astype(np.float32)).max(axis=1) / 7).astype(np.float16)
+    qweight, packed_scales, channel_scales = v.pack_weight_with_scale(t16(w), t16(scale))
+    q = O.c_quantize_rows(w, scale)
+    assert np.array_equal(qweight.cpu().numpy(), O.c_pack_wgt_v1(q))
+    assert np.array_equal(packed_scales.cpu().numpy().view(np.uint16), O.c_pack_wscales_v1(scale, K).view(np.uint16))
+    assert np.array_equal(channel_scales.cpu().numpy().view(np.uint16), scale.view(np.uint16))
+    # derived scales: absmax / 7 with clip 1 (vdm_w4a4_kernel.cu:730-763)
+    q2, p2, s2 = v.quantize_weight_per_channel(t16(w))
+    s_want = O.c_row_scale(w, 1.0)
+    assert np.array_equal(s2.cpu().numpy().view(np.uint16), s_want.view(np.uint16))
+    assert np.array_equal(q2.cpu().numpy(), O.c_pack_wgt_v1(O.c_quantize_rows(w, s_want)))
+    assert np.array_equal(p2.cpu().numpy().view(np.uint16), O.c_pack_wscales_v1(s_want, K).view(np.uint16))
+
+
+def test_weight_relayout_roundtrip_and_cache():
+    from dsaquant_amd import _lib
+
+    v = vk()
+    lib = _lib.load()
+    rng = np.random.default_rng(8)
+    N, K = 384, 448
+    qw = rng.integers(-8, 8, (N, K), dtype=np.int8)
+    v1 = t16(O.np_pack_wgt_v1(qw))
+    ws = rng.random(N).astype(np.float16)
+    sv1 = t16(O.np_pack_wscales_v1(ws, K))
+    native, plain = v._native_weights(v1, sv1)
+    assert v._native_weights(v1, sv1)[0] is native  # cached
+    assert np.array_equal(unpack_native(native.cpu().numpy(), K), qw)
+    assert np.array_equal(plain.cpu().numpy().view(np.uint16), ws.view(np.uint16))
+    back = torch.empty_like(v1)
+    _lib.check(lib.vdmq_weight_native_to_v1(native.data_ptr(), back.data_ptr(), N, K, None))
+    torch.cuda.synchronize()
+    assert torch.equal(back, v1)
+
+
+def test_quantize_activation_per_token_v1_and_prequantized():
+    v = vk()
+    M, K, N = 300, 192, 256
+    x, qw, ws, _ = O.synth_linear(M, K, N, seed=9)
+    qact, ascales, act_scales = v.quantize_activation_per_token(t16(x), 0.95)
+    s = O.c_row_scale(x, 0.95)
+    q = O.c_quantize_rows(x, s)
+    assert qact.shape == (512, K // 2) and ascales.shape == (512, K // 64) and act_scales.shape == (M,)
+    assert np.array_equal(qact.cpu().numpy(), O.c_pack_act_v1(q))
+    assert np.array_equal(ascales.cpu().numpy().view(np.uint16), O.c_pack_ascales_v1(s, K).view(np.uint16))
+    assert np.array_equal(act_scales.cpu().numpy().view(np.uint16), s.view(np.uint16))
+    y = v.linear_prequantized(qact, ascales, t16(O.np_pack_wgt_v1(qw)), t16(O.np_pack_wscales_v1(ws, K)))
+    assert y.shape == (512, N)
+    want = O.np_epilogue(O.np_gemm_i32(q, qw), s, ws, None)
+    got = y.cpu().numpy()
+    assert np.array_equal(got[:M].view(np.uint16), want.view(np.uint16))
+    assert not got[M:].any()  # padded rows: zero activations, scale 1
+
+
+# --------------------------------------------------------------- fused QKV
+
+def test_fused_qkv_is_bitwise_three_separate_calls():
+    """What the reference's tests/test_vdm_qkv_fuse_smoke.py compares."""
+    v = vk()
+    M, K, N = 257, 1536, 1536
+    x = O.synth_linear(M, K, N, seed=2)[0]
+    parts = [O.synth_linear(8, K, N, seed=20 + i) for i in range(3)]
+    W = [t16(O.np_pack_wgt_v1(p[1])) for p in parts]
+    S = [t16(O.np_pack_wscales_v1(p[2], K)) for p in parts]
+    B = [t16(p[3]) for p in parts]
+    xt = t16(x).reshape(1, M, K)
+    sep = [v.linear_vdm_w4a4(xt, W[i], S[i], B[i], clip_ratio=0.95) for i in range(3)]
+    q, k, val = v.linear_vdm_w4a4_qkv(xt, W[0], S[0], W[1], S[1], W[2], S[2], B[0], None, B[2], clip_ratio=0.95)
+    assert q.shape == (1, M, N) and q.data_ptr() != k.data_ptr()
+    assert torch.equal(q, sep[0]) and torch.equal(val, sep[2])
+    k_nobias = v.linear_vdm_w4a4(xt, W[1], S[1], None, clip_ratio=0.95)
+    assert torch.equal(k, k_nobias)  # a missing bias is a zero bias: h + 0 == h in fp16
+    # cached concatenation path
+    wq = torch.cat(W, 0).contiguous()
+    sq = torch.cat(S, 0).contiguous()
+    bq = torch.cat(B, 0).contiguous()
+    q2, k2, v2 = v.linear_vdm_w4a4_qkv(xt, W[0], S[0], W[1], S[1], W[2], S[2], clip_ratio=0.95, w_qkv_packed=wq, w_qkv_scale=sq, qkv_bias_half=bq)
+    assert torch.equal(q2, sep[0]) and torch.equal(k2, sep[1]) and torch.equal(v2, sep[2])
+
+
+# ---------------------------------------------------- full-size properties
+
+def test_config3_sized_rows_sampled_against_oracle_and_ragged_tail():
+    """Wan-14B 720p fused QKV shape with the ragged M = 75600 + 37: a sample of
+    rows (including the last tile's tail) against the oracle, every row's token
+    scale, and the un-ragged prefix against a second run with M = 75600."""
+    v = vk()
+    M, K, N = 75637, 5120, 15360
+    g = torch.Generator(device="cpu").manual_seed(0)
+    x = torch.randn((M, K), generator=g, dtype=torch.float32)
+    cols = torch.randperm(K, generator=g)[: int(np.ceil(0.01 * K))]
+    x[:, cols] *= 20
+    x = x.half()
+    _, qw, ws, bias = O.synth_linear(1, K, N, seed=0)
+    qv1, sv1, b = t16(O.np_pack_wgt_v1(qw)), t16(O.np_pack_wscales_v1(ws, K)), t16(bias)
+    xd = x.to(DEV)
+    print("config-3 ragged linear", flush=True)
+    y = v.linear_vdm_w4a4(xd, qv1, sv1, b, clip_ratio=1.0)
+    y0 = v.linear_vdm_w4a4(xd[:75600], qv1, sv1, b, clip_ratio=1.0)
+    torch.cuda.synchronize()
+    assert torch.equal(y[:75600], y0)
+    rows = np.concatenate([np.arange(0, 64), np.arange(37800, 37832), np.arange(75580, M)])
+    want, _, _, _ = O.np_linear(x[rows].numpy(), qw, ws, bias, 1.0)
+    assert np.array_equal(y[torch.from_numpy(rows).to(DEV)].cpu().numpy().view(np.uint16), want.view(np.uint16))
+    # row-permutation equivariance on a shuffled block (exact)
+    perm = torch.randperm(4096, generator=g)
+    yp = v.linear_vdm_w4a4(xd[:4096][perm.to(DEV)], qv1, sv1, b, clip_ratio=1.0)
+    assert torch.equal(yp, y[:4096][perm.to(DEV)])
+    _, sc = v.quantize_activation_native(xd, 1.0)
+    assert np.array_equal(sc.cpu().numpy().view(np.uint16), O.np_row_scale(x.numpy(), 1.0).view(np.uint16))

@@ -1,0 +1,255 @@
+"""CPU-side checks: the C ABI loads and exports what include/vdmq.h declares,
+and the host logic that mirrors the reference's Python modules (QuantLinear,
+packed checkpoints, fused-QKV dispatch) behaves like the source it restates.
+No compute call is made on the library here (there is no GPU)."""
+import re
+from pathlib import Path
+
+import pytest
+import torch
+import torch.nn as nn
+
+ROOT = Path(__file__).resolve().parents[1]
+
+
+def test_library_exports_every_declared_symbol():
+    from dsaquant_amd import _lib
+
+    header = (ROOT / "include" / "vdmq.h").read_text()
+    declared = set(re.findall(r"\b(vdmq_[a-z0-9_]+)\s*\(", header))
+    declared.discard("vdmq_stream_t")
+    assert declared, "no declarations found"
+    lib = _lib.load()
+    for name in sorted(declared):
+        assert hasattr(lib, name), f"libvdmq.so does not export {name}"
+    assert declared == set(_lib.SIGNATURES), "ctypes signatures and header disagree"
+    # pure host calls
+    assert lib.vdmq_version() >= 1
+    assert lib.vdmq_arch() == b"gfx950"
+    assert lib.vdmq_k_padded(64) % 64 == 0 and lib.vdmq_k_padded(64) >= 64
+    assert lib.vdmq_k_padded(5120) == 5120
+    assert lib.vdmq_workspace_bytes(100, 1536) >= 100 * 768 + 200
+
+
+def test_abi_rejects_bad_shapes_without_touching_the_gpu():
+    from dsaquant_amd import _lib
+
+    lib = _lib.load()
+    fake = 4096  # a non-null, 16-byte aligned address; never dereferenced because the checks fail first
+    assert lib.vdmq_quantize_act(fake, 4, 96, 96, 1.0, fake, fake, None) == -2
+    assert b"K must be" in lib.vdmq_last_error()
+    assert lib.vdmq_gemm_w4a4(fake, fake, fake, fake, None, fake, 0, 4, 64, 128, 64, None) == -2
+    assert b"N must be" in lib.vdmq_last_error()
+    assert lib.vdmq_gemm_w4a4(None, fake, fake, fake, None, fake, 0, 4, 128, 128, 128, None) == -1
+    assert lib.vdmq_gemm_w4a4(fake, fake, fake + 4, fake, None, fake, 0, 4, 128, 128, 128, None) == -1
+    assert b"aligned" in lib.vdmq_last_error()
+    assert lib.vdmq_gemm_w4a4(fake, fake, fake, fake, None, fake, 7, 4, 128, 128, 128, None) == -1
+    assert lib.vdmq_linear_w4a4(fake, 4, 128, 128, 1.0, fake, fake, None, fake, 0, 128, 128, fake, 16, None) == -4
+    assert lib.vdmq_act_v1_to_native(fake, fake, 100, 128, fake, fake, None) == -2
+    assert lib.vdmq_quantize_act(fake, 0, 128, 128, 1.0, fake, fake, None) == 0  # empty input is fine
+    with pytest.raises(_lib.VdmqError):
+        _lib.check(-2)
+
+
+def test_kernel_wrapper_is_unavailable_without_a_gpu_and_never_falls_back():
+    from dsaquant_amd.kernels import vdm_w4a4 as v
+
+    if torch.cuda.is_available():
+        pytest.skip("GPU present")
+    assert v.is_available() is False
+    assert v.load_error() is not None
+    with pytest.raises(BaseException):
+        v.linear_vdm_w4a4(torch.zeros(4, 128), torch.zeros(128, 64, dtype=torch.uint8), torch.zeros(128, 2, dtype=torch.float16))
+    assert (v.BLOCK_M, v.BLOCK_N, v.WARP_K) == (256, 128, 64)
+    assert v.build_config()["arch_list"] == "gfx950"
+
+
+def _qparams():
+    return {"w": {"bit": 4, "sym": True, "granularity": "per_channel", "group_size": -1, "round_zero": True, "use_grad_scaling": True, "cali": "mse"},
+            "act": {"bit": 4, "sym": True}}
+
+
+def _make_ql(i=64, o=128, bias=True):
+    from dsaquant_amd.quantization.quant_linear import QuantLinear
+
+    return QuantLinear(nn.Linear(i, o, bias=bias), {"w": "lsq", "act": "dynamic"}, _qparams())
+
+
+def test_quantlinear_attributes_and_fake_quant_path():
+    torch.manual_seed(1)
+    ql = _make_ql()
+    for name, val in dict(use_wq=False, use_aq=False, use_hadamard=False, use_timestep_scaling=False, use_kernel=False,
+                          use_kernel_fused=False, use_vdm_kernel=False, kernel_clip_ratio=0.95, _bias_half=None, in_features=64,
+                          out_features=128).items():
+        assert getattr(ql, name) == val
+    x = torch.randn(9, 64)
+    y_fp = ql(x)
+    assert torch.allclose(y_fp, torch.nn.functional.linear(x, ql.weight, ql.bias))
+    ql.set_quant_state(use_wq=True, use_aq=True)
+    y = ql(x)
+    # closed form of the fake-quant path: symmetric int4, scale = absmax/7 clamped at 1e-5, per row
+    ws = ql.weight.detach().abs().amax(dim=1, keepdim=True).clamp(min=1e-5) / 7
+    wq = torch.clamp(torch.round(ql.weight.detach() / ws), -8, 7) * ws
+    xs = x.abs().amax(dim=1, keepdim=True).clamp(min=1e-5) / 7
+    xq = torch.clamp(torch.round(x / xs), -8, 7) * xs
+    assert torch.allclose(y, torch.nn.functional.linear(xq, wq, ql.bias), atol=1e-6)
+    assert torch.equal(ql.wquantizer.scale, ws)
+    # the activation scale is frozen after the first call (quant_linear.py:77-78)
+    y2 = ql(x * 100)
+    xq2 = torch.clamp(torch.round(x * 100 / xs), -8, 7) * xs
+    assert torch.allclose(y2, torch.nn.functional.linear(xq2, wq, ql.bias), atol=1e-6)
+    assert "use_vdm_kernel=False" in ql.extra_repr()
+    with pytest.raises(NotImplementedError):
+        ql.set_hadamard(True)
+    keys = set(ql.state_dict())
+    assert {"weight", "bias", "wquantizer.scale", "aquantizer.scale"} <= keys
+
+
+def test_uniform_quantizer_asymmetric_and_granularities():
+    from dsaquant_amd.quantization.quant_linear import UniformQuantizer
+
+    x = torch.tensor([[0.0, 1.0, 2.0, 3.0], [-1.0, 0.0, 1.0, 15.0]])
+    q = UniformQuantizer(bit=4, sym=False)
+    y = q(x)
+    assert torch.allclose(y[0], x[0], atol=1e-6)  # 0..3 on a 16-level grid of step 0.2
+    assert (q.P, q.N) == (15, 0) and q.zero_point is not None
+    for gran, rows in (("per_tensor", 1), ("per_channel", 2), ("per_token", 2)):
+        u = UniformQuantizer(granularity=gran)
+        u(x)
+        assert u.scale.shape[0] == rows
+    with pytest.raises(ValueError):
+        UniformQuantizer(granularity="nope")(x)
+    g = UniformQuantizer(granularity="per_group", group_size=2)
+    g(x)
+    assert g.scale.shape[0] == 4
+
+
+def test_enable_kernel_mode_fails_loudly_without_the_library_or_gpu():
+    if torch.cuda.is_available():
+        pytest.skip("GPU present")
+    ql = _make_ql()
+    ql.wquantizer(ql.weight.detach())
+    with pytest.raises(AssertionError, match="not compiled/available"):
+        ql.enable_vdm_kernel_mode()
+    assert ql.use_vdm_kernel is False and ql.weight is not None
+
+
+class _Attn(nn.Module):
+    def __init__(self, dim=128, cross=False):
+        super().__init__()
+        self.to_q, self.to_k, self.to_v = _make_ql(dim, dim), _make_ql(dim, dim), _make_ql(dim, dim)
+        self.cross_attention_dim_head = 64 if cross else None
+        self.fused_projections = False
+
+
+class _Toy(nn.Module):
+    def __init__(self):
+        super().__init__()
+        self.pre = nn.Linear(8, 128)
+        self.blocks = nn.ModuleList([_Attn(), _Attn(cross=True)])
+
+
+def _synthetic_packed_ckpt(model, legacy=False):
+    from dsaquant_amd.checkpoints import packed_checkpoint as pc
+    from dsaquant_amd.quantization.quant_linear import QuantLinear
+
+    sd = {}
+    for k, v in model.state_dict().items():
+        if ".wquantizer." in k or ".aquantizer." in k:
+            continue
+        sd[k] = v.detach().clone()
+    sfx = pc._LEGACY_BUFFER_SUFFIXES if legacy else pc.VDM_BUFFER_SUFFIXES
+    for name, m in model.named_modules():
+        if isinstance(m, QuantLinear):
+            n, k = m.out_features, m.in_features
+            del sd[f"{name}.weight"]
+            sd[f"{name}.{sfx[0]}"] = torch.randint(0, 256, (n, k // 2), dtype=torch.uint8)
+            sd[f"{name}.{sfx[1]}"] = torch.rand(n, k // 64).half()
+            sd[f"{name}.{sfx[2]}"] = torch.rand(n).half()
+    fmt = pc._LEGACY_PACKED_CHECKPOINT_FORMAT if legacy else pc.PACKED_CHECKPOINT_FORMAT
+    return {"format": fmt, "metadata": {"note": "synthetic"}, "model": sd}
+
+
+@pytest.mark.parametrize("legacy", [False, True])
+def test_packed_checkpoint_loader_contract(legacy, tmp_path):
+    from dsaquant_amd.checkpoints import packed_checkpoint as pc
+    from dsaquant_amd.quantization.quant_linear import QuantLinear
+
+    torch.manual_seed(0)
+    src = _Toy()
+    ckpt = _synthetic_packed_ckpt(src, legacy)
+    assert pc.is_packed_checkpoint(ckpt) and not pc.is_packed_checkpoint({"model": {}}) and not pc.is_packed_checkpoint([1])
+    # through a file, with the safe loader
+    path = str(tmp_path / "packed.pt")
+    torch.save(ckpt, path)
+    loaded = pc.load_quant_checkpoint(path, dcp_loader=lambda p: pytest.fail("dcp loader must not be used for .pt"))
+    assert pc.load_quant_checkpoint("some_dir", dcp_loader=lambda p: {"dcp": p}) == {"dcp": "some_dir"}
+
+    model = _Toy()
+    missing, unexpected = pc.load_packed_quantized_model(model, loaded, quant_linear_cls=QuantLinear, dtype=torch.float16,
+                                                        device=torch.device("cpu"), require_vdm_kernel=False)
+    assert missing == [] and unexpected == []
+    n = 0
+    for name, m in model.named_modules():
+        if isinstance(m, QuantLinear):
+            n += 1
+            assert m.use_vdm_kernel and not m.use_kernel and m.weight is None and m.wquantizer is None and m.aquantizer is None
+            assert m.use_wq and m.use_aq
+            assert m.vdm_weight_packed.dtype == torch.uint8 and m.vdm_weight_scale_packed.dtype == torch.float16
+            assert m._bias_half.dtype == torch.float16 and torch.equal(m._bias_half, m.bias.half())
+            key = f"{name}.{(pc._LEGACY_BUFFER_SUFFIXES if legacy else pc.VDM_BUFFER_SUFFIXES)[0]}"
+            assert torch.equal(m.vdm_weight_packed, ckpt["model"][key])
+    assert n == 6
+    assert model.pre.weight.dtype == torch.float16 and torch.equal(model.pre.weight, src.pre.weight.half())
+
+    # exporter: what goes back to disk
+    sd = pc.packed_state_dict_from_model(model)
+    assert not any(".wquantizer." in k or ".aquantizer." in k or k.endswith("._bias_half") or k.endswith("to_q.weight") for k in sd)
+    assert sd["blocks.0.to_q.vdm_weight_packed"].dtype == torch.uint8
+    out = str(tmp_path / "again.pt")
+    pc.save_packed_checkpoint(model, out, metadata={"a": 1})
+    again = torch.load(out, weights_only=True)
+    assert again["format"] == pc.PACKED_CHECKPOINT_FORMAT and again["metadata"] == {"a": 1}
+    assert set(again["model"]) == set(sd)
+
+    pc.enable_fused_qkv(model, quant_linear_cls=QuantLinear, attention_cls=_Attn, use_fused_qkv=True)
+    assert all(b.use_fused_qkv_kernel and b.qkv_kernel_backend == "vdm" for b in model.blocks)
+
+
+def test_packed_checkpoint_loader_errors():
+    from dsaquant_amd.checkpoints import packed_checkpoint as pc
+    from dsaquant_amd.quantization.quant_linear import QuantLinear
+
+    kw = dict(quant_linear_cls=QuantLinear, dtype=torch.float16, device=torch.device("cpu"), require_vdm_kernel=False)
+    with pytest.raises(ValueError, match="Unsupported checkpoint format"):
+        pc.load_packed_quantized_model(_Toy(), {"format": "other", "model": {}}, **kw)
+    ckpt = _synthetic_packed_ckpt(_Toy())
+    del ckpt["model"]["blocks.1.to_k.vdm_weight_scale"]
+    with pytest.raises(KeyError, match="missing 1 VDM buffers"):
+        pc.load_packed_quantized_model(_Toy(), ckpt, **kw)
+    plain = nn.Sequential(nn.Linear(4, 4))
+    with pytest.raises(RuntimeError, match="No QuantLinear"):
+        pc.load_packed_quantized_model(plain, {"format": pc.PACKED_CHECKPOINT_FORMAT, "model": plain.state_dict()}, **kw)
+    if not torch.cuda.is_available():
+        with pytest.raises(AssertionError):
+            pc.load_packed_quantized_model(_Toy(), _synthetic_packed_ckpt(_Toy()), quant_linear_cls=QuantLinear,
+                                           dtype=torch.float16, device=torch.device("cpu"))
+
+
+def test_fused_qkv_dispatch_falls_through_to_separate_projections_on_cpu():
+    from dsaquant_amd.fused_qkv import get_qkv_projections
+
+    torch.manual_seed(3)
+    attn = _Attn()
+    x = torch.randn(2, 5, 128)
+    q, k, v = get_qkv_projections(attn, x, None)
+    assert torch.equal(q, attn.to_q(x)) and torch.equal(k, attn.to_k(x)) and torch.equal(v, attn.to_v(x))
+    enc = torch.randn(2, 3, 128)
+    cross = _Attn(cross=True)
+    q, k, v = get_qkv_projections(cross, x, enc)
+    assert q.shape == (2, 5, 128) and k.shape == (2, 3, 128) and torch.equal(v, cross.to_v(enc))
+    # fp fused projections (attention.py:109-116)
+    attn.fused_projections = True
+    attn.to_qkv = nn.Linear(128, 384)
+    q, k, v = get_qkv_projections(attn, x, None)
+    assert torch.equal(torch.cat([q, k, v], -1), attn.to_qkv(x))
