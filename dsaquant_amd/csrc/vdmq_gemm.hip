@@ -25,6 +25,8 @@ typedef int v4i __attribute__((ext_vector_type(4)));
 typedef int v16i __attribute__((ext_vector_type(16)));
 typedef unsigned int u32x4 __attribute__((ext_vector_type(4)));
 typedef unsigned int u32x2 __attribute__((ext_vector_type(2)));
+typedef _Float16 f16x2 __attribute__((ext_vector_type(2)));
+typedef _Float16 f16x4 __attribute__((ext_vector_type(4)));
 
 constexpr int kRowBytes = kKStep / 2; /* bytes of one operand row per K step */
 
@@ -155,7 +157,7 @@ __global__ __launch_bounds__(WAVES_M *WAVES_N *kWaveSize) void gemm_w4a4_kernel(
         const int m = m0 + wm0 + mi * 32 + l32;
         if (m >= M) continue;
         float as = 0.0f;
-        if (!ACC_OUT) as = __half2float(ascale[m]);
+        if (!ACC_OUT) as = static_cast<float>(reinterpret_cast<const _Float16 *>(ascale)[m]);
 #pragma unroll
         for (int ni = 0; ni < Cfg::kNI; ++ni) {
 #pragma unroll
@@ -168,22 +170,17 @@ __global__ __launch_bounds__(WAVES_M *WAVES_N *kWaveSize) void gemm_w4a4_kernel(
                     for (int e = 0; e < 4; ++e) o[e] = acc[ni][mi][rg * 4 + e] >> 8;
                     *reinterpret_cast<v4i *>(acc_out + static_cast<int64_t>(m) * N + n) = o;
                 } else {
-                    const u32x2 wsb = *reinterpret_cast<const u32x2 *>(wscale + n);
-                    const __half2 ws01 = __builtin_bit_cast(__half2, wsb.x), ws23 = __builtin_bit_cast(__half2, wsb.y);
-                    const float ws[4] = {__low2float(ws01), __high2float(ws01), __low2float(ws23), __high2float(ws23)};
+                    const f16x4 ws = *reinterpret_cast<const f16x4 *>(wscale + n);
                     float v[4];
 #pragma unroll
-                    for (int e = 0; e < 4; ++e) v[e] = static_cast<float>(acc[ni][mi][rg * 4 + e] >> 8) * (as * ws[e]);
+                    for (int e = 0; e < 4; ++e)
+                        v[e] = static_cast<float>(acc[ni][mi][rg * 4 + e] >> 8) * (as * static_cast<float>(ws[e]));
                     if (out_dtype == VDMQ_OUT_F16) {
-                        __half2 h01 = __floats2half2_rn(v[0], v[1]);
-                        __half2 h23 = __floats2half2_rn(v[2], v[3]);
-                        if (bias != nullptr) {
-                            const u32x2 bb = *reinterpret_cast<const u32x2 *>(bias + n);
-                            h01 = __hadd2(h01, __builtin_bit_cast(__half2, bb.x));
-                            h23 = __hadd2(h23, __builtin_bit_cast(__half2, bb.y));
-                        }
-                        u32x2 o = {__builtin_bit_cast(uint32_t, h01), __builtin_bit_cast(uint32_t, h23)};
-                        *reinterpret_cast<u32x2 *>(static_cast<__half *>(out) + static_cast<int64_t>(m) * ldo + n) = o;
+                        // float -> _Float16 conversions round to nearest even
+                        f16x4 h = {static_cast<_Float16>(v[0]), static_cast<_Float16>(v[1]), static_cast<_Float16>(v[2]),
+                                   static_cast<_Float16>(v[3])};
+                        if (bias != nullptr) h += *reinterpret_cast<const f16x4 *>(bias + n); /* one fp16 add per element */
+                        *reinterpret_cast<f16x4 *>(static_cast<__half *>(out) + static_cast<int64_t>(m) * ldo + n) = h;
                     } else {
                         // bf16 output (not offered by the reference): same fp32 product, the
                         // fp16-rounded bias added in fp32, one rounding to bf16.
@@ -194,7 +191,7 @@ __global__ __launch_bounds__(WAVES_M *WAVES_N *kWaveSize) void gemm_w4a4_kernel(
 #pragma unroll
                             for (int e = 0; e < 2; ++e) {
                                 float f = v[2 * e2 + e];
-                                if (bias != nullptr) f += __half2float(bias[n + 2 * e2 + e]);
+                                if (bias != nullptr) f += static_cast<float>(reinterpret_cast<const _Float16 *>(bias)[n + 2 * e2 + e]);
                                 uint32_t u = __float_as_uint(f);
                                 u = (f != f) ? 0x7FC00000u : u + 0x7FFFu + ((u >> 16) & 1u); /* RNE */
                                 pk |= (u >> 16) << (16 * e);

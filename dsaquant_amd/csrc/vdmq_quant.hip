@@ -18,6 +18,7 @@ namespace {
 
 typedef unsigned short u16x2 __attribute__((ext_vector_type(2)));
 typedef unsigned int u32x4 __attribute__((ext_vector_type(4)));
+typedef _Float16 f16x2 __attribute__((ext_vector_type(2)));
 
 __device__ __forceinline__ uint32_t pk_max_u16(uint32_t a, uint32_t b) {
     u16x2 r = __builtin_elementwise_max(__builtin_bit_cast(u16x2, a), __builtin_bit_cast(u16x2, b));
@@ -25,7 +26,7 @@ __device__ __forceinline__ uint32_t pk_max_u16(uint32_t a, uint32_t b) {
 }
 
 __device__ __forceinline__ float half_bits_to_float(uint32_t bits16) {
-    return __half2float(__ushort_as_half(static_cast<unsigned short>(bits16)));
+    return static_cast<float>(__builtin_bit_cast(_Float16, static_cast<unsigned short>(bits16)));
 }
 
 template <typename T>
@@ -75,9 +76,9 @@ __device__ __forceinline__ uint32_t quantize_word_fast(u32x4 v, float rscale) {
     uint32_t acc = 0;
 #pragma unroll
     for (int i = 0; i < 4; ++i) {
-        float2 f = __half22float2(__builtin_bit_cast(__half2, w[i]));
-        float t0 = __builtin_amdgcn_fmed3f(f.x * rscale, -8.0f, 7.0f);
-        float t1 = __builtin_amdgcn_fmed3f(f.y * rscale, -8.0f, 7.0f);
+        const f16x2 h = __builtin_bit_cast(f16x2, w[i]);
+        float t0 = __builtin_amdgcn_fmed3f(static_cast<float>(h[0]) * rscale, -8.0f, 7.0f);
+        float t1 = __builtin_amdgcn_fmed3f(static_cast<float>(h[1]) * rscale, -8.0f, 7.0f);
         acc += __float_as_uint(t0 + kMagic) << (8 * i);
         acc += __float_as_uint(t1 + kMagic) << (8 * i + 4);
     }
