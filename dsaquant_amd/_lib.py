@@ -8,7 +8,8 @@ from pathlib import Path
 from typing import Optional
 
 _PKG = Path(__file__).resolve().parent
-LIB_PATH = _PKG / "libvdmq.so"
+# VDMQ_LIBRARY points at another build of the same C ABI (e.g. a tuning variant)
+LIB_PATH = Path(os.environ.get("VDMQ_LIBRARY", str(_PKG / "libvdmq.so")))
 CSRC = _PKG / "csrc"
 
 _LIB: Optional[ctypes.CDLL] = None

@@ -3,9 +3,12 @@
 //   acc[m,n] = sum_k qx[m,k] * qw[n,k]   exact int32
 //   out[m,n] = fp16(float(acc) * (float(as[m]) * float(ws[n]))) (+ bias[n] in fp16)
 //
-// Packed int4 tiles of both operands (row-major, 64 bytes = 128 k per row and
-// K step) are staged through LDS.  A lane reads 16 bytes (32 nibbles) of one
-// row and widens each 32-bit word p into two MFMA operand registers
+// Data path.  Both operands are row-major packed int4 (64 bytes = 128 k per
+// row and K step).  A workgroup owns a BM x BN output tile and walks K through
+// a ring of LDS stages filled by 128-bit direct-to-LDS loads
+// (global_load_lds_dwordx4: no VGPR staging, no ds_write).  A lane reads 16
+// bytes (32 nibbles) of one row from LDS and widens each 32-bit word p into two
+// MFMA operand registers
 //     lo = (p << 4) & 0xF0F0F0F0   (even-k nibbles, as int8 = 16*q)
 //     hi =  p       & 0xF0F0F0F0   (odd-k nibbles,  as int8 = 16*q)
 // Both operands are widened the same way, so k pairs up correctly whatever
@@ -16,6 +19,17 @@
 // MFMA orientation: the A operand holds weight rows (n), the B operand token
 // rows (m), so a lane's four consecutive accumulator registers are four
 // consecutive n of one token: an 8-byte fp16 store.
+//
+// LDS layout of a stage: rows 0..BN-1 are weight rows, BN..BN+BM-1 token rows,
+// 64 bytes each; the four 16-byte pieces of row r are stored at piece index
+// p ^ ((r/4)%4), which makes the 16 lanes of a ds_read_b128 phase hit 16
+// different bank groups (measured: zero bank conflicts).
+//
+// Synchronisation: the direct-to-LDS loads are tracked by vmcnt only and the
+// stage ring is published with raw s_barrier (no fence: a workgroup fence
+// would drain every load in flight), so the waits are written by hand below.
+#include <type_traits>
+
 #include "vdmq_internal.h"
 
 namespace vdmq {
@@ -24,16 +38,24 @@ namespace {
 typedef int v4i __attribute__((ext_vector_type(4)));
 typedef int v16i __attribute__((ext_vector_type(16)));
 typedef unsigned int u32x4 __attribute__((ext_vector_type(4)));
-typedef unsigned int u32x2 __attribute__((ext_vector_type(2)));
-typedef _Float16 f16x2 __attribute__((ext_vector_type(2)));
 typedef _Float16 f16x4 __attribute__((ext_vector_type(4)));
+typedef _Float16 f16x8 __attribute__((ext_vector_type(8)));
+
+#define VDMQ_GLOBAL_PTR(p) ((const __attribute__((address_space(1))) void *)(p))
+#define VDMQ_LDS_PTR(p) ((__attribute__((address_space(3))) void *)(p))
 
 constexpr int kRowBytes = kKStep / 2; /* bytes of one operand row per K step */
 
-// LDS byte offset of 16-byte piece `p` (0..3) of tile row `r`.  XOR-ing the
-// piece index with (r/4)%4 spreads 16 consecutive rows reading the same piece
-// over all 64 banks.
-__device__ __forceinline__ int lds_piece_offset(int r, int p) { return r * kRowBytes + ((p ^ ((r >> 2) & 3)) << 4); }
+// s_waitcnt immediate for gfx9: vmcnt[3:0] | expcnt[6:4] | lgkmcnt[11:8] | vmcnt[15:14]
+constexpr int waitcnt_imm(int vm, int lgkm) { return (vm & 15) | ((vm >> 4) << 14) | (7 << 4) | ((lgkm & 15) << 8); }
+
+__device__ __forceinline__ void lds_barrier() {
+    asm volatile("" ::: "memory");
+#ifndef VDMQ_DBG_NOBARRIER
+    __builtin_amdgcn_s_barrier();
+#endif
+    asm volatile("" ::: "memory");
+}
 
 __device__ __forceinline__ v4i widen(uint32_t p0, uint32_t p1) {
     v4i r;
@@ -44,65 +66,161 @@ __device__ __forceinline__ v4i widen(uint32_t p0, uint32_t p1) {
     return r;
 }
 
-template <int BM, int BN, int WAVES_M, int WAVES_N>
+template <int BM_, int BN_, int WAVES_M_, int WAVES_N_, int STAGES_, int OCC_ = 1>
 struct GemmCfg {
-    static constexpr int kThreads = WAVES_M * WAVES_N * kWaveSize;
+    static constexpr int kOccupancy = OCC_; /* workgroups per CU the register budget must allow */
+    static constexpr int BM = BM_, BN = BN_, WAVES_M = WAVES_M_, WAVES_N = WAVES_N_, STAGES = STAGES_;
+    static constexpr int kWaves = WAVES_M * WAVES_N;
+    static constexpr int kThreads = kWaves * kWaveSize;
     static constexpr int kWaveM = BM / WAVES_M;
     static constexpr int kWaveN = BN / WAVES_N;
     static constexpr int kMI = kWaveM / 32;
     static constexpr int kNI = kWaveN / 32;
-    static constexpr int kStageBytes = (BM + BN) * kRowBytes;
-    static constexpr int kPieces = (BM + BN) * 4; /* 16-byte pieces per stage */
-    static constexpr int kPiecesPerThread = kPieces / kThreads;
-    static_assert(kPieces % kThreads == 0, "stage must divide evenly over the threads");
-    static_assert(kWaveM % 32 == 0 && kWaveN % 32 == 0, "wave tile is made of 32x32 MFMA tiles");
+    static constexpr int kRows = BM + BN;
+    static constexpr int kStageBytes = kRows * kRowBytes;
+    static constexpr int kLdsBytes = kStageBytes * STAGES;
+    // one direct-to-LDS instruction of one wave fills 16 rows (1 KiB)
+    static constexpr int kRowBlocks = kRows / 16;
+    static constexpr int kLoads = kRowBlocks / kWaves; /* per wave (= per lane) and stage */
+    // epilogue staging: one 32-row strip of the wave tile as fp16, rows padded by 16 bytes
+    static constexpr int kStageRowBytes = kWaveN * 2 + 16;
+    static constexpr int kStagingBytes = 32 * kStageRowBytes;
+    static constexpr int kPiecesPerRow = kWaveN / 8; /* 16-byte pieces of one strip row */
+    static_assert(kStagingBytes * kWaves <= kStageBytes * STAGES_, "epilogue staging reuses the stage ring");
+    static_assert(kRowBlocks % kWaves == 0, "row blocks must divide evenly over the waves");
+    static_assert(BN % 16 == 0 && kWaveM % 32 == 0 && kWaveN % 32 == 0, "tile shape");
+    static_assert(kLoads * (STAGES - 1) < 64, "vmcnt is a 6-bit counter");
 };
 
-template <typename Cfg, int BM, int BN>
-__device__ __forceinline__ void load_stage(u32x4 (&regs)[Cfg::kPiecesPerThread], const uint8_t *__restrict__ A,
-                                           const uint8_t *__restrict__ W, int m0, int n0, int M, int N, int ldk, int kbyte) {
+// Issue the direct-to-LDS loads of one stage.  `woff`/`xoff` are per-lane byte
+// offsets (clamped to valid rows) from the wave-uniform bases.
+template <typename Cfg>
+__device__ __forceinline__ void issue_stage(const uint8_t *wbase, const uint8_t *xbase, const uint32_t (&off)[Cfg::kLoads],
+                                            uint8_t *lds_stage, int wave) {
 #pragma unroll
-    for (int i = 0; i < Cfg::kPiecesPerThread; ++i) {
-        const int q = i * Cfg::kThreads + threadIdx.x;
-        const int r = q >> 2, p = q & 3;
-        u32x4 v = {0u, 0u, 0u, 0u};
-        if (r < BN) {
-            const int n = n0 + r;
-            if (n < N) v = *reinterpret_cast<const u32x4 *>(W + static_cast<int64_t>(n) * ldk + kbyte + p * 16);
-        } else {
-            const int m = m0 + (r - BN);
-            if (m < M) v = *reinterpret_cast<const u32x4 *>(A + static_cast<int64_t>(m) * ldk + kbyte + p * 16);
-        }
-        regs[i] = v;
+    for (int i = 0; i < Cfg::kLoads; ++i) {
+        const int rb = i * Cfg::kWaves + wave; /* wave-uniform row block */
+        const uint8_t *base = (rb * 16 < Cfg::BN) ? wbase : xbase;
+        __builtin_amdgcn_global_load_lds(VDMQ_GLOBAL_PTR(base + off[i]), VDMQ_LDS_PTR(lds_stage + rb * 1024), 16, 0, 0);
     }
 }
 
 template <typename Cfg>
-__device__ __forceinline__ void store_stage(const u32x4 (&regs)[Cfg::kPiecesPerThread], uint8_t *lds) {
+__device__ __forceinline__ void read_frags(u32x4 (&wf)[Cfg::kNI], u32x4 (&xf)[Cfg::kMI], const uint8_t *lds_stage, uint32_t waddr,
+                                           uint32_t xaddr) {
 #pragma unroll
-    for (int i = 0; i < Cfg::kPiecesPerThread; ++i) {
-        const int q = i * Cfg::kThreads + threadIdx.x;
-        *reinterpret_cast<u32x4 *>(lds + lds_piece_offset(q >> 2, q & 3)) = regs[i];
+    for (int ni = 0; ni < Cfg::kNI; ++ni) wf[ni] = *reinterpret_cast<const u32x4 *>(lds_stage + waddr + ni * 32 * kRowBytes);
+#pragma unroll
+    for (int mi = 0; mi < Cfg::kMI; ++mi) xf[mi] = *reinterpret_cast<const u32x4 *>(lds_stage + xaddr + mi * 32 * kRowBytes);
+}
+
+// Operand registers of one K=32 MFMA step for the whole wave tile.
+template <typename Cfg>
+struct Operands {
+    v4i a[Cfg::kNI]; /* weight rows */
+    v4i b[Cfg::kMI]; /* token rows */
+};
+
+template <typename Cfg, int HALF>
+__device__ __forceinline__ void widen_frags(Operands<Cfg> &o, const u32x4 (&wf)[Cfg::kNI], const u32x4 (&xf)[Cfg::kMI]) {
+#pragma unroll
+    for (int ni = 0; ni < Cfg::kNI; ++ni) o.a[ni] = HALF ? widen(wf[ni].z, wf[ni].w) : widen(wf[ni].x, wf[ni].y);
+#pragma unroll
+    for (int mi = 0; mi < Cfg::kMI; ++mi) o.b[mi] = HALF ? widen(xf[mi].z, xf[mi].w) : widen(xf[mi].x, xf[mi].y);
+}
+
+template <typename Cfg>
+__device__ __forceinline__ void mma_step(v16i (&acc)[Cfg::kNI][Cfg::kMI], const Operands<Cfg> &o) {
+#pragma unroll
+    for (int ni = 0; ni < Cfg::kNI; ++ni)
+#pragma unroll
+        for (int mi = 0; mi < Cfg::kMI; ++mi) acc[ni][mi] = __builtin_amdgcn_mfma_i32_32x32x32_i8(o.a[ni], o.b[mi], acc[ni][mi], 0, 0, 0);
+}
+
+// Instruction-mix hint for one half K step (2 x kNI*kMI MFMAs): one MFMA, then
+// three widening VALU ops; the LDS reads (and, in the second half, the global
+// loads) are spread over the first MFMAs.  Without it the widening ops pile up
+// in front of the first MFMA of the region and the matrix pipe idles.
+template <typename Cfg, bool WITH_VMEM>
+__device__ __forceinline__ void schedule_half_step() {
+    constexpr int kMfma = 2 * Cfg::kNI * Cfg::kMI;
+    constexpr int kDs = Cfg::kNI + Cfg::kMI;
+#pragma unroll
+    for (int i = 0; i < kMfma; ++i) {
+        __builtin_amdgcn_sched_group_barrier(0x008, 1, 0); /* MFMA */
+        if (i < kDs) __builtin_amdgcn_sched_group_barrier(0x100, 1, 0); /* DS read */
+        if (WITH_VMEM && i >= kDs && i < kDs + Cfg::kLoads) __builtin_amdgcn_sched_group_barrier(0x020, 1, 0); /* VMEM read */
+        __builtin_amdgcn_sched_group_barrier(0x002, 3, 0); /* VALU */
     }
 }
 
-// Rows 0..BN-1 of a stage are weight rows, rows BN..BN+BM-1 token rows.
-template <int BM, int BN, int WAVES_M, int WAVES_N, bool ACC_OUT>
-__global__ __launch_bounds__(WAVES_M *WAVES_N *kWaveSize) void gemm_w4a4_kernel(
-    const uint8_t *__restrict__ A, const uint8_t *__restrict__ W, const __half *__restrict__ ascale,
-    const __half *__restrict__ wscale, const __half *__restrict__ bias, void *__restrict__ out, int out_dtype,
-    int32_t *__restrict__ acc_out, int M, int N, int ldk, int64_t ldo, int tiles_n) {
-    using Cfg = GemmCfg<BM, BN, WAVES_M, WAVES_N>;
-    __shared__ __attribute__((aligned(16))) uint8_t lds[2][Cfg::kStageBytes];
+// Tile order.  Workgroups are dealt round-robin to the 8 XCDs (each with its own
+// L2), so workgroup b runs on XCD b%8 as its (b/8)-th.  Each XCD walks
+// "super-tiles" of kGroupM x kGroupN tiles (32 = its CU count): the tiles that are
+// resident on an XCD together share kGroupM token row-blocks and kGroupN weight
+// row-blocks, and the 8 XCDs work on neighbouring super-tiles at any moment.
+constexpr int kXcds = 8, kGroupM = 8, kGroupN = 4;
 
-    const int tile_m = blockIdx.x / tiles_n;
-    const int tile_n = blockIdx.x % tiles_n;
+struct TileMap {
+    int tiles_m, tiles_n, super_n, total_super;
+};
+
+__device__ __forceinline__ bool map_tile(const TileMap &tm, int bid, int &tile_m, int &tile_n) {
+    const int xcd = bid % kXcds, slot = bid / kXcds;
+    const int per = kGroupM * kGroupN;
+    const int st = (slot / per) * kXcds + xcd;
+    const int j = slot % per;
+    if (st >= tm.total_super) return false;
+    tile_m = (st / tm.super_n) * kGroupM + j / kGroupN;
+    tile_n = (st % tm.super_n) * kGroupN + j % kGroupN;
+    return tile_m < tm.tiles_m && tile_n < tm.tiles_n;
+}
+
+template <typename Cfg, bool ACC_OUT>
+__global__ __launch_bounds__(Cfg::kThreads, Cfg::kOccupancy * Cfg::kWaves / 4) void gemm_w4a4_kernel(const uint8_t *__restrict__ A, const uint8_t *__restrict__ W,
+                                                                  const __half *__restrict__ ascale, const __half *__restrict__ wscale,
+                                                                  const __half *__restrict__ bias, void *__restrict__ out, int out_dtype,
+                                                                  int32_t *__restrict__ acc_out, int M, int N, int ldk, int64_t ldo,
+                                                                  TileMap tmap) {
+    constexpr int BM = Cfg::BM, BN = Cfg::BN, S = Cfg::STAGES, L = Cfg::kLoads;
+    extern __shared__ __attribute__((aligned(1024))) uint8_t lds[];
+
+    int tile_m, tile_n;
+    if (!map_tile(tmap, blockIdx.x, tile_m, tile_n)) return;
     const int m0 = tile_m * BM, n0 = tile_n * BN;
     const int lane = threadIdx.x & 63;
-    const int wave = threadIdx.x >> 6;
-    const int wm0 = (wave / WAVES_N) * Cfg::kWaveM; /* within the tile */
-    const int wn0 = (wave % WAVES_N) * Cfg::kWaveN;
+    const int wave = __builtin_amdgcn_readfirstlane(threadIdx.x >> 6);
+    const int wm0 = (wave / Cfg::WAVES_N) * Cfg::kWaveM; /* within the tile */
+    const int wn0 = (wave % Cfg::WAVES_N) * Cfg::kWaveN;
     const int l32 = lane & 31, lh = lane >> 5;
+
+    // ---- global -> LDS: per-lane source offsets (rows clamped into range: rows
+    // beyond M or N are loaded from the last valid row and never stored)
+    uint32_t goff[L];
+    {
+        const int r16 = lane >> 2;                    /* row inside the 16-row block */
+        const int piece = (lane & 3) ^ ((lane >> 4) & 3); /* (r/4)%4 == (lane/16)%4 inside a block */
+        const int wrows = min(BN, N - n0), xrows = min(BM, M - m0);
+#pragma unroll
+        for (int i = 0; i < L; ++i) {
+            const int r = (i * Cfg::kWaves + wave) * 16 + r16;
+            const int rr = r < BN ? min(r, wrows - 1) : min(r - BN, xrows - 1);
+            goff[i] = static_cast<uint32_t>(rr) * static_cast<uint32_t>(ldk) + piece * 16;
+        }
+    }
+    const uint8_t *wbase = W + static_cast<int64_t>(n0) * ldk;
+    const uint8_t *xbase = A + static_cast<int64_t>(m0) * ldk;
+
+    // ---- LDS -> registers: per-lane fragment addresses for the two 128-bit
+    // reads (j) of a K step; lanes 32..63 take the odd pieces
+    const int swz = (lane >> 2) & 3;
+    uint32_t waddr[2], xaddr[2];
+#pragma unroll
+    for (int j = 0; j < 2; ++j) {
+        const int piece = ((2 * j + lh) ^ swz) << 4;
+        waddr[j] = (wn0 + l32) * kRowBytes + piece;
+        xaddr[j] = (BN + wm0 + l32) * kRowBytes + piece;
+    }
 
     v16i acc[Cfg::kNI][Cfg::kMI];
 #pragma unroll
@@ -113,45 +231,122 @@ __global__ __launch_bounds__(WAVES_M *WAVES_N *kWaveSize) void gemm_w4a4_kernel(
             for (int r = 0; r < 16; ++r) acc[ni][mi][r] = 0;
 
     const int ksteps = ldk / kRowBytes;
-    u32x4 regs[Cfg::kPiecesPerThread];
-    load_stage<Cfg, BM, BN>(regs, A, W, m0, n0, M, N, ldk, 0);
-    store_stage<Cfg>(regs, lds[0]);
-    __syncthreads();
 
-    for (int kt = 0; kt < ksteps; ++kt) {
-        const uint8_t *cur = lds[kt & 1];
-        if (kt + 1 < ksteps) load_stage<Cfg, BM, BN>(regs, A, W, m0, n0, M, N, ldk, (kt + 1) * kRowBytes);
+    // prologue: fill S-1... all S stages of the ring (as far as K reaches)
+#pragma unroll
+    for (int s = 0; s < S; ++s)
+        if (s < ksteps) issue_stage<Cfg>(wbase + s * kRowBytes, xbase + s * kRowBytes, goff, lds + s * Cfg::kStageBytes, wave);
+    if (ksteps >= S)
+        __builtin_amdgcn_s_waitcnt(waitcnt_imm(L * (S - 1), 15));
+    else
+        __builtin_amdgcn_s_waitcnt(waitcnt_imm(0, 15));
+    lds_barrier();
 
-#pragma unroll
-        for (int j = 0; j < 2; ++j) {
-            u32x4 wf[Cfg::kNI], xf[Cfg::kMI];
-#pragma unroll
-            for (int ni = 0; ni < Cfg::kNI; ++ni)
-                wf[ni] = *reinterpret_cast<const u32x4 *>(cur + lds_piece_offset(wn0 + ni * 32 + l32, 2 * j + lh));
-#pragma unroll
-            for (int mi = 0; mi < Cfg::kMI; ++mi)
-                xf[mi] = *reinterpret_cast<const u32x4 *>(cur + lds_piece_offset(BN + wm0 + mi * 32 + l32, 2 * j + lh));
-#pragma unroll
-            for (int h = 0; h < 2; ++h) {
-                v4i a[Cfg::kNI], b[Cfg::kMI];
-#pragma unroll
-                for (int ni = 0; ni < Cfg::kNI; ++ni) a[ni] = h ? widen(wf[ni].z, wf[ni].w) : widen(wf[ni].x, wf[ni].y);
-#pragma unroll
-                for (int mi = 0; mi < Cfg::kMI; ++mi) b[mi] = h ? widen(xf[mi].z, xf[mi].w) : widen(xf[mi].x, xf[mi].y);
-#pragma unroll
-                for (int ni = 0; ni < Cfg::kNI; ++ni)
-#pragma unroll
-                    for (int mi = 0; mi < Cfg::kMI; ++mi)
-                        acc[ni][mi] = __builtin_amdgcn_mfma_i32_32x32x32_i8(a[ni], b[mi], acc[ni][mi], 0, 0, 0);
-            }
-        }
+    // Software pipeline.  F0/F1 are the raw LDS fragments of the two 128-bit
+    // reads (j = 0, 1) of a stage; `lo` holds the widened first half of the
+    // fragment about to be consumed, prepared one half step ahead.
+    u32x4 wf0[Cfg::kNI], xf0[Cfg::kMI], wf1[Cfg::kNI], xf1[Cfg::kMI];
+    Operands<Cfg> lo, hi;
+    read_frags<Cfg>(wf0, xf0, lds, waddr[0], xaddr[0]);
+    widen_frags<Cfg, 0>(lo, wf0, xf0);
 
-        if (kt + 1 < ksteps) store_stage<Cfg>(regs, lds[(kt + 1) & 1]);
-        __syncthreads();
-    }
+    // One K step.  STEADY: stage kt+S exists (so the slot is refilled, S-1 stages
+    // are in flight at the wait, and a next stage exists) -- a branch-free body
+    // the scheduler can interleave as one region per half step.
+    int cur = 0; /* ring slot of stage kt */
+    auto k_step = [&](int kt, auto steady_tag) {
+        constexpr bool STEADY = decltype(steady_tag)::value;
+        // ---- first half: consume (kt, j=0), fetch (kt, j=1)
+        read_frags<Cfg>(wf1, xf1, lds + cur * Cfg::kStageBytes, waddr[1], xaddr[1]);
+        widen_frags<Cfg, 1>(hi, wf0, xf0);
+        mma_step<Cfg>(acc, lo);
+        mma_step<Cfg>(acc, hi);
+        widen_frags<Cfg, 0>(lo, wf1, xf1);
+        schedule_half_step<Cfg, false>();
+
+        // Stage kt+1 must have landed and every wave must be done reading stage
+        // kt before its slot is refilled.  In steady state S-1 stages are in
+        // flight, so "at most S-2 stages outstanding" means stage kt+1 is in.
+#ifdef VDMQ_DBG_NOLOAD
+        if (STEADY)
+            __builtin_amdgcn_s_waitcnt(waitcnt_imm(63, 0));
+#else
+        if (STEADY)
+            __builtin_amdgcn_s_waitcnt(waitcnt_imm(L * (S - 2), 0));
+#endif
+        else
+            __builtin_amdgcn_s_waitcnt(waitcnt_imm(0, 0));
+        lds_barrier();
+
+        // ---- second half: consume (kt, j=1), refill the slot, fetch (kt+1, j=0)
+        // (the LDS reads come first in program order: the compiler must assume the
+        // direct-to-LDS loads may alias them and would not move reads above)
+        const int nxt = cur + 1 == S ? 0 : cur + 1;
+        if (STEADY || kt + 1 < ksteps) read_frags<Cfg>(wf0, xf0, lds + nxt * Cfg::kStageBytes, waddr[0], xaddr[0]);
+#ifndef VDMQ_DBG_NOLOAD
+        if (STEADY) issue_stage<Cfg>(wbase + (kt + S) * kRowBytes, xbase + (kt + S) * kRowBytes, goff, lds + cur * Cfg::kStageBytes, wave);
+#endif
+        cur = nxt;
+        widen_frags<Cfg, 1>(hi, wf1, xf1);
+        mma_step<Cfg>(acc, lo);
+        mma_step<Cfg>(acc, hi);
+        widen_frags<Cfg, 0>(lo, wf0, xf0);
+        schedule_half_step<Cfg, STEADY>();
+    };
+    int kt = 0;
+    for (; kt + S < ksteps; ++kt) k_step(kt, std::true_type{});
+    for (; kt < ksteps; ++kt) k_step(kt, std::false_type{});
 
     // Epilogue.  Accumulator register r of a 32x32 tile holds
     // n = 8*(r/4) + 4*(lane/32) + r%4, m = lane%32.
+    if (!ACC_OUT && out_dtype == VDMQ_OUT_F16) {
+        // fp16 path: scale in the accumulator layout, round to fp16, transpose one
+        // 32-row strip at a time through LDS (the stage ring is idle: every wave
+        // passed the last barrier after its final LDS read and no load is in
+        // flight), then add the bias and store 16 bytes per lane so that a row's
+        // kWaveN outputs leave as whole 128-byte lines.
+        constexpr int PR = Cfg::kPiecesPerRow, RS = Cfg::kStageRowBytes;
+        uint8_t *stg = lds + wave * Cfg::kStagingBytes;
+        const _Float16 *as_p = reinterpret_cast<const _Float16 *>(ascale);
+        f16x4 wsv[Cfg::kNI][4];
+#pragma unroll
+        for (int ni = 0; ni < Cfg::kNI; ++ni)
+#pragma unroll
+            for (int rg = 0; rg < 4; ++rg) {
+                const int n = n0 + wn0 + ni * 32 + rg * 8 + lh * 4;
+                wsv[ni][rg] = *reinterpret_cast<const f16x4 *>(wscale + min(n, N - 4));
+            }
+        const int ncol = n0 + wn0 + (lane % PR) * 8;
+        f16x8 bv = {0, 0, 0, 0, 0, 0, 0, 0};
+        if (bias != nullptr && ncol < N) bv = *reinterpret_cast<const f16x8 *>(bias + ncol);
+#pragma unroll
+        for (int mi = 0; mi < Cfg::kMI; ++mi) {
+            const int m = m0 + wm0 + mi * 32 + l32;
+            const float as = static_cast<float>(as_p[min(m, M - 1)]);
+#pragma unroll
+            for (int ni = 0; ni < Cfg::kNI; ++ni)
+#pragma unroll
+                for (int rg = 0; rg < 4; ++rg) {
+                    f16x4 h;
+#pragma unroll
+                    for (int e = 0; e < 4; ++e) {
+                        const float v = static_cast<float>(acc[ni][mi][rg * 4 + e] >> 8) * (as * static_cast<float>(wsv[ni][rg][e]));
+                        h[e] = static_cast<_Float16>(v); /* round to nearest even */
+                    }
+                    *reinterpret_cast<f16x4 *>(stg + l32 * RS + (ni * 32 + rg * 8 + lh * 4) * 2) = h;
+                }
+#pragma unroll
+            for (int it = 0; it < PR / 2; ++it) {
+                const int row = it * (64 / PR) + lane / PR;
+                f16x8 hv = *reinterpret_cast<const f16x8 *>(stg + row * RS + (lane % PR) * 16);
+                if (bias != nullptr) hv += bv; /* one fp16 add per element */
+                const int mrow = m0 + wm0 + mi * 32 + row;
+                if (mrow < M && ncol < N)
+                    *reinterpret_cast<f16x8 *>(static_cast<__half *>(out) + static_cast<int64_t>(mrow) * ldo + ncol) = hv;
+            }
+        }
+        return;
+    }
 #pragma unroll
     for (int mi = 0; mi < Cfg::kMI; ++mi) {
         const int m = m0 + wm0 + mi * 32 + l32;
@@ -170,56 +365,62 @@ __global__ __launch_bounds__(WAVES_M *WAVES_N *kWaveSize) void gemm_w4a4_kernel(
                     for (int e = 0; e < 4; ++e) o[e] = acc[ni][mi][rg * 4 + e] >> 8;
                     *reinterpret_cast<v4i *>(acc_out + static_cast<int64_t>(m) * N + n) = o;
                 } else {
+                    // bf16 output (not offered by the reference): same fp32 product, the
+                    // fp16 bias added in fp32, one rounding to bf16.
                     const f16x4 ws = *reinterpret_cast<const f16x4 *>(wscale + n);
-                    float v[4];
+                    uint32_t o[2];
 #pragma unroll
-                    for (int e = 0; e < 4; ++e)
-                        v[e] = static_cast<float>(acc[ni][mi][rg * 4 + e] >> 8) * (as * static_cast<float>(ws[e]));
-                    if (out_dtype == VDMQ_OUT_F16) {
-                        // float -> _Float16 conversions round to nearest even
-                        f16x4 h = {static_cast<_Float16>(v[0]), static_cast<_Float16>(v[1]), static_cast<_Float16>(v[2]),
-                                   static_cast<_Float16>(v[3])};
-                        if (bias != nullptr) h += *reinterpret_cast<const f16x4 *>(bias + n); /* one fp16 add per element */
-                        *reinterpret_cast<f16x4 *>(static_cast<__half *>(out) + static_cast<int64_t>(m) * ldo + n) = h;
-                    } else {
-                        // bf16 output (not offered by the reference): same fp32 product, the
-                        // fp16-rounded bias added in fp32, one rounding to bf16.
-                        uint32_t o[2];
+                    for (int e2 = 0; e2 < 2; ++e2) {
+                        uint32_t pk = 0;
 #pragma unroll
-                        for (int e2 = 0; e2 < 2; ++e2) {
-                            uint32_t pk = 0;
-#pragma unroll
-                            for (int e = 0; e < 2; ++e) {
-                                float f = v[2 * e2 + e];
-                                if (bias != nullptr) f += static_cast<float>(reinterpret_cast<const _Float16 *>(bias)[n + 2 * e2 + e]);
-                                uint32_t u = __float_as_uint(f);
-                                u = (f != f) ? 0x7FC00000u : u + 0x7FFFu + ((u >> 16) & 1u); /* RNE */
-                                pk |= (u >> 16) << (16 * e);
-                            }
-                            o[e2] = pk;
+                        for (int e = 0; e < 2; ++e) {
+                            float f = static_cast<float>(acc[ni][mi][rg * 4 + 2 * e2 + e] >> 8) * (as * static_cast<float>(ws[2 * e2 + e]));
+                            if (bias != nullptr) f += static_cast<float>(reinterpret_cast<const _Float16 *>(bias)[n + 2 * e2 + e]);
+                            uint32_t u = __float_as_uint(f);
+                            u = (f != f) ? 0x7FC00000u : u + 0x7FFFu + ((u >> 16) & 1u); /* RNE */
+                            pk |= (u >> 16) << (16 * e);
                         }
-                        u32x2 ov = {o[0], o[1]};
-                        *reinterpret_cast<u32x2 *>(static_cast<uint16_t *>(out) + static_cast<int64_t>(m) * ldo + n) = ov;
+                        o[e2] = pk;
                     }
+                    typedef unsigned int u32x2 __attribute__((ext_vector_type(2)));
+                    u32x2 ov = {o[0], o[1]};
+                    *reinterpret_cast<u32x2 *>(static_cast<uint16_t *>(out) + static_cast<int64_t>(m) * ldo + n) = ov;
                 }
             }
         }
     }
 }
 
-template <int BM, int BN, int WAVES_M, int WAVES_N>
+template <typename Cfg>
 int launch_cfg(const uint8_t *qact, const __half *ascale, const uint8_t *wq, const __half *wscale, const __half *bias, void *out,
                int out_dtype, int32_t *acc_out, int64_t M, int64_t N, int64_t K, int64_t ldo, hipStream_t s) {
-    const int tiles_m = static_cast<int>(ceil_div(M, BM));
-    const int tiles_n = static_cast<int>(ceil_div(N, BN));
+    TileMap tm;
+    tm.tiles_m = static_cast<int>(ceil_div(M, Cfg::BM));
+    tm.tiles_n = static_cast<int>(ceil_div(N, Cfg::BN));
+    const int super_m = static_cast<int>(ceil_div(tm.tiles_m, kGroupM));
+    tm.super_n = static_cast<int>(ceil_div(tm.tiles_n, kGroupN));
+    tm.total_super = super_m * tm.super_n;
+    const int rounds = static_cast<int>(ceil_div(tm.total_super, kXcds));
+    const dim3 grid(static_cast<unsigned>(rounds) * kXcds * kGroupM * kGroupN), block(Cfg::kThreads);
     const int ldk = static_cast<int>(k_padded(K) / 2);
-    const dim3 grid(static_cast<unsigned>(tiles_m) * tiles_n), block(WAVES_M * WAVES_N * kWaveSize);
-    if (acc_out != nullptr) {
-        hipLaunchKernelGGL((gemm_w4a4_kernel<BM, BN, WAVES_M, WAVES_N, true>), grid, block, 0, s, qact, wq, ascale, wscale, bias, out,
-                           out_dtype, acc_out, static_cast<int>(M), static_cast<int>(N), ldk, ldo, tiles_n);
+
+    // LDS above 64 KiB has to be requested once per kernel
+    static bool attr_done[2] = {false, false};
+    const int which = acc_out != nullptr ? 1 : 0;
+    auto kacc = gemm_w4a4_kernel<Cfg, true>;
+    auto kout = gemm_w4a4_kernel<Cfg, false>;
+    if (!attr_done[which]) {
+        hipError_t e = hipFuncSetAttribute(which ? reinterpret_cast<const void *>(kacc) : reinterpret_cast<const void *>(kout),
+                                           hipFuncAttributeMaxDynamicSharedMemorySize, Cfg::kLdsBytes);
+        if (e != hipSuccess) return fail(VDMQ_ELAUNCH, "hipFuncSetAttribute(%d bytes of LDS): %s", Cfg::kLdsBytes, hipGetErrorString(e));
+        attr_done[which] = true;
+    }
+    if (which) {
+        hipLaunchKernelGGL(kacc, grid, block, Cfg::kLdsBytes, s, qact, wq, ascale, wscale, bias, out, out_dtype, acc_out,
+                           static_cast<int>(M), static_cast<int>(N), ldk, ldo, tm);
     } else {
-        hipLaunchKernelGGL((gemm_w4a4_kernel<BM, BN, WAVES_M, WAVES_N, false>), grid, block, 0, s, qact, wq, ascale, wscale, bias, out,
-                           out_dtype, acc_out, static_cast<int>(M), static_cast<int>(N), ldk, ldo, tiles_n);
+        hipLaunchKernelGGL(kout, grid, block, Cfg::kLdsBytes, s, qact, wq, ascale, wscale, bias, out, out_dtype, acc_out,
+                           static_cast<int>(M), static_cast<int>(N), ldk, ldo, tm);
     }
     return check_launch("gemm_w4a4_kernel");
 }
@@ -229,7 +430,10 @@ int launch_cfg(const uint8_t *qact, const __half *ascale, const uint8_t *wq, con
 int launch_gemm(const uint8_t *qact, const __half *ascale, const uint8_t *wq, const __half *wscale, const __half *bias, void *out,
                 int out_dtype, int32_t *acc_out, int64_t M, int64_t N, int64_t K, int64_t ldo, hipStream_t s) {
     if (M == 0 || N == 0) return VDMQ_OK;
-    return launch_cfg<256, 128, 2, 2>(qact, ascale, wq, wscale, bias, out, out_dtype, acc_out, M, N, K, ldo, s);
+#ifndef VDMQ_GEMM_CFG
+#define VDMQ_GEMM_CFG 256, 256, 4, 2, 3, 1
+#endif
+    return launch_cfg<GemmCfg<VDMQ_GEMM_CFG>>(qact, ascale, wq, wscale, bias, out, out_dtype, acc_out, M, N, K, ldo, s);
 }
 
 }  // namespace vdmq
