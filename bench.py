@@ -103,6 +103,9 @@ def main():
     ap.add_argument("--warmup", type=int, default=5)
     ap.add_argument("--workload", default="wan14b_720p_block", choices=sorted(WORKLOADS))
     ap.add_argument("--no-cpu-baseline", action="store_true")
+    ap.add_argument("--calibrate-copy", action="store_true",
+                    help="also run the library's plain 1 GiB copy kernel three times first, so that a rocprofv3 --pmc FETCH_SIZE / WRITE_SIZE "
+                         "run holds a copy kernel of known size to scale the counters by")
     args = ap.parse_args()
     if args.gpus != 1:
         print("bench.py measures one GPU: the path shards by token rows with no exchange; run with --gpus 1", file=sys.stderr)
@@ -119,6 +122,15 @@ def main():
     torch.cuda.set_device(dev)
     wl = WORKLOADS[args.workload]
     M = wl["M"]
+
+    if args.calibrate_copy:
+        # the library's plain 128-bit copy kernel: reads 1 GiB, writes 1 GiB
+        src = torch.zeros(1 << 30, dtype=torch.uint8, device=dev)
+        dst = torch.empty_like(src)
+        for _ in range(3):
+            _lib.check(lib.vdmq_copy_u128(src.data_ptr(), dst.data_ptr(), src.numel(), torch.cuda.current_stream(dev).cuda_stream))
+        torch.cuda.synchronize()
+        del src, dst
 
     layers = []
     for i, (name, K, N) in enumerate(wl["linears"]):

@@ -37,6 +37,7 @@ SIGNATURES = {
     "vdmq_act_v1_to_native": (_int, [_p, _p, _i64, _i64, _p, _p, _p]),
     "vdmq_row_scale": (_int, [_p, _i64, _i64, _f32, _p, _p]),
     "vdmq_quantize_weight_native": (_int, [_p, _p, _p, _i64, _i64, _p]),
+    "vdmq_copy_u128": (_int, [_p, _p, _i64, _p]),
 }
 
 

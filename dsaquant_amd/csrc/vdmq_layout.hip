@@ -137,9 +137,25 @@ __global__ __launch_bounds__(256) void act_to_native_kernel(const uint32_t *__re
     if (widx < M) scale_h[widx] = ascales_v1[ascale_v1_index(widx, 0, KG)];
 }
 
+// Plain copy with 128-bit accesses (non-temporal loads, like the quantizer's):
+// a kernel of known traffic to scale hardware counters by.
+typedef unsigned int u32x4 __attribute__((ext_vector_type(4)));
+__global__ __launch_bounds__(256) void copy_u128_kernel(const u32x4 *__restrict__ src, u32x4 *__restrict__ dst, int64_t n) {
+    const int64_t i = static_cast<int64_t>(blockIdx.x) * blockDim.x + threadIdx.x;
+    if (i < n) dst[i] = __builtin_nontemporal_load(src + i);
+}
+
 unsigned blocks_for(int64_t n) { return static_cast<unsigned>(ceil_div(n > 0 ? n : 1, 256)); }
 
 }  // namespace
+
+int launch_copy_u128(const void *src, void *dst, int64_t bytes, hipStream_t s) {
+    const int64_t n = bytes / 16;
+    if (n == 0) return VDMQ_OK;
+    hipLaunchKernelGGL(copy_u128_kernel, dim3(blocks_for(n)), dim3(256), 0, s, static_cast<const u32x4 *>(src),
+                       static_cast<u32x4 *>(dst), n);
+    return check_launch("copy_u128_kernel");
+}
 
 int launch_weight_relayout(const void *src, void *dst, int64_t N, int64_t K, bool to_native, hipStream_t s) {
     const int Kp = static_cast<int>(k_padded(K));

@@ -128,6 +128,12 @@ int vdmq_row_scale(const void *w, int64_t rows, int64_t K, float clip, void *sca
  * returns are then vdmq_weight_native_to_v1 + vdmq_wscale_plain_to_v1. */
 int vdmq_quantize_weight_native(const void *w, const void *scale_h, void *wq_native, int64_t N, int64_t K, vdmq_stream_t stream);
 
+/* Plain device-to-device copy kernel with 128-bit accesses (bytes % 16 == 0).
+ * No counterpart in the reference: a kernel of exactly known HBM traffic
+ * (bytes read + bytes written), run next to the hot-path kernels when hardware
+ * traffic counters are collected so that their readings can be scaled. */
+int vdmq_copy_u128(const void *src, void *dst, int64_t bytes, vdmq_stream_t stream);
+
 #ifdef __cplusplus
 }
 #endif
