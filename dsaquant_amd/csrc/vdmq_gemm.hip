@@ -44,7 +44,6 @@ typedef _Float16 f16x8 __attribute__((ext_vector_type(8)));
 #define VDMQ_GLOBAL_PTR(p) ((const __attribute__((address_space(1))) void *)(p))
 #define VDMQ_LDS_PTR(p) ((__attribute__((address_space(3))) void *)(p))
 
-constexpr int kRowBytes = kKStep / 2; /* bytes of one operand row per K step */
 
 // s_waitcnt immediate for gfx9: vmcnt[3:0] | expcnt[6:4] | lgkmcnt[11:8] | vmcnt[15:14]
 constexpr int waitcnt_imm(int vm, int lgkm) { return (vm & 15) | ((vm >> 4) << 14) | (7 << 4) | ((lgkm & 15) << 8); }
@@ -66,9 +65,17 @@ __device__ __forceinline__ v4i widen(uint32_t p0, uint32_t p1) {
     return r;
 }
 
-template <int BM_, int BN_, int WAVES_M_, int WAVES_N_, int STAGES_, int OCC_ = 1>
+template <int BM_, int BN_, int WAVES_M_, int WAVES_N_, int STAGES_, int OCC_ = 1, int KSTEP_ = 128>
 struct GemmCfg {
     static constexpr int kOccupancy = OCC_; /* workgroups per CU the register budget must allow */
+    static constexpr int kKStepElems = KSTEP_;       /* k per LDS stage: 128 or 256 */
+    static constexpr int kRowBytes = KSTEP_ / 2;     /* bytes of one operand row per stage */
+    static constexpr int kPieces = kRowBytes / 16;   /* 16-byte pieces per row: 4 or 8 */
+    static constexpr int kReads = kPieces / 2;       /* 128-bit fragment reads per lane and stage */
+    static constexpr int kSwzShift = kPieces == 4 ? 2 : 1; /* piece index is XORed with (row >> shift) % kPieces */
+    static constexpr int kDmaRows = 64 / kPieces;    /* rows filled by one direct-to-LDS wave instruction */
+    static_assert(KSTEP_ == 128 || KSTEP_ == 256, "K step");
+    static_assert(kKStep % KSTEP_ == 0, "native rows are padded to kKStep");
     static constexpr int BM = BM_, BN = BN_, WAVES_M = WAVES_M_, WAVES_N = WAVES_N_, STAGES = STAGES_;
     static constexpr int kWaves = WAVES_M * WAVES_N;
     static constexpr int kThreads = kWaves * kWaveSize;
@@ -79,8 +86,8 @@ struct GemmCfg {
     static constexpr int kRows = BM + BN;
     static constexpr int kStageBytes = kRows * kRowBytes;
     static constexpr int kLdsBytes = kStageBytes * STAGES;
-    // one direct-to-LDS instruction of one wave fills 16 rows (1 KiB)
-    static constexpr int kRowBlocks = kRows / 16;
+    // one direct-to-LDS instruction of one wave fills kDmaRows rows (1 KiB)
+    static constexpr int kRowBlocks = kRows / kDmaRows;
     static constexpr int kLoads = kRowBlocks / kWaves; /* per wave (= per lane) and stage */
     // epilogue staging: one 32-row strip of the wave tile as fp16, rows padded by 16 bytes
     static constexpr int kStageRowBytes = kWaveN * 2 + 16;
@@ -88,7 +95,7 @@ struct GemmCfg {
     static constexpr int kPiecesPerRow = kWaveN / 8; /* 16-byte pieces of one strip row */
     static_assert(kStagingBytes * kWaves <= kStageBytes * STAGES_, "epilogue staging reuses the stage ring");
     static_assert(kRowBlocks % kWaves == 0, "row blocks must divide evenly over the waves");
-    static_assert(BN % 16 == 0 && kWaveM % 32 == 0 && kWaveN % 32 == 0, "tile shape");
+    static_assert(BN % kDmaRows == 0 && kWaveM % 32 == 0 && kWaveN % 32 == 0, "tile shape");
     static_assert(kLoads * (STAGES - 1) < 64, "vmcnt is a 6-bit counter");
 };
 
@@ -100,7 +107,7 @@ __device__ __forceinline__ void issue_stage(const uint8_t *wbase, const uint8_t 
 #pragma unroll
     for (int i = 0; i < Cfg::kLoads; ++i) {
         const int rb = i * Cfg::kWaves + wave; /* wave-uniform row block */
-        const uint8_t *base = (rb * 16 < Cfg::BN) ? wbase : xbase;
+        const uint8_t *base = (rb * Cfg::kDmaRows < Cfg::BN) ? wbase : xbase;
         __builtin_amdgcn_global_load_lds(VDMQ_GLOBAL_PTR(base + off[i]), VDMQ_LDS_PTR(lds_stage + rb * 1024), 16, 0, 0);
     }
 }
@@ -109,9 +116,9 @@ template <typename Cfg>
 __device__ __forceinline__ void read_frags(u32x4 (&wf)[Cfg::kNI], u32x4 (&xf)[Cfg::kMI], const uint8_t *lds_stage, uint32_t waddr,
                                            uint32_t xaddr) {
 #pragma unroll
-    for (int ni = 0; ni < Cfg::kNI; ++ni) wf[ni] = *reinterpret_cast<const u32x4 *>(lds_stage + waddr + ni * 32 * kRowBytes);
+    for (int ni = 0; ni < Cfg::kNI; ++ni) wf[ni] = *reinterpret_cast<const u32x4 *>(lds_stage + waddr + ni * 32 * Cfg::kRowBytes);
 #pragma unroll
-    for (int mi = 0; mi < Cfg::kMI; ++mi) xf[mi] = *reinterpret_cast<const u32x4 *>(lds_stage + xaddr + mi * 32 * kRowBytes);
+    for (int mi = 0; mi < Cfg::kMI; ++mi) xf[mi] = *reinterpret_cast<const u32x4 *>(lds_stage + xaddr + mi * 32 * Cfg::kRowBytes);
 }
 
 // Operand registers of one K=32 MFMA step for the whole wave tile.
@@ -163,6 +170,7 @@ constexpr int kXcds = 8, kGroupM = 8, kGroupN = 4;
 
 struct TileMap {
     int tiles_m, tiles_n, super_n, total_super;
+    int stream_out; /* non-temporal output stores */
 };
 
 __device__ __forceinline__ bool map_tile(const TileMap &tm, int bid, int &tile_m, int &tile_n) {
@@ -194,16 +202,16 @@ __global__ __launch_bounds__(Cfg::kThreads, Cfg::kOccupancy * Cfg::kWaves / 4) v
     const int wn0 = (wave % Cfg::WAVES_N) * Cfg::kWaveN;
     const int l32 = lane & 31, lh = lane >> 5;
 
+    constexpr int RB = Cfg::kRowBytes, R = Cfg::kReads;
     // ---- global -> LDS: per-lane source offsets (rows clamped into range: rows
     // beyond M or N are loaded from the last valid row and never stored)
     uint32_t goff[L];
     {
-        const int r16 = lane >> 2;                    /* row inside the 16-row block */
-        const int piece = (lane & 3) ^ ((lane >> 4) & 3); /* (r/4)%4 == (lane/16)%4 inside a block */
         const int wrows = min(BN, N - n0), xrows = min(BM, M - m0);
 #pragma unroll
         for (int i = 0; i < L; ++i) {
-            const int r = (i * Cfg::kWaves + wave) * 16 + r16;
+            const int r = (i * Cfg::kWaves + wave) * Cfg::kDmaRows + lane / Cfg::kPieces; /* stage row this lane fills */
+            const int piece = (lane % Cfg::kPieces) ^ ((r >> Cfg::kSwzShift) % Cfg::kPieces);
             const int rr = r < BN ? min(r, wrows - 1) : min(r - BN, xrows - 1);
             goff[i] = static_cast<uint32_t>(rr) * static_cast<uint32_t>(ldk) + piece * 16;
         }
@@ -211,15 +219,16 @@ __global__ __launch_bounds__(Cfg::kThreads, Cfg::kOccupancy * Cfg::kWaves / 4) v
     const uint8_t *wbase = W + static_cast<int64_t>(n0) * ldk;
     const uint8_t *xbase = A + static_cast<int64_t>(m0) * ldk;
 
-    // ---- LDS -> registers: per-lane fragment addresses for the two 128-bit
-    // reads (j) of a K step; lanes 32..63 take the odd pieces
-    const int swz = (lane >> 2) & 3;
-    uint32_t waddr[2], xaddr[2];
+    // ---- LDS -> registers: per-lane fragment addresses for the R 128-bit reads
+    // (j) of a stage; lanes 32..63 take the odd pieces.  Tile row offsets are
+    // multiples of 32, so the swizzle term only depends on the lane.
+    const int swz = (l32 >> Cfg::kSwzShift) % Cfg::kPieces;
+    uint32_t waddr[R], xaddr[R];
 #pragma unroll
-    for (int j = 0; j < 2; ++j) {
+    for (int j = 0; j < R; ++j) {
         const int piece = ((2 * j + lh) ^ swz) << 4;
-        waddr[j] = (wn0 + l32) * kRowBytes + piece;
-        xaddr[j] = (BN + wm0 + l32) * kRowBytes + piece;
+        waddr[j] = (wn0 + l32) * RB + piece;
+        xaddr[j] = (BN + wm0 + l32) * RB + piece;
     }
 
     v16i acc[Cfg::kNI][Cfg::kMI];
@@ -230,68 +239,73 @@ __global__ __launch_bounds__(Cfg::kThreads, Cfg::kOccupancy * Cfg::kWaves / 4) v
 #pragma unroll
             for (int r = 0; r < 16; ++r) acc[ni][mi][r] = 0;
 
-    const int ksteps = ldk / kRowBytes;
+    const int ksteps = ldk / RB;
 
-    // prologue: fill S-1... all S stages of the ring (as far as K reaches)
+    // prologue: fill the ring (as far as K reaches), wait for stage 0
 #pragma unroll
     for (int s = 0; s < S; ++s)
-        if (s < ksteps) issue_stage<Cfg>(wbase + s * kRowBytes, xbase + s * kRowBytes, goff, lds + s * Cfg::kStageBytes, wave);
+        if (s < ksteps) issue_stage<Cfg>(wbase + s * RB, xbase + s * RB, goff, lds + s * Cfg::kStageBytes, wave);
     if (ksteps >= S)
         __builtin_amdgcn_s_waitcnt(waitcnt_imm(L * (S - 1), 15));
     else
         __builtin_amdgcn_s_waitcnt(waitcnt_imm(0, 15));
     lds_barrier();
 
-    // Software pipeline.  F0/F1 are the raw LDS fragments of the two 128-bit
-    // reads (j = 0, 1) of a stage; `lo` holds the widened first half of the
-    // fragment about to be consumed, prepared one half step ahead.
-    u32x4 wf0[Cfg::kNI], xf0[Cfg::kMI], wf1[Cfg::kNI], xf1[Cfg::kMI];
+    // Software pipeline.  fa/fb hold the raw LDS fragments of the 128-bit read
+    // being consumed and of the next one; `lo` holds the widened first half of
+    // the fragment about to be consumed, prepared one step ahead.
+    u32x4 wfa[Cfg::kNI], xfa[Cfg::kMI], wfb[Cfg::kNI], xfb[Cfg::kMI];
     Operands<Cfg> lo, hi;
-    read_frags<Cfg>(wf0, xf0, lds, waddr[0], xaddr[0]);
-    widen_frags<Cfg, 0>(lo, wf0, xf0);
+    read_frags<Cfg>(wfa, xfa, lds, waddr[0], xaddr[0]);
+    widen_frags<Cfg, 0>(lo, wfa, xfa);
 
-    // One K step.  STEADY: stage kt+S exists (so the slot is refilled, S-1 stages
-    // are in flight at the wait, and a next stage exists) -- a branch-free body
-    // the scheduler can interleave as one region per half step.
+    // One stage (K step).  STEADY: stage kt+S exists (so the slot is refilled,
+    // S-1 stages are in flight at the wait, and a next stage exists) -- a
+    // branch-free body the scheduler can interleave as one region per read.
+    // Read j of the stage is consumed while read j+1 (or read 0 of the next
+    // stage) is fetched; the ring is published by ONE barrier per stage, placed
+    // before the last read's MFMAs: by then every wave has finished its LDS
+    // reads of the stage, so its slot can be refilled.
     int cur = 0; /* ring slot of stage kt */
     auto k_step = [&](int kt, auto steady_tag) {
         constexpr bool STEADY = decltype(steady_tag)::value;
-        // ---- first half: consume (kt, j=0), fetch (kt, j=1)
-        read_frags<Cfg>(wf1, xf1, lds + cur * Cfg::kStageBytes, waddr[1], xaddr[1]);
-        widen_frags<Cfg, 1>(hi, wf0, xf0);
-        mma_step<Cfg>(acc, lo);
-        mma_step<Cfg>(acc, hi);
-        widen_frags<Cfg, 0>(lo, wf1, xf1);
-        schedule_half_step<Cfg, false>();
-
-        // Stage kt+1 must have landed and every wave must be done reading stage
-        // kt before its slot is refilled.  In steady state S-1 stages are in
-        // flight, so "at most S-2 stages outstanding" means stage kt+1 is in.
-#ifdef VDMQ_DBG_NOLOAD
-        if (STEADY)
-            __builtin_amdgcn_s_waitcnt(waitcnt_imm(63, 0));
-#else
-        if (STEADY)
-            __builtin_amdgcn_s_waitcnt(waitcnt_imm(L * (S - 2), 0));
-#endif
-        else
-            __builtin_amdgcn_s_waitcnt(waitcnt_imm(0, 0));
-        lds_barrier();
-
-        // ---- second half: consume (kt, j=1), refill the slot, fetch (kt+1, j=0)
-        // (the LDS reads come first in program order: the compiler must assume the
-        // direct-to-LDS loads may alias them and would not move reads above)
+        const uint8_t *stage = lds + cur * Cfg::kStageBytes;
         const int nxt = cur + 1 == S ? 0 : cur + 1;
-        if (STEADY || kt + 1 < ksteps) read_frags<Cfg>(wf0, xf0, lds + nxt * Cfg::kStageBytes, waddr[0], xaddr[0]);
+#pragma unroll
+        for (int j = 0; j < R; ++j) {
+            // fragments alternate between the a and b register sets
+            auto &wc = (j & 1) ? wfb : wfa;
+            auto &xc = (j & 1) ? xfb : xfa;
+            auto &wn = (j & 1) ? wfa : wfb;
+            auto &xn = (j & 1) ? xfa : xfb;
+            if (j + 1 < R) {
+                read_frags<Cfg>(wn, xn, stage, waddr[j + 1], xaddr[j + 1]);
+            } else {
+                // Stage kt+1 must have landed and every wave must be done reading
+                // stage kt before its slot is refilled.  In steady state S-1 stages
+                // are in flight, so "at most S-2 outstanding" means kt+1 is in.
+                if (STEADY)
+                    __builtin_amdgcn_s_waitcnt(waitcnt_imm(L * (S - 2), 0));
+                else
+                    __builtin_amdgcn_s_waitcnt(waitcnt_imm(0, 0));
+                lds_barrier();
+                // (the LDS reads come first in program order: the compiler must assume
+                // the direct-to-LDS loads may alias them and would not move reads above)
+                if (STEADY || kt + 1 < ksteps) read_frags<Cfg>(wn, xn, lds + nxt * Cfg::kStageBytes, waddr[0], xaddr[0]);
 #ifndef VDMQ_DBG_NOLOAD
-        if (STEADY) issue_stage<Cfg>(wbase + (kt + S) * kRowBytes, xbase + (kt + S) * kRowBytes, goff, lds + cur * Cfg::kStageBytes, wave);
+                if (STEADY) issue_stage<Cfg>(wbase + (kt + S) * RB, xbase + (kt + S) * RB, goff, lds + cur * Cfg::kStageBytes, wave);
 #endif
+            }
+            widen_frags<Cfg, 1>(hi, wc, xc);
+            mma_step<Cfg>(acc, lo);
+            mma_step<Cfg>(acc, hi);
+            widen_frags<Cfg, 0>(lo, wn, xn);
+            if (j + 1 < R)
+                schedule_half_step<Cfg, false>();
+            else
+                schedule_half_step<Cfg, STEADY>();
+        }
         cur = nxt;
-        widen_frags<Cfg, 1>(hi, wf1, xf1);
-        mma_step<Cfg>(acc, lo);
-        mma_step<Cfg>(acc, hi);
-        widen_frags<Cfg, 0>(lo, wf0, xf0);
-        schedule_half_step<Cfg, STEADY>();
     };
     int kt = 0;
     for (; kt + S < ksteps; ++kt) k_step(kt, std::true_type{});
@@ -341,8 +355,16 @@ __global__ __launch_bounds__(Cfg::kThreads, Cfg::kOccupancy * Cfg::kWaves / 4) v
                 f16x8 hv = *reinterpret_cast<const f16x8 *>(stg + row * RS + (lane % PR) * 16);
                 if (bias != nullptr) hv += bv; /* one fp16 add per element */
                 const int mrow = m0 + wm0 + mi * 32 + row;
-                if (mrow < M && ncol < N)
-                    *reinterpret_cast<f16x8 *>(static_cast<__half *>(out) + static_cast<int64_t>(mrow) * ldo + ncol) = hv;
+                if (mrow < M && ncol < N) {
+                    f16x8 *dst = reinterpret_cast<f16x8 *>(static_cast<__half *>(out) + static_cast<int64_t>(mrow) * ldo + ncol);
+                    // A large output is not re-read before it falls out of the caches anyway:
+                    // streaming it keeps the operands (and the next quantizer's writes) in
+                    // the Infinity Cache (measured: next quantizer 5.76 -> 6.01 TB/s).
+                    if (tmap.stream_out)
+                        __builtin_nontemporal_store(hv, dst);
+                    else
+                        *dst = hv;
+                }
             }
         }
         return;
@@ -400,6 +422,7 @@ int launch_cfg(const uint8_t *qact, const __half *ascale, const uint8_t *wq, con
     const int super_m = static_cast<int>(ceil_div(tm.tiles_m, kGroupM));
     tm.super_n = static_cast<int>(ceil_div(tm.tiles_n, kGroupN));
     tm.total_super = super_m * tm.super_n;
+    tm.stream_out = (M * N * 2 > (int64_t(224) << 20)) ? 1 : 0;
     const int rounds = static_cast<int>(ceil_div(tm.total_super, kXcds));
     const dim3 grid(static_cast<unsigned>(rounds) * kXcds * kGroupM * kGroupN), block(Cfg::kThreads);
     const int ldk = static_cast<int>(k_padded(K) / 2);
@@ -431,7 +454,7 @@ int launch_gemm(const uint8_t *qact, const __half *ascale, const uint8_t *wq, co
                 int out_dtype, int32_t *acc_out, int64_t M, int64_t N, int64_t K, int64_t ldo, hipStream_t s) {
     if (M == 0 || N == 0) return VDMQ_OK;
 #ifndef VDMQ_GEMM_CFG
-#define VDMQ_GEMM_CFG 256, 256, 4, 2, 3, 1
+#define VDMQ_GEMM_CFG 256, 256, 2, 4, 2, 1, 256
 #endif
     return launch_cfg<GemmCfg<VDMQ_GEMM_CFG>>(qact, ascale, wq, wscale, bias, out, out_dtype, acc_out, M, N, K, ldo, s);
 }

@@ -9,9 +9,9 @@
 
 namespace vdmq {
 
-// The GEMM consumes K in steps of this many elements; native rows are padded
-// with zero nibbles up to a multiple of it.
-constexpr int kKStep = 128;
+// Native rows are padded with zero nibbles up to a multiple of this many
+// elements; the GEMM consumes K in steps that divide it (128 or 256).
+constexpr int kKStep = 256;
 
 constexpr int kWaveSize = 64;
 

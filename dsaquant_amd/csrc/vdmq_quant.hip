@@ -116,9 +116,19 @@ __device__ __forceinline__ bool scale_is_ordinary(__half s) {
 
 constexpr int kRowsPerBlock = 4; /* one wave per row */
 
+template <bool STREAM>
+__device__ __forceinline__ void store_word(uint32_t *p, uint32_t w) {
+    if (STREAM)
+        __builtin_nontemporal_store(w, p);
+    else
+        *p = w;
+}
+
 // NCH = number of 512-element chunks (one 128-bit load per lane each) that
-// cover the padded row.
-template <int NCH>
+// cover the padded row.  STREAM_OUT: write the nibbles with non-temporal
+// stores -- measured faster once the output no longer fits the 256 MB
+// Infinity Cache (5.35 -> 5.9 TB/s at K = 13824, M = 75600), slower below.
+template <int NCH, bool STREAM_OUT>
 __global__ __launch_bounds__(kRowsPerBlock * kWaveSize) void quantize_rows_kernel(const __half *__restrict__ x, int64_t ldx,
                                                                                   int M, int K, int Kp, float clip,
                                                                                   uint8_t *__restrict__ qact,
@@ -153,7 +163,7 @@ __global__ __launch_bounds__(kRowsPerBlock * kWaveSize) void quantize_rows_kerne
 #pragma unroll
         for (int c = 0; c < NCH; ++c) {
             const int k0 = c * 512 + lane * 8;
-            if (k0 < Kp) dst[c * 64 + lane] = quantize_word_fast(v[c], rscale);
+            if (k0 < Kp) store_word<STREAM_OUT>(dst + c * 64 + lane, quantize_word_fast(v[c], rscale));
         }
     } else {
         float mx = 0.0f;
@@ -166,7 +176,7 @@ __global__ __launch_bounds__(kRowsPerBlock * kWaveSize) void quantize_rows_kerne
 #pragma unroll
         for (int c = 0; c < NCH; ++c) {
             const int k0 = c * 512 + lane * 8;
-            if (k0 < Kp) dst[c * 64 + lane] = quantize_word_exact(v[c], rscale);
+            if (k0 < Kp) store_word<STREAM_OUT>(dst + c * 64 + lane, quantize_word_exact(v[c], rscale));
         }
     }
     if (lane == 0) scale_h[row] = sh;
@@ -221,10 +231,17 @@ __global__ __launch_bounds__(256) void quantize_given_scale_kernel(const __half 
     reinterpret_cast<uint32_t *>(q)[idx] = quantize_word_exact(v, rscale);
 }
 
+constexpr int64_t kStreamOutBytes = int64_t(224) << 20; /* outputs larger than this bypass the caches */
+
 template <int NCH>
 int launch_reg(const __half *x, int64_t M, int64_t K, int64_t ldx, float clip, uint8_t *qact, __half *scale_h, hipStream_t s) {
     const unsigned grid = static_cast<unsigned>(ceil_div(M, kRowsPerBlock));
-    hipLaunchKernelGGL(quantize_rows_kernel<NCH>, dim3(grid), dim3(kRowsPerBlock * kWaveSize), 0, s, x, ldx, static_cast<int>(M),
+    if (M * (k_padded(K) / 2) > kStreamOutBytes) {
+        hipLaunchKernelGGL((quantize_rows_kernel<NCH, true>), dim3(grid), dim3(kRowsPerBlock * kWaveSize), 0, s, x, ldx,
+                           static_cast<int>(M), static_cast<int>(K), static_cast<int>(k_padded(K)), clip, qact, scale_h);
+        return check_launch("quantize_rows_kernel");
+    }
+    hipLaunchKernelGGL((quantize_rows_kernel<NCH, false>), dim3(grid), dim3(kRowsPerBlock * kWaveSize), 0, s, x, ldx, static_cast<int>(M),
                        static_cast<int>(K), static_cast<int>(k_padded(K)), clip, qact, scale_h);
     return check_launch("quantize_rows_kernel");
 }
