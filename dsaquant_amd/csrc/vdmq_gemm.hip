@@ -166,11 +166,14 @@ __device__ __forceinline__ void schedule_half_step() {
 // "super-tiles" of kGroupM x kGroupN tiles (32 = its CU count): the tiles that are
 // resident on an XCD together share kGroupM token row-blocks and kGroupN weight
 // row-blocks, and the 8 XCDs work on neighbouring super-tiles at any moment.
-constexpr int kXcds = 8, kGroupM = 8, kGroupN = 4;
+#ifndef VDMQ_GROUP_M
+#define VDMQ_GROUP_M 8
+#define VDMQ_GROUP_N 4
+#endif
+constexpr int kXcds = 8, kGroupM = VDMQ_GROUP_M, kGroupN = VDMQ_GROUP_N;
 
 struct TileMap {
     int tiles_m, tiles_n, super_n, total_super;
-    int stream_out; /* non-temporal output stores */
 };
 
 __device__ __forceinline__ bool map_tile(const TileMap &tm, int bid, int &tile_m, int &tile_n) {
@@ -179,18 +182,27 @@ __device__ __forceinline__ bool map_tile(const TileMap &tm, int bid, int &tile_m
     const int st = (slot / per) * kXcds + xcd;
     const int j = slot % per;
     if (st >= tm.total_super) return false;
+#ifdef VDMQ_ORDER_M_FIRST
+    // consecutive super-tiles run down the token axis: an XCD keeps its weight super-column in L2
+    const int super_m = tm.total_super / tm.super_n;
+    tile_m = (st % super_m) * kGroupM + j / kGroupN;
+    tile_n = (st / super_m) * kGroupN + j % kGroupN;
+#else
     tile_m = (st / tm.super_n) * kGroupM + j / kGroupN;
     tile_n = (st % tm.super_n) * kGroupN + j % kGroupN;
+#endif
     return tile_m < tm.tiles_m && tile_n < tm.tiles_n;
 }
 
-template <typename Cfg, bool ACC_OUT>
+// OUT_MODE: 0 = scaled output, 1 = scaled output with non-temporal stores, 2 = raw int32 accumulators
+template <typename Cfg, int OUT_MODE>
 __global__ __launch_bounds__(Cfg::kThreads, Cfg::kOccupancy * Cfg::kWaves / 4) void gemm_w4a4_kernel(const uint8_t *__restrict__ A, const uint8_t *__restrict__ W,
                                                                   const __half *__restrict__ ascale, const __half *__restrict__ wscale,
                                                                   const __half *__restrict__ bias, void *__restrict__ out, int out_dtype,
                                                                   int32_t *__restrict__ acc_out, int M, int N, int ldk, int64_t ldo,
                                                                   TileMap tmap) {
     constexpr int BM = Cfg::BM, BN = Cfg::BN, S = Cfg::STAGES, L = Cfg::kLoads;
+    constexpr bool ACC_OUT = OUT_MODE == 2, STREAM_OUT = OUT_MODE == 1;
     extern __shared__ __attribute__((aligned(1024))) uint8_t lds[];
 
     int tile_m, tile_n;
@@ -360,7 +372,7 @@ __global__ __launch_bounds__(Cfg::kThreads, Cfg::kOccupancy * Cfg::kWaves / 4) v
                     // A large output is not re-read before it falls out of the caches anyway:
                     // streaming it keeps the operands (and the next quantizer's writes) in
                     // the Infinity Cache (measured: next quantizer 5.76 -> 6.01 TB/s).
-                    if (tmap.stream_out)
+                    if (STREAM_OUT)
                         __builtin_nontemporal_store(hv, dst);
                     else
                         *dst = hv;
@@ -422,29 +434,32 @@ int launch_cfg(const uint8_t *qact, const __half *ascale, const uint8_t *wq, con
     const int super_m = static_cast<int>(ceil_div(tm.tiles_m, kGroupM));
     tm.super_n = static_cast<int>(ceil_div(tm.tiles_n, kGroupN));
     tm.total_super = super_m * tm.super_n;
-    tm.stream_out = (M * N * 2 > (int64_t(224) << 20)) ? 1 : 0;
     const int rounds = static_cast<int>(ceil_div(tm.total_super, kXcds));
     const dim3 grid(static_cast<unsigned>(rounds) * kXcds * kGroupM * kGroupN), block(Cfg::kThreads);
     const int ldk = static_cast<int>(k_padded(K) / 2);
 
+    // A large output is not re-read before it falls out of the caches anyway:
+    // streaming it keeps the operands (and the next quantizer's writes) in the
+    // Infinity Cache.
+#ifdef VDMQ_DBG_NOSTREAM
+    const bool stream_out = false;
+#else
+    const bool stream_out = M * N * 2 > (int64_t(224) << 20);
+#endif
+    const int which = acc_out != nullptr ? 2 : (stream_out ? 1 : 0);
+    using Kernel = void (*)(const uint8_t *, const uint8_t *, const __half *, const __half *, const __half *, void *, int, int32_t *, int,
+                            int, int, int64_t, TileMap);
+    const Kernel kernels[3] = {gemm_w4a4_kernel<Cfg, 0>, gemm_w4a4_kernel<Cfg, 1>, gemm_w4a4_kernel<Cfg, 2>};
     // LDS above 64 KiB has to be requested once per kernel
-    static bool attr_done[2] = {false, false};
-    const int which = acc_out != nullptr ? 1 : 0;
-    auto kacc = gemm_w4a4_kernel<Cfg, true>;
-    auto kout = gemm_w4a4_kernel<Cfg, false>;
+    static bool attr_done[3] = {false, false, false};
     if (!attr_done[which]) {
-        hipError_t e = hipFuncSetAttribute(which ? reinterpret_cast<const void *>(kacc) : reinterpret_cast<const void *>(kout),
-                                           hipFuncAttributeMaxDynamicSharedMemorySize, Cfg::kLdsBytes);
+        hipError_t e = hipFuncSetAttribute(reinterpret_cast<const void *>(kernels[which]), hipFuncAttributeMaxDynamicSharedMemorySize,
+                                           Cfg::kLdsBytes);
         if (e != hipSuccess) return fail(VDMQ_ELAUNCH, "hipFuncSetAttribute(%d bytes of LDS): %s", Cfg::kLdsBytes, hipGetErrorString(e));
         attr_done[which] = true;
     }
-    if (which) {
-        hipLaunchKernelGGL(kacc, grid, block, Cfg::kLdsBytes, s, qact, wq, ascale, wscale, bias, out, out_dtype, acc_out,
-                           static_cast<int>(M), static_cast<int>(N), ldk, ldo, tm);
-    } else {
-        hipLaunchKernelGGL(kout, grid, block, Cfg::kLdsBytes, s, qact, wq, ascale, wscale, bias, out, out_dtype, acc_out,
-                           static_cast<int>(M), static_cast<int>(N), ldk, ldo, tm);
-    }
+    hipLaunchKernelGGL(kernels[which], grid, block, Cfg::kLdsBytes, s, qact, wq, ascale, wscale, bias, out, out_dtype, acc_out,
+                       static_cast<int>(M), static_cast<int>(N), ldk, ldo, tm);
     return check_launch("gemm_w4a4_kernel");
 }
 
