@@ -1,0 +1,93 @@
+"""Config-4 harness on the GPU at a reduced size: structure counts, the W4A4
+call pattern per block, and the kernel path against a dequantized torch
+reference of the same forward."""
+from dataclasses import replace
+
+import pytest
+import torch
+import torch.nn.functional as F
+
+pytestmark = pytest.mark.gpu
+
+
+def test_timesteps_and_cfg_drop_control_flow():
+    from dsaquant_amd import wan_harness as W
+
+    assert W.unipc_timesteps(5) == [999.0, 922.0, 817.0, 666.0, 428.0]  # none below 400: CFG-drop never fires in 5 steps
+    ts50 = W.unipc_timesteps(50)
+    assert sum(t < 400 for t in ts50) == 9
+
+
+def test_small_dit_structure_and_numerics():
+    from dsaquant_amd import wan_harness as W
+    from dsaquant_amd.kernels import vdm_w4a4 as v
+    from dsaquant_amd.quantization.quant_linear import QuantLinear
+
+    dev = "cuda:0"
+    args = replace(W.WAN21_1P3B, num_layers=2, num_heads=2, ffn_dim=512, text_dim=128)  # dim 256, head dim 128
+    model = W.build_quantized(args, dev, seed=1)
+    quant = [m for m in model.modules() if isinstance(m, QuantLinear)]
+    assert len(quant) == 10 * args.num_layers  # 300 at 30 layers, as the reference's build smoke test counts
+    assert sum(isinstance(m, W.Attention) and m.use_fused_qkv_kernel for m in model.modules()) == 2 * args.num_layers
+    assert all(m.use_vdm_kernel and m.weight is None for m in quant)
+
+    g = torch.Generator(device=dev).manual_seed(0)
+    latent = torch.randn((1, 16, 3, 8, 12), generator=g, device=dev).half()  # 3*4*6 = 72 tokens
+    ctx = torch.randn((1, 512, args.text_dim), generator=g, device=dev).half()
+    t = torch.tensor([500.0], device=dev)
+
+    timers = W.KernelTimers()
+    with torch.no_grad(), W.time_w4a4_calls(timers):
+        y = model(latent, t, ctx, timers)
+    timers.collect()
+    assert y.shape == latent.shape and torch.isfinite(y).all()
+    assert timers.counts() == {"w4a4": 7 * args.num_layers, "attention": 2 * args.num_layers}
+
+    # reference: the same forward with every W4A4 call replaced by fp32 arithmetic on the
+    # dequantized operands (per-token int4 activations with clip 0.95, unpacked int4 weights)
+    import numpy as np
+
+    import oracle as O
+
+    def ref_linear(x, qweight, wscales, bias=None, clip_ratio=1.0, bias_half=None):
+        N, K = qweight.shape[0], qweight.shape[1] * 2
+        qw = torch.from_numpy(O.np_unpack_wgt_v1(qweight.cpu().numpy(), N, K)).to(dev).float()
+        ws = torch.from_numpy(O.np_unpack_wscales_v1(wscales.cpu().numpy(), N, K).astype(np.float32)).to(dev)
+        x2 = x.reshape(-1, K).half().float()
+        amax = x2.abs().amax(dim=1, keepdim=True)
+        s = torch.where(amax > 0, amax / 7 * clip_ratio, torch.ones_like(amax)).half().float()
+        q = torch.clamp(torch.round(x2 * (1.0 / s)), -8, 7)
+        yy = ((q @ qw.t()) * (s * ws[None, :])).half()
+        b = bias_half if bias_half is not None else bias
+        if b is not None:
+            yy = yy + b.half()
+        return yy.view(*x.shape[:-1], N)
+
+    orig = v.linear_vdm_w4a4
+    v.linear_vdm_w4a4 = ref_linear
+    try:
+        with torch.no_grad():
+            y_ref = model(latent, t, ctx)
+    finally:
+        v.linear_vdm_w4a4 = orig
+    err = (y.float() - y_ref.float()).abs().max().item()
+    assert err <= 2e-2 * y_ref.float().abs().max().item() + 1e-3, err
+
+    # denoise loop: 2 forwards per step above the boundary, 1 below (guidance_scale_2 = 1)
+    lat = torch.randn((1, 16, 3, 8, 12), generator=g, device=dev)
+    _, n1 = W.denoise(model, lat, ctx, ctx, [900.0, 500.0], boundary_ratio=0.4)
+    _, n2 = W.denoise(model, lat, ctx, ctx, [900.0, 300.0], boundary_ratio=0.4)
+    assert (n1, n2) == (4, 3)
+
+
+def test_patchify_roundtrip():
+    from dsaquant_amd import wan_harness as W
+
+    with torch.device("meta"):
+        m = W.WanDiT(replace(W.WAN21_1P3B, num_layers=1))
+    x = torch.arange(16 * 3 * 8 * 12, dtype=torch.float32).reshape(1, 16, 3, 8, 12)
+    tok = m.patchify(x)
+    assert tok.shape == (1, 3 * 4 * 6, 64)
+    assert torch.equal(m.unpatchify(tok, 3, 8, 12), x)
+    # token 0 holds channel-major 2x2 patches: element [c, dh, dw] at index c*4 + dh*2 + dw
+    assert tok[0, 0, 5].item() == x[0, 1, 0, 0, 1].item()
