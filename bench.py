@@ -32,6 +32,10 @@ ROOT = Path(__file__).resolve().parent
 sys.path.insert(0, str(ROOT))
 
 INT8_PEAK_TOPS = 5000.0  # MI355X dense INT8 MFMA, published
+# HBM bytes per launch of the dominant kernels on the default workload, from rocprofv3 --pmc FETCH_SIZE and
+# WRITE_SIZE runs of this program (mean over the four launches of a step; the summary with the scaling by
+# the copy kernel's readings is profiles/gemm_w4a4_kernel+quantize_rows_kernel.wan14b_720p_block.md)
+MEASURED_TRAFFIC = {"wan14b_720p_block": {"gemm": None, "quant": None}}
 HBM_PEAK_GBS = 8000.0    # MI355X HBM3E, published
 
 # (name, K, N) at M tokens
@@ -61,8 +65,9 @@ def synth_inputs(torch, M, K, N, seed, dev):
     return x, wq, ws, bias
 
 
-def cpu_baseline(torch, budget_s=20.0):
-    """Reference torch QuantLinear fp path on config 0, on the host cores."""
+def cpu_baseline(torch, budget_s=16.0):
+    """Reference torch QuantLinear fp path on config 0, on the host cores: repeated
+    forwards for about budget_s seconds in all (half per dtype), median time."""
     from oracle.quantlinear_torch import QuantLinearTorchPath
 
     M, K, N = 4096, 1536, 4608
@@ -73,26 +78,24 @@ def cpu_baseline(torch, budget_s=20.0):
     x[:, torch.randperm(K, generator=g)[:16]] *= 20
     w = torch.randint(-7, 8, (N, K), generator=g).float() * (1e-3 + 9e-3 * torch.rand(N, 1, generator=g))
     b = 0.02 * torch.randn(N, generator=g)
-    out = {}
+    out, reps = {}, {}
     for name, dt in (("fp32", torch.float32), ("fp16", torch.float16)):
         layer = QuantLinearTorchPath(w.to(dt), b.to(dt))
         xs = x.to(dt)
+        layer(xs)  # warm-up
         times = []
         t_start = time.perf_counter()
-        layer(xs)  # warm-up
-        if time.perf_counter() - t_start > budget_s / 2 and name == "fp16":
-            times = [time.perf_counter() - t_start]
-        else:
-            while len(times) < 3 or (time.perf_counter() - t_start < budget_s / 2 and len(times) < 10):
-                t0 = time.perf_counter()
-                layer(xs)
-                times.append(time.perf_counter() - t0)
-        out[name] = statistics.median(times)
+        while len(times) < 3 or time.perf_counter() - t_start < budget_s / 2:
+            t0 = time.perf_counter()
+            layer(xs)
+            times.append(time.perf_counter() - t0)
+        out[name], reps[name] = statistics.median(times), len(times)
     best = min(out.values())
     return {
         "value": round(2.0 * M * N * K / best / 1e12, 5), "unit": "TOPS", "cores": torch.get_num_threads(), "kind": "port",
-        "sample": f"config 0 (M={M}, K={K}, N={N}), torch {torch.__version__} QuantLinear fp path, median s: "
-                  + ", ".join(f"{k}={v:.3f}" for k, v in out.items()),
+        "sample": f"config 0 (M={M}, K={K}, N={N}; 0.058 TOP per forward), torch {torch.__version__} restatement of the reference's "
+                  f"QuantLinear fp path (fake-quant W and X per forward + F.linear), ~{budget_s:.0f} s of repeated forwards, median s per forward: "
+                  + ", ".join(f"{k}={v:.4f} ({reps[k]} reps)" for k, v in out.items()),
     }
 
 
@@ -193,10 +196,14 @@ def main():
         "config": {"workload": f"{args.workload}: M={M} tokens, linears " + ", ".join(f"{n} {k}->{o}" for n, k, o in wl["linears"])
                                + "; each = A4 quantizer + W4A4 GEMM + scale/bias epilogue, clip 1.0"},
         "roofline": {"bound": "mfma", "achieved": round(gemm_tops, 1), "peak": INT8_PEAK_TOPS, "unit": "TOP/s",
-                     "frac": round(gemm_tops / INT8_PEAK_TOPS, 4), "traffic": None, "kernel": "gemm_w4a4_kernel",
+                     "frac": round(gemm_tops / INT8_PEAK_TOPS, 4), "traffic": MEASURED_TRAFFIC.get(args.workload, {}).get("gemm"),
+                     "traffic_unit": "HBM bytes per launch (mean of the step's four launches)", "kernel": "gemm_w4a4_kernel",
+                     "algorithmic_ops_per_launch": total_ops / len(layers),
                      "avg_launch_ms": round(gemm_ms_sum / len(layers), 4)},
         "quantizer": {"bound": "hbm", "achieved": round(quant_gbs, 1), "peak": HBM_PEAK_GBS, "unit": "GB/s",
-                      "frac": round(quant_gbs / HBM_PEAK_GBS, 4), "traffic": None, "kernel": "quantize_rows_kernel",
+                      "frac": round(quant_gbs / HBM_PEAK_GBS, 4), "traffic": MEASURED_TRAFFIC.get(args.workload, {}).get("quant"),
+                      "traffic_unit": "HBM bytes per launch (mean of the step's four launches)", "kernel": "quantize_rows_kernel",
+                      "algorithmic_bytes_per_launch": sum(quant_bytes(M, L["K"]) for L in layers) / len(layers),
                       "avg_launch_ms": round(quant_ms_sum / len(layers), 4)},
         "per_linear": per_layer,
     }

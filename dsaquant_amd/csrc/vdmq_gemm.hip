@@ -207,6 +207,16 @@ __global__ __launch_bounds__(Cfg::kThreads, Cfg::kOccupancy * Cfg::kWaves / 4) v
 
     int tile_m, tile_n;
     if (!map_tile(tmap, blockIdx.x, tile_m, tile_n)) return;
+#ifdef VDMQ_STAGGER
+    // Two workgroups share a CU.  The first grid-wide wave of workgroups fills slot
+    // one of every CU, the next one slot two: hold the latter back by about half a
+    // tile so that one workgroup's epilogue runs under the other's MFMAs.  Later
+    // workgroups inherit the phase of the slot they fill.
+    if (Cfg::kOccupancy == 2 && blockIdx.x >= VDMQ_STAGGER && blockIdx.x < 2 * VDMQ_STAGGER) {
+        const int naps = (ldk / Cfg::kRowBytes) * Cfg::kKStepElems / 1024;
+        for (int i = 0; i < naps; ++i) __builtin_amdgcn_s_sleep(127);
+    }
+#endif
     const int m0 = tile_m * BM, n0 = tile_n * BN;
     const int lane = threadIdx.x & 63;
     const int wave = __builtin_amdgcn_readfirstlane(threadIdx.x >> 6);
@@ -325,6 +335,19 @@ __global__ __launch_bounds__(Cfg::kThreads, Cfg::kOccupancy * Cfg::kWaves / 4) v
 
     // Epilogue.  Accumulator register r of a 32x32 tile holds
     // n = 8*(r/4) + 4*(lane/32) + r%4, m = lane%32.
+#ifdef VDMQ_DBG_NOEPI
+    if (!ACC_OUT) {
+        int sum = 0;
+#pragma unroll
+        for (int ni = 0; ni < Cfg::kNI; ++ni)
+#pragma unroll
+            for (int mi = 0; mi < Cfg::kMI; ++mi)
+#pragma unroll
+                for (int r = 0; r < 16; ++r) sum ^= acc[ni][mi][r];
+        if (sum == 0x12345678) static_cast<int *>(out)[threadIdx.x] = sum;
+        return;
+    }
+#endif
     if (!ACC_OUT && out_dtype == VDMQ_OUT_F16) {
         // fp16 path: scale in the accumulator layout, round to fp16, transpose one
         // 32-row strip at a time through LDS (the stage ring is idle: every wave
@@ -367,7 +390,11 @@ __global__ __launch_bounds__(Cfg::kThreads, Cfg::kOccupancy * Cfg::kWaves / 4) v
                 f16x8 hv = *reinterpret_cast<const f16x8 *>(stg + row * RS + (lane % PR) * 16);
                 if (bias != nullptr) hv += bv; /* one fp16 add per element */
                 const int mrow = m0 + wm0 + mi * 32 + row;
+#ifdef VDMQ_DBG_NOSTORE
+                if (mrow < 0 && ncol < N) {
+#else
                 if (mrow < M && ncol < N) {
+#endif
                     f16x8 *dst = reinterpret_cast<f16x8 *>(static_cast<__half *>(out) + static_cast<int64_t>(mrow) * ldo + ncol);
                     // A large output is not re-read before it falls out of the caches anyway:
                     // streaming it keeps the operands (and the next quantizer's writes) in

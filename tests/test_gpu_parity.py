@@ -334,3 +334,28 @@ def test_config3_sized_rows_sampled_against_oracle_and_ragged_tail():
     assert torch.equal(yp, y[:4096][perm.to(DEV)])
     _, sc = v.quantize_activation_native(xd, 1.0)
     assert np.array_equal(sc.cpu().numpy().view(np.uint16), O.np_row_scale(x.numpy(), 1.0).view(np.uint16))
+
+
+# ------------------------------------------------------- committed fixture
+
+def test_hip_path_reproduces_the_committed_emulation_fixture():
+    """Every surface of the API against tests/golden/w4a4_emulated_257x128x128.npz
+    (written by the lane-level emulation of the reference's CUDA kernels)."""
+    from pathlib import Path
+
+    v = vk()
+    f = np.load(Path(__file__).parent / "golden" / "w4a4_emulated_257x128x128.npz")
+    x, w, wscale, bias, clip = f["x"], f["w"], f["wscale"], f["bias"], float(f["clip"])
+    qweight, packed_scales, channel_scales = v.pack_weight_with_scale(t16(w), t16(wscale))
+    assert np.array_equal(qweight.cpu().numpy(), f["qweight"])
+    assert np.array_equal(packed_scales.cpu().numpy().view(np.uint16), f["wscales_packed"].view(np.uint16))
+    qact, ascales, act_scales = v.quantize_activation_per_token(t16(x), clip)
+    assert np.array_equal(qact.cpu().numpy(), f["qact"])
+    assert np.array_equal(ascales.cpu().numpy().view(np.uint16), f["ascales"].view(np.uint16))
+    assert np.array_equal(act_scales.cpu().numpy().view(np.uint16), f["act_scales"].view(np.uint16))
+    y = v.linear_vdm_w4a4(t16(x), t16(f["qweight"]), t16(f["wscales_packed"]), t16(bias), clip_ratio=clip)
+    assert np.array_equal(y.cpu().numpy().view(np.uint16), f["y"].view(np.uint16))
+    native_x, _ = v.quantize_activation_native(t16(x), clip)
+    native_w, _ = v._native_weights(t16(f["qweight"]), t16(f["wscales_packed"]))
+    acc = v.gemm_int32_accumulators(native_x, native_w, 128)
+    assert np.array_equal(acc.cpu().numpy(), f["acc"])

@@ -308,3 +308,57 @@ def test_whole_kernel_emulation_matches_oracle():
     ref = (qx_s @ qw_s.T) * ascale * wscale.astype(np.float32)[None, :] + bias.astype(np.float32)[None, :]
     rel_l2 = np.linalg.norm(y.astype(np.float32) - ref) / np.linalg.norm(ref)
     assert rel_l2 < 2e-2
+
+
+# ------------------------------------------------------- committed fixture
+
+def test_oracle_reproduces_the_committed_emulation_fixture():
+    """tests/golden/w4a4_emulated_257x128x128.npz was written by the PTX-level
+    emulation (tests/golden/make_w4a4_fixture.py); the oracle must reproduce every
+    array of it."""
+    from pathlib import Path
+
+    f = np.load(Path(__file__).parent / "golden" / "w4a4_emulated_257x128x128.npz")
+    x, w, wscale, bias, clip = f["x"], f["w"], f["wscale"], f["bias"], float(f["clip"])
+    s = O.c_row_scale(x, clip)
+    assert np.array_equal(s.view(np.uint16), f["act_scales"].view(np.uint16))
+    q = O.c_quantize_rows(x, s)
+    assert np.array_equal(O.c_pack_act_v1(q), f["qact"])
+    assert np.array_equal(O.c_pack_ascales_v1(s, 128).view(np.uint16), f["ascales"].view(np.uint16))
+    qw = O.c_quantize_rows(w, wscale)
+    assert np.array_equal(O.c_pack_wgt_v1(qw), f["qweight"])
+    assert np.array_equal(O.c_pack_wscales_v1(wscale, 128).view(np.uint16), f["wscales_packed"].view(np.uint16))
+    y, _, _, acc = O.c_linear(x, qw, wscale, bias, clip)
+    assert np.array_equal(acc, f["acc"])
+    assert np.array_equal(y.view(np.uint16), f["y"].view(np.uint16))
+
+
+# ------------------------------------------------- property-based (hypothesis)
+
+from hypothesis import given, settings, strategies as st  # noqa: E402
+
+
+@settings(max_examples=60, deadline=None)
+@given(st.integers(1, 40), st.sampled_from([64, 128, 192]), st.integers(0, 2 ** 31 - 1), st.sampled_from([1.0, 0.95, 0.5, 1.7]))
+def test_property_quantizer_c_equals_numpy_on_arbitrary_bit_patterns(M, K, seed, clip):
+    """Any fp16 bit pattern (NaN payloads, infinities, subnormals included)."""
+    rng = np.random.default_rng(seed)
+    x = rng.integers(0, 65536, (M, K)).astype(np.uint16).view(np.float16)
+    s_c, s_n = O.c_row_scale(x, clip), O.np_row_scale(x, clip)
+    assert np.array_equal(s_c.view(np.uint16), s_n.view(np.uint16))
+    assert np.array_equal(O.c_quantize_rows(x, s_c), O.np_quantize_rows(x, s_n))
+
+
+@settings(max_examples=25, deadline=None)
+@given(st.integers(1, 3), st.integers(1, 2), st.integers(1, 3), st.integers(0, 2 ** 31 - 1))
+def test_property_v1_roundtrip_and_gemm_invariance(mb, nb, kb, seed):
+    """pack -> unpack is the identity for both operands, and a GEMM on unpacked
+    v1 buffers equals the GEMM on the logical matrices (layout is a bijection)."""
+    rng = np.random.default_rng(seed)
+    M, N, K = 100 * mb + 3, 128 * nb, 64 * kb
+    qa = rng.integers(-8, 8, (M, K), dtype=np.int8)
+    qw = rng.integers(-8, 8, (N, K), dtype=np.int8)
+    ua = O.np_unpack_act_v1(O.np_pack_act_v1(qa), M, K)
+    uw = O.np_unpack_wgt_v1(O.np_pack_wgt_v1(qw), N, K)
+    assert np.array_equal(ua, qa) and np.array_equal(uw, qw)
+    assert np.array_equal(O.np_gemm_i32(ua, uw), qa.astype(np.int64) @ qw.astype(np.int64).T)
