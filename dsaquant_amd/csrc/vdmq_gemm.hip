@@ -3,8 +3,8 @@
 //   acc[m,n] = sum_k qx[m,k] * qw[n,k]   exact int32
 //   out[m,n] = fp16(float(acc) * (float(as[m]) * float(ws[n]))) (+ bias[n] in fp16)
 //
-// Data path.  Both operands are row-major packed int4 (64 bytes = 128 k per
-// row and K step).  A workgroup owns a BM x BN output tile and walks K through
+// Data path.  Both operands are row-major packed int4; a K step takes 128 or
+// 256 k (64 or 128 bytes) of every row.  A workgroup owns a BM x BN output tile and walks K through
 // a ring of LDS stages filled by 128-bit direct-to-LDS loads
 // (global_load_lds_dwordx4: no VGPR staging, no ds_write).  A lane reads 16
 // bytes (32 nibbles) of one row from LDS and widens each 32-bit word p into two
@@ -14,16 +14,17 @@
 // Both operands are widened the same way, so k pairs up correctly whatever
 // order the MFMA consumes the bytes in, and v_mfma_i32_32x32x32_i8 accumulates
 // 256 * sum(qx*qw) exactly (|16q| <= 128, K <= 65536 keeps |acc| < 2^31).
-// The epilogue shifts the factor 256 out before converting to float.
+// The epilogue folds the factor 1/256 (a power of two, exact) into the scale.
 //
 // MFMA orientation: the A operand holds weight rows (n), the B operand token
 // rows (m), so a lane's four consecutive accumulator registers are four
 // consecutive n of one token: an 8-byte fp16 store.
 //
 // LDS layout of a stage: rows 0..BN-1 are weight rows, BN..BN+BM-1 token rows,
-// 64 bytes each; the four 16-byte pieces of row r are stored at piece index
-// p ^ ((r/4)%4), which makes the 16 lanes of a ds_read_b128 phase hit 16
-// different bank groups (measured: zero bank conflicts).
+// 64 or 128 bytes each; the 16-byte pieces of row r are stored at piece index
+// p ^ ((r/4)%4) (four pieces) or p ^ ((r/2)%8) (eight), which makes the 16
+// lanes of a ds_read_b128 phase hit 16 different bank groups (measured: zero
+// bank conflicts).
 //
 // Synchronisation: the direct-to-LDS loads are tracked by vmcnt only and the
 // stage ring is published with raw s_barrier (no fence: a workgroup fence
@@ -357,13 +358,16 @@ __global__ __launch_bounds__(Cfg::kThreads, Cfg::kOccupancy * Cfg::kWaves / 4) v
         constexpr int PR = Cfg::kPiecesPerRow, RS = Cfg::kStageRowBytes;
         uint8_t *stg = lds + wave * Cfg::kStagingBytes;
         const _Float16 *as_p = reinterpret_cast<const _Float16 *>(ascale);
-        f16x4 wsv[Cfg::kNI][4];
+        // channel scales of this wave's columns as fp32, once per tile
+        float wsf[Cfg::kNI][4][4];
 #pragma unroll
         for (int ni = 0; ni < Cfg::kNI; ++ni)
 #pragma unroll
             for (int rg = 0; rg < 4; ++rg) {
                 const int n = n0 + wn0 + ni * 32 + rg * 8 + lh * 4;
-                wsv[ni][rg] = *reinterpret_cast<const f16x4 *>(wscale + min(n, N - 4));
+                const f16x4 w4 = *reinterpret_cast<const f16x4 *>(wscale + min(n, N - 4));
+#pragma unroll
+                for (int e = 0; e < 4; ++e) wsf[ni][rg][e] = static_cast<float>(w4[e]);
             }
         const int ncol = n0 + wn0 + (lane % PR) * 8;
         f16x8 bv = {0, 0, 0, 0, 0, 0, 0, 0};
@@ -371,7 +375,11 @@ __global__ __launch_bounds__(Cfg::kThreads, Cfg::kOccupancy * Cfg::kWaves / 4) v
 #pragma unroll
         for (int mi = 0; mi < Cfg::kMI; ++mi) {
             const int m = m0 + wm0 + mi * 32 + l32;
-            const float as = static_cast<float>(as_p[min(m, M - 1)]);
+            // The accumulator holds 256*acc.  float(256*acc) = 256*float(acc) exactly (|acc| < 2^24),
+            // and scaling the token scale by 2^-8 is exact too, so
+            //   float(256*acc) * fl((as/256) * ws) == fl(float(acc) * fl(as * ws))   bit for bit
+            // (no under- or overflow: as*ws/256 >= 2^-56, |256*acc| < 2^31).
+            const float as = static_cast<float>(as_p[min(m, M - 1)]) * 0.00390625f;
 #pragma unroll
             for (int ni = 0; ni < Cfg::kNI; ++ni)
 #pragma unroll
@@ -379,7 +387,7 @@ __global__ __launch_bounds__(Cfg::kThreads, Cfg::kOccupancy * Cfg::kWaves / 4) v
                     f16x4 h;
 #pragma unroll
                     for (int e = 0; e < 4; ++e) {
-                        const float v = static_cast<float>(acc[ni][mi][rg * 4 + e] >> 8) * (as * static_cast<float>(wsv[ni][rg][e]));
+                        const float v = static_cast<float>(acc[ni][mi][rg * 4 + e]) * (as * wsf[ni][rg][e]);
                         h[e] = static_cast<_Float16>(v); /* round to nearest even */
                     }
                     *reinterpret_cast<f16x4 *>(stg + l32 * RS + (ni * 32 + rg * 8 + lh * 4) * 2) = h;
@@ -498,7 +506,17 @@ int launch_gemm(const uint8_t *qact, const __half *ascale, const uint8_t *wq, co
 #ifndef VDMQ_GEMM_CFG
 #define VDMQ_GEMM_CFG 256, 256, 2, 4, 2, 1, 256
 #endif
-    return launch_cfg<GemmCfg<VDMQ_GEMM_CFG>>(qact, ascale, wq, wscale, bias, out, out_dtype, acc_out, M, N, K, ldo, s);
+#ifndef VDMQ_GEMM_SMALL_CFG
+#define VDMQ_GEMM_SMALL_CFG 128, 128, 2, 2, 3, 2, 128
+#endif
+    // Few large tiles leave CUs idle (M = 512 text tokens: 2 x 40 tiles of 256 x 256 on 256 CUs):
+    // below two tiles per CU use 128 x 128 tiles, two workgroups per CU.
+    using Big = GemmCfg<VDMQ_GEMM_CFG>;
+    const int64_t big_tiles = ceil_div(M, Big::BM) * ceil_div(N, Big::BN);
+#ifndef VDMQ_DBG_NO_SMALL
+    if (big_tiles < 512) return launch_cfg<GemmCfg<VDMQ_GEMM_SMALL_CFG>>(qact, ascale, wq, wscale, bias, out, out_dtype, acc_out, M, N, K, ldo, s);
+#endif
+    return launch_cfg<Big>(qact, ascale, wq, wscale, bias, out, out_dtype, acc_out, M, N, K, ldo, s);
 }
 
 }  // namespace vdmq
