@@ -226,7 +226,7 @@ def np_gemm_i32(qx: np.ndarray, qw: np.ndarray) -> np.ndarray:
 def np_epilogue(acc, as_h, ws_h, bias_h=None) -> np.ndarray:
     """vdm_w4a4_kernel.cu:243-274, 557-569."""
     s = as_h.astype(np.float32)[:, None] * ws_h.astype(np.float32)[None, :]
-    with np.errstate(over="ignore"):
+    with np.errstate(over="ignore", invalid="ignore"):
         h = (acc.astype(np.float32) * s).astype(np.float16)
         if bias_h is not None:
             # exact sum of two fp16 values in float64, one rounding to fp16

@@ -304,6 +304,61 @@ def test_fused_qkv_is_bitwise_three_separate_calls():
     assert torch.equal(q2, sep[0]) and torch.equal(k2, sep[1]) and torch.equal(v2, sep[2])
 
 
+# --------------------------- large-tile configuration, strided C-ABI calls
+
+def test_large_tile_configuration_accumulators_and_linear():
+    """Shapes with enough 256 x 256 tiles to take the large-tile kernel (the
+    small shapes above run on the 128 x 128 one), ragged in M, N and K."""
+    v = vk()
+    M, N, K = 4100, 8320, 640
+    rng = np.random.default_rng(5)
+    qx = rng.integers(-8, 8, (M, K), dtype=np.int8)
+    qw = rng.integers(-8, 8, (N, K), dtype=np.int8)
+    Kp = v.k_padded(K)
+    print(f"large-tile acc M={M} N={N} K={K}", flush=True)
+    acc = v.gemm_int32_accumulators(t16(pack_native(qx, Kp)), t16(pack_native(qw, Kp)), K)
+    torch.cuda.synchronize()
+    assert np.array_equal(acc.cpu().numpy(), O.np_gemm_i32(qx, qw))
+    M, K, N = 8197, 1536, 4224
+    x, qw, ws, bias = O.synth_linear(M, K, N, seed=11)
+    x = special_rows(x)
+    print(f"large-tile linear M={M} K={K} N={N}", flush=True)
+    y = v.linear_vdm_w4a4(t16(x), t16(O.np_pack_wgt_v1(qw)), t16(O.np_pack_wscales_v1(ws, K)), t16(bias), clip_ratio=0.95)
+    torch.cuda.synchronize()
+    want = O.np_linear(x, qw, ws, bias, 0.95)[0]
+    got = y.cpu().numpy()
+    assert np.array_equal(got.view(np.uint16), want.view(np.uint16))
+
+
+def test_c_abi_with_row_strides():
+    """vdmq_linear_w4a4 called directly with an input row stride > K and an
+    output row stride > N: the columns beyond N stay untouched."""
+    from dsaquant_amd import _lib
+
+    v = vk()
+    lib = _lib.load()
+    M, K, N, ldx, ldo = 300, 320, 128, 384, 200
+    x, qw, ws, bias = O.synth_linear(M, K, N, seed=21)
+    xs = torch.full((M, ldx), 1000.0, dtype=torch.float16, device=DEV)  # the pad columns would change every row scale
+    xs[:, :K] = t16(x)
+    native_w = t16(pack_native(qw, v.k_padded(K)))
+    out = torch.full((M, ldo), -3.0, dtype=torch.float16, device=DEV)
+    wsb = int(lib.vdmq_workspace_bytes(M, K))
+    wsp = torch.empty(wsb, dtype=torch.uint8, device=DEV)
+    wsd, bd = t16(ws), t16(bias)
+    print("strided C-ABI linear", flush=True)
+    _lib.check(lib.vdmq_linear_w4a4(xs.data_ptr(), M, K, ldx, 1.0, native_w.data_ptr(), wsd.data_ptr(), bd.data_ptr(), out.data_ptr(), 0, N,
+                                    ldo, wsp.data_ptr(), wsb, torch.cuda.current_stream().cuda_stream))
+    torch.cuda.synchronize()
+    got = out.cpu().numpy()
+    want = O.np_linear(x, qw, ws, bias, 1.0)[0]
+    assert np.array_equal(got[:, :N].view(np.uint16), want.view(np.uint16))
+    assert (got[:, N:] == np.float16(-3.0)).all()
+    # a workspace one byte short is refused before anything is launched
+    assert lib.vdmq_linear_w4a4(xs.data_ptr(), M, K, ldx, 1.0, native_w.data_ptr(), wsd.data_ptr(), bd.data_ptr(), out.data_ptr(), 0, N, ldo,
+                                wsp.data_ptr(), wsb - 1, torch.cuda.current_stream().cuda_stream) == -4
+
+
 # ---------------------------------------------------- full-size properties
 
 def test_config3_sized_rows_sampled_against_oracle_and_ragged_tail():
