@@ -145,20 +145,24 @@ __device__ __forceinline__ void mma_step(v16i (&acc)[Cfg::kNI][Cfg::kMI], const 
         for (int mi = 0; mi < Cfg::kMI; ++mi) acc[ni][mi] = __builtin_amdgcn_mfma_i32_32x32x32_i8(o.a[ni], o.b[mi], acc[ni][mi], 0, 0, 0);
 }
 
-// Instruction-mix hint for one half K step (2 x kNI*kMI MFMAs): one MFMA, then
-// three widening VALU ops; the LDS reads (and, in the second half, the global
-// loads) are spread over the first MFMAs.  Without it the widening ops pile up
-// in front of the first MFMA of the region and the matrix pipe idles.
-template <typename Cfg, bool WITH_VMEM>
-__device__ __forceinline__ void schedule_half_step() {
-    constexpr int kMfma = 2 * Cfg::kNI * Cfg::kMI;
-    constexpr int kDs = Cfg::kNI + Cfg::kMI;
-#pragma unroll
-    for (int i = 0; i < kMfma; ++i) {
+// Instruction-mix hints.  A read's work is split into two scheduling regions of
+// kNI*kMI MFMAs each (closed by a full scheduling barrier, so the scheduler
+// cannot pile one region's widening ops up in the other): every MFMA is
+// followed by its share of the widening VALU ops (4.5 per MFMA for a 128 x 64
+// wave tile: 4 and 5 alternately); the LDS reads ride on the first MFMAs of the first region, the
+// direct-to-LDS loads on those of the second.
+template <typename Cfg, int NDS, int NVMEM, int I = 0>
+__device__ __forceinline__ void schedule_region() {
+    constexpr int kMfma = Cfg::kNI * Cfg::kMI;
+    constexpr int kValu = (Cfg::kNI + Cfg::kMI) * 6; /* widening ops of the region */
+    if constexpr (I < kMfma) {
         __builtin_amdgcn_sched_group_barrier(0x008, 1, 0); /* MFMA */
-        if (i < kDs) __builtin_amdgcn_sched_group_barrier(0x100, 1, 0); /* DS read */
-        if (WITH_VMEM && i >= kDs && i < kDs + Cfg::kLoads) __builtin_amdgcn_sched_group_barrier(0x020, 1, 0); /* VMEM read */
-        __builtin_amdgcn_sched_group_barrier(0x002, 3, 0); /* VALU */
+        if constexpr (I < NDS) __builtin_amdgcn_sched_group_barrier(0x100, 1, 0); /* DS read */
+        if constexpr (I < NVMEM) __builtin_amdgcn_sched_group_barrier(0x020, 1, 0); /* VMEM read */
+        __builtin_amdgcn_sched_group_barrier(0x002, kValu * (I + 1) / kMfma - kValu * I / kMfma, 0); /* VALU */
+        schedule_region<Cfg, NDS, NVMEM, I + 1>();
+    } else {
+        __builtin_amdgcn_sched_barrier(0);
     }
 }
 
@@ -315,18 +319,19 @@ __global__ __launch_bounds__(Cfg::kThreads, Cfg::kOccupancy * Cfg::kWaves / 4) v
                 // (the LDS reads come first in program order: the compiler must assume
                 // the direct-to-LDS loads may alias them and would not move reads above)
                 if (STEADY || kt + 1 < ksteps) read_frags<Cfg>(wn, xn, lds + nxt * Cfg::kStageBytes, waddr[0], xaddr[0]);
-#ifndef VDMQ_DBG_NOLOAD
-                if (STEADY) issue_stage<Cfg>(wbase + (kt + S) * RB, xbase + (kt + S) * RB, goff, lds + cur * Cfg::kStageBytes, wave);
-#endif
             }
             widen_frags<Cfg, 1>(hi, wc, xc);
             mma_step<Cfg>(acc, lo);
-            mma_step<Cfg>(acc, hi);
+            schedule_region<Cfg, Cfg::kNI + Cfg::kMI, 0>();
+#ifndef VDMQ_DBG_NOLOAD
+            if (STEADY && j + 1 == R) issue_stage<Cfg>(wbase + (kt + S) * RB, xbase + (kt + S) * RB, goff, lds + cur * Cfg::kStageBytes, wave);
+#endif
             widen_frags<Cfg, 0>(lo, wn, xn);
-            if (j + 1 < R)
-                schedule_half_step<Cfg, false>();
+            mma_step<Cfg>(acc, hi);
+            if (STEADY && j + 1 == R)
+                schedule_region<Cfg, 0, Cfg::kLoads>();
             else
-                schedule_half_step<Cfg, STEADY>();
+                schedule_region<Cfg, 0, 0>();
         }
         cur = nxt;
     };
