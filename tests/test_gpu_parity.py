@@ -306,23 +306,28 @@ def test_fused_qkv_is_bitwise_three_separate_calls():
 
 # --------------------------- large-tile configuration, strided C-ABI calls
 
-def test_large_tile_configuration_accumulators_and_linear():
-    """Shapes with enough 256 x 256 tiles to take the large-tile kernel (the
-    small shapes above run on the 128 x 128 one), ragged in M, N and K."""
+@pytest.mark.parametrize("M,N,K", [(4100, 8320, 640), (8200, 8320, 2304)])
+def test_mid_and_large_tile_configurations_accumulators(M, N, K):
+    """The library picks the tile configuration from the shape: 128 x 128 tiles for the small shapes above,
+    256 x 128 for a few hundred large tiles or short K (first case), 256 x 256 beyond (second case).
+    Both are ragged in M and N; the first also in K."""
     v = vk()
-    M, N, K = 4100, 8320, 640
     rng = np.random.default_rng(5)
     qx = rng.integers(-8, 8, (M, K), dtype=np.int8)
     qw = rng.integers(-8, 8, (N, K), dtype=np.int8)
     Kp = v.k_padded(K)
-    print(f"large-tile acc M={M} N={N} K={K}", flush=True)
+    print(f"tile-config acc M={M} N={N} K={K}", flush=True)
     acc = v.gemm_int32_accumulators(t16(pack_native(qx, Kp)), t16(pack_native(qw, Kp)), K)
     torch.cuda.synchronize()
     assert np.array_equal(acc.cpu().numpy(), O.np_gemm_i32(qx, qw))
-    M, K, N = 8197, 1536, 4224
+
+
+@pytest.mark.parametrize("M,K,N", [(8197, 1536, 4224), (8197, 2048, 8448)])
+def test_mid_and_large_tile_configurations_linear(M, K, N):
+    v = vk()
     x, qw, ws, bias = O.synth_linear(M, K, N, seed=11)
     x = special_rows(x)
-    print(f"large-tile linear M={M} K={K} N={N}", flush=True)
+    print(f"tile-config linear M={M} K={K} N={N}", flush=True)
     y = v.linear_vdm_w4a4(t16(x), t16(O.np_pack_wgt_v1(qw)), t16(O.np_pack_wscales_v1(ws, K)), t16(bias), clip_ratio=0.95)
     torch.cuda.synchronize()
     want = O.np_linear(x, qw, ws, bias, 0.95)[0]
