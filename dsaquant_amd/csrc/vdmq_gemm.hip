@@ -473,7 +473,10 @@ int launch_cfg(const uint8_t *qact, const __half *ascale, const uint8_t *wq, con
     tm.tiles_n = static_cast<int>(ceil_div(N, Cfg::BN));
     const int super_m = static_cast<int>(ceil_div(tm.tiles_m, kGroupM));
     tm.super_n = static_cast<int>(ceil_div(tm.tiles_n, kGroupN));
-    tm.total_super = super_m * tm.super_n;
+    const int64_t total_super = static_cast<int64_t>(super_m) * tm.super_n;
+    if (total_super * kGroupM * kGroupN + kXcds * kGroupM * kGroupN > (int64_t(1) << 31) - 1)
+        return fail(VDMQ_ESHAPE, "M x N = %lld x %lld needs more workgroups than one launch can hold", (long long)M, (long long)N);
+    tm.total_super = static_cast<int>(total_super);
     const int rounds = static_cast<int>(ceil_div(tm.total_super, kXcds));
     const dim3 grid(static_cast<unsigned>(rounds) * kXcds * kGroupM * kGroupN), block(Cfg::kThreads);
     const int ldk = static_cast<int>(k_padded(K) / 2);
@@ -490,13 +493,16 @@ int launch_cfg(const uint8_t *qact, const __half *ascale, const uint8_t *wq, con
     using Kernel = void (*)(const uint8_t *, const uint8_t *, const __half *, const __half *, const __half *, void *, int, int32_t *, int,
                             int, int, int64_t, TileMap);
     const Kernel kernels[3] = {gemm_w4a4_kernel<Cfg, 0>, gemm_w4a4_kernel<Cfg, 1>, gemm_w4a4_kernel<Cfg, 2>};
-    // LDS above 64 KiB has to be requested once per kernel
-    static bool attr_done[3] = {false, false, false};
-    if (!attr_done[which]) {
+    // LDS above 64 KiB has to be requested once per kernel and device
+    constexpr int kMaxDevices = 64;
+    static bool attr_done[kMaxDevices][3] = {};
+    int dev = 0;
+    if (hipGetDevice(&dev) != hipSuccess || dev < 0 || dev >= kMaxDevices) return fail(VDMQ_ELAUNCH, "no current HIP device");
+    if (!attr_done[dev][which]) {
         hipError_t e = hipFuncSetAttribute(reinterpret_cast<const void *>(kernels[which]), hipFuncAttributeMaxDynamicSharedMemorySize,
                                            Cfg::kLdsBytes);
         if (e != hipSuccess) return fail(VDMQ_ELAUNCH, "hipFuncSetAttribute(%d bytes of LDS): %s", Cfg::kLdsBytes, hipGetErrorString(e));
-        attr_done[which] = true;
+        attr_done[dev][which] = true;
     }
     hipLaunchKernelGGL(kernels[which], grid, block, Cfg::kLdsBytes, s, qact, wq, ascale, wscale, bias, out, out_dtype, acc_out,
                        static_cast<int>(M), static_cast<int>(N), ldk, ldo, tm);
