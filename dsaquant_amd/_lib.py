@@ -16,6 +16,8 @@ _LIB: Optional[ctypes.CDLL] = None
 
 VDMQ_OUT_F16 = 0
 VDMQ_OUT_BF16 = 1
+VDMQ_ACT_NONE = 0
+VDMQ_ACT_GELU_TANH = 1
 
 # name -> (restype, argtypes); every symbol include/vdmq.h declares
 _i64, _p, _f32, _int = ctypes.c_int64, ctypes.c_void_p, ctypes.c_float, ctypes.c_int
@@ -25,10 +27,13 @@ SIGNATURES = {
     "vdmq_last_error": (ctypes.c_char_p, []),
     "vdmq_k_padded": (_i64, [_i64]),
     "vdmq_quantize_act": (_int, [_p, _i64, _i64, _i64, _f32, _p, _p, _p]),
+    "vdmq_quantize_act_ex": (_int, [_p, _i64, _i64, _i64, _f32, _int, _p, _p, _p]),
+    "vdmq_gelu_tanh_f16": (_int, [_p, _p, _i64, _p]),
     "vdmq_gemm_w4a4": (_int, [_p, _p, _p, _p, _p, _p, _int, _i64, _i64, _i64, _i64, _p]),
     "vdmq_gemm_w4a4_acc": (_int, [_p, _p, _p, _i64, _i64, _i64, _p]),
     "vdmq_workspace_bytes": (_i64, [_i64, _i64]),
     "vdmq_linear_w4a4": (_int, [_p, _i64, _i64, _i64, _f32, _p, _p, _p, _p, _int, _i64, _i64, _p, _i64, _p]),
+    "vdmq_linear_w4a4_ex": (_int, [_p, _i64, _i64, _i64, _f32, _int, _p, _p, _p, _p, _int, _i64, _i64, _p, _i64, _p]),
     "vdmq_weight_v1_to_native": (_int, [_p, _p, _i64, _i64, _p]),
     "vdmq_weight_native_to_v1": (_int, [_p, _p, _i64, _i64, _p]),
     "vdmq_wscale_v1_to_plain": (_int, [_p, _p, _i64, _i64, _p]),

@@ -76,16 +76,31 @@ const char *vdmq_arch(void) { return "gfx950"; }
 const char *vdmq_last_error(void) { return g_error; }
 int64_t vdmq_k_padded(int64_t K) { return k_padded(K); }
 
-int vdmq_quantize_act(const void *x, int64_t M, int64_t K, int64_t ldx, float clip, void *qact, void *scale_h, vdmq_stream_t stream) {
+int vdmq_quantize_act_ex(const void *x, int64_t M, int64_t K, int64_t ldx, float clip, int act, void *qact, void *scale_h,
+                         vdmq_stream_t stream) {
     VDMQ_TRY(check_k(K));
     VDMQ_TRY(check_m(M));
+    if (act != VDMQ_ACT_NONE && act != VDMQ_ACT_GELU_TANH) return fail(VDMQ_EINVAL, "unknown activation %d", act);
     if (M == 0) return VDMQ_OK;
     VDMQ_TRY(check_ptr(x, "x"));
     VDMQ_TRY(check_ptr(qact, "qact"));
     VDMQ_TRY(check_ptr(scale_h, "scale_h", false));
     if (ldx < K || ldx % 8 != 0) return fail(VDMQ_ESHAPE, "ldx must be >= K and a multiple of 8 (got %lld)", (long long)ldx);
-    return launch_quantize_act(static_cast<const __half *>(x), M, K, ldx, clip, static_cast<uint8_t *>(qact),
+    return launch_quantize_act(static_cast<const __half *>(x), M, K, ldx, clip, act, static_cast<uint8_t *>(qact),
                                static_cast<__half *>(scale_h), as_stream(stream));
+}
+
+int vdmq_quantize_act(const void *x, int64_t M, int64_t K, int64_t ldx, float clip, void *qact, void *scale_h, vdmq_stream_t stream) {
+    return vdmq_quantize_act_ex(x, M, K, ldx, clip, VDMQ_ACT_NONE, qact, scale_h, stream);
+}
+
+int vdmq_gelu_tanh_f16(const void *x, void *y, int64_t n, vdmq_stream_t stream) {
+    if (n < 0 || n % 2 != 0) return fail(VDMQ_ESHAPE, "n must be a non-negative even count (got %lld)", (long long)n);
+    if (n == 0) return VDMQ_OK;
+    VDMQ_TRY(check_ptr(x, "x", false));
+    VDMQ_TRY(check_ptr(y, "y", false));
+    if ((reinterpret_cast<uintptr_t>(x) | reinterpret_cast<uintptr_t>(y)) & 3u) return fail(VDMQ_EINVAL, "x and y must be 4-byte aligned");
+    return launch_gelu_tanh(static_cast<const __half *>(x), static_cast<__half *>(y), n, as_stream(stream));
 }
 
 static int gemm_checked(const void *qact, const void *ascale, const void *wq, const void *wscale, const void *bias, void *out,
@@ -127,9 +142,9 @@ int64_t vdmq_workspace_bytes(int64_t M, int64_t K) {
     return q + (M * 2 + 255) / 256 * 256;
 }
 
-int vdmq_linear_w4a4(const void *x, int64_t M, int64_t K, int64_t ldx, float clip, const void *wq, const void *wscale,
-                     const void *bias, void *out, int out_dtype, int64_t N, int64_t ldo, void *workspace, int64_t workspace_bytes,
-                     vdmq_stream_t stream) {
+int vdmq_linear_w4a4_ex(const void *x, int64_t M, int64_t K, int64_t ldx, float clip, int act, const void *wq, const void *wscale,
+                        const void *bias, void *out, int out_dtype, int64_t N, int64_t ldo, void *workspace, int64_t workspace_bytes,
+                        vdmq_stream_t stream) {
     VDMQ_TRY(check_k(K));
     VDMQ_TRY(check_n(N));
     VDMQ_TRY(check_m(M));
@@ -140,8 +155,15 @@ int vdmq_linear_w4a4(const void *x, int64_t M, int64_t K, int64_t ldx, float cli
                     (long long)vdmq_workspace_bytes(M, K));
     uint8_t *qact = static_cast<uint8_t *>(workspace);
     void *scale = qact + (M * (k_padded(K) / 2) + 255) / 256 * 256;
-    VDMQ_TRY(vdmq_quantize_act(x, M, K, ldx, clip, qact, scale, stream));
+    VDMQ_TRY(vdmq_quantize_act_ex(x, M, K, ldx, clip, act, qact, scale, stream));
     return vdmq_gemm_w4a4(qact, scale, wq, wscale, bias, out, out_dtype, M, N, K, ldo, stream);
+}
+
+int vdmq_linear_w4a4(const void *x, int64_t M, int64_t K, int64_t ldx, float clip, const void *wq, const void *wscale,
+                     const void *bias, void *out, int out_dtype, int64_t N, int64_t ldo, void *workspace, int64_t workspace_bytes,
+                     vdmq_stream_t stream) {
+    return vdmq_linear_w4a4_ex(x, M, K, ldx, clip, VDMQ_ACT_NONE, wq, wscale, bias, out, out_dtype, N, ldo, workspace, workspace_bytes,
+                               stream);
 }
 
 int vdmq_weight_v1_to_native(const void *qweight_v1, void *wq_native, int64_t N, int64_t K, vdmq_stream_t stream) {

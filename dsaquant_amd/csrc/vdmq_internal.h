@@ -23,8 +23,9 @@ inline int64_t ceil_div(int64_t a, int64_t b) { return (a + b - 1) / b; }
 inline bool aligned16(const void *p) { return (reinterpret_cast<uintptr_t>(p) & 15u) == 0; }
 
 // kernels' host launchers (no argument checking: the extern "C" layer does it)
-int launch_quantize_act(const __half *x, int64_t M, int64_t K, int64_t ldx, float clip, uint8_t *qact, __half *scale_h,
+int launch_quantize_act(const __half *x, int64_t M, int64_t K, int64_t ldx, float clip, int act, uint8_t *qact, __half *scale_h,
                         hipStream_t stream);
+int launch_gelu_tanh(const __half *x, __half *y, int64_t n, hipStream_t stream);
 int launch_row_scale(const __half *x, int64_t rows, int64_t K, float clip, __half *scale_h, hipStream_t stream);
 int launch_quantize_given_scale(const __half *x, const __half *scale_h, int64_t rows, int64_t K, uint8_t *q, hipStream_t stream);
 int launch_gemm(const uint8_t *qact, const __half *ascale, const uint8_t *wq, const __half *wscale, const __half *bias,

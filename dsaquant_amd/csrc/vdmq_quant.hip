@@ -114,6 +114,42 @@ __device__ __forceinline__ bool scale_is_ordinary(__half s) {
     return b != 0u && b < 0x7C00u;
 }
 
+// GELU, tanh approximation, on an fp16 value: the fp32 evaluation a framework
+// applies to an fp16 tensor (the reference's FeedForward uses
+// activation_fn="gelu-approximate", dit_block.py:56), rounded once to fp16:
+//   u = sqrt(2/pi) * (x + 0.044715 * x^3),  gelu = 0.5 * x * (1 + tanh(u)).
+// 0.5 * (1 + tanh(u)) is evaluated as 1 / (1 + exp(-2u)): no cancellation in the
+// negative tail, so the fp32 result is a few ulp(fp32) from the exact value and
+// the fp16 result is the correctly rounded one except next to a rounding boundary.
+// +inf -> +inf, -inf -> NaN (= -inf * 0, as the formula gives), NaN -> NaN.
+__device__ __forceinline__ float gelu_tanh_f32(float x) {
+    // -2 * log2(e) * u = x * (c1 + c2 * x^2): the exponent of 2 in exp(-2u)
+    constexpr float kC1 = -2.8853900817779268f * 0.7978845608028654f;
+    constexpr float kC2 = kC1 * 0.044715f;
+    const float a = x * __builtin_fmaf(kC2, x * x, kC1);
+    const float e = __builtin_amdgcn_exp2f(a);
+    return x * __builtin_amdgcn_rcpf(1.0f + e);
+}
+
+__device__ __forceinline__ uint32_t gelu_tanh_pair(uint32_t w) {
+    const f16x2 h = __builtin_bit_cast(f16x2, w);
+    f16x2 r;
+    r[0] = static_cast<_Float16>(gelu_tanh_f32(static_cast<float>(h[0])));
+    r[1] = static_cast<_Float16>(gelu_tanh_f32(static_cast<float>(h[1])));
+    return __builtin_bit_cast(uint32_t, r);
+}
+
+template <int ACT>
+__device__ __forceinline__ u32x4 apply_act(u32x4 v) {
+    if (ACT == VDMQ_ACT_GELU_TANH) {
+        v.x = gelu_tanh_pair(v.x);
+        v.y = gelu_tanh_pair(v.y);
+        v.z = gelu_tanh_pair(v.z);
+        v.w = gelu_tanh_pair(v.w);
+    }
+    return v;
+}
+
 constexpr int kRowsPerBlock = 4; /* one wave per row */
 
 template <bool STREAM>
@@ -128,7 +164,10 @@ __device__ __forceinline__ void store_word(uint32_t *p, uint32_t w) {
 // cover the padded row.  STREAM_OUT: write the nibbles with non-temporal
 // stores -- measured faster once the output no longer fits the 256 MB
 // Infinity Cache (5.35 -> 5.9 TB/s at K = 13824, M = 75600), slower below.
-template <int NCH, bool STREAM_OUT>
+// ACT: an elementwise activation applied to the row (in fp32, rounded to fp16)
+// before it is quantized: the activation kernel between two linears, its write
+// and the quantizer's re-read of its output are saved.
+template <int NCH, bool STREAM_OUT, int ACT>
 __global__ __launch_bounds__(kRowsPerBlock * kWaveSize) void quantize_rows_kernel(const __half *__restrict__ x, int64_t ldx,
                                                                                   int M, int K, int Kp, float clip,
                                                                                   uint8_t *__restrict__ qact,
@@ -142,7 +181,7 @@ __global__ __launch_bounds__(kRowsPerBlock * kWaveSize) void quantize_rows_kerne
 #pragma unroll
     for (int c = 0; c < NCH; ++c) {
         const int k0 = c * 512 + lane * 8;
-        v[c] = k0 < K ? __builtin_nontemporal_load(src + c * 64 + lane) : u32x4{0u, 0u, 0u, 0u};
+        v[c] = k0 < K ? apply_act<ACT>(__builtin_nontemporal_load(src + c * 64 + lane)) : u32x4{0u, 0u, 0u, 0u};
     }
 
     uint32_t m2 = 0;
@@ -183,6 +222,7 @@ __global__ __launch_bounds__(kRowsPerBlock * kWaveSize) void quantize_rows_kerne
 }
 
 // Any K: two passes over the row (the second one is served by the caches).
+template <int ACT>
 __global__ __launch_bounds__(kRowsPerBlock * kWaveSize) void quantize_rows_anyk_kernel(const __half *__restrict__ x, int64_t ldx,
                                                                                        int M, int K, int Kp, float clip,
                                                                                        uint8_t *__restrict__ qact,
@@ -192,13 +232,13 @@ __global__ __launch_bounds__(kRowsPerBlock * kWaveSize) void quantize_rows_anyk_
     if (row >= M) return;
     const u32x4 *src = reinterpret_cast<const u32x4 *>(x + row * ldx);
     float mx = 0.0f;
-    for (int k0 = lane * 8; k0 < K; k0 += 512) mx = absmax_exact(src[k0 / 8], mx);
+    for (int k0 = lane * 8; k0 < K; k0 += 512) mx = absmax_exact(apply_act<ACT>(src[k0 / 8]), mx);
     mx = wave_max(mx);
     const __half sh = scale_from_absmax(mx, clip);
     const float rscale = 1.0f / __half2float(sh);
     uint32_t *dst = reinterpret_cast<uint32_t *>(qact + row * (Kp / 2));
     for (int k0 = lane * 8; k0 < Kp; k0 += 512) {
-        u32x4 v = k0 < K ? src[k0 / 8] : u32x4{0u, 0u, 0u, 0u};
+        u32x4 v = k0 < K ? apply_act<ACT>(src[k0 / 8]) : u32x4{0u, 0u, 0u, 0u};
         dst[k0 / 8] = quantize_word_exact(v, rscale);
     }
     if (lane == 0) scale_h[row] = sh;
@@ -233,27 +273,25 @@ __global__ __launch_bounds__(256) void quantize_given_scale_kernel(const __half 
 
 constexpr int64_t kStreamOutBytes = int64_t(224) << 20; /* outputs larger than this bypass the caches */
 
-template <int NCH>
+template <int NCH, int ACT>
 int launch_reg(const __half *x, int64_t M, int64_t K, int64_t ldx, float clip, uint8_t *qact, __half *scale_h, hipStream_t s) {
     const unsigned grid = static_cast<unsigned>(ceil_div(M, kRowsPerBlock));
     if (M * (k_padded(K) / 2) > kStreamOutBytes) {
-        hipLaunchKernelGGL((quantize_rows_kernel<NCH, true>), dim3(grid), dim3(kRowsPerBlock * kWaveSize), 0, s, x, ldx,
+        hipLaunchKernelGGL((quantize_rows_kernel<NCH, true, ACT>), dim3(grid), dim3(kRowsPerBlock * kWaveSize), 0, s, x, ldx,
                            static_cast<int>(M), static_cast<int>(K), static_cast<int>(k_padded(K)), clip, qact, scale_h);
         return check_launch("quantize_rows_kernel");
     }
-    hipLaunchKernelGGL((quantize_rows_kernel<NCH, false>), dim3(grid), dim3(kRowsPerBlock * kWaveSize), 0, s, x, ldx, static_cast<int>(M),
-                       static_cast<int>(K), static_cast<int>(k_padded(K)), clip, qact, scale_h);
+    hipLaunchKernelGGL((quantize_rows_kernel<NCH, false, ACT>), dim3(grid), dim3(kRowsPerBlock * kWaveSize), 0, s, x, ldx,
+                       static_cast<int>(M), static_cast<int>(K), static_cast<int>(k_padded(K)), clip, qact, scale_h);
     return check_launch("quantize_rows_kernel");
 }
 
-}  // namespace
-
-int launch_quantize_act(const __half *x, int64_t M, int64_t K, int64_t ldx, float clip, uint8_t *qact, __half *scale_h,
-                        hipStream_t s) {
-    if (M == 0) return VDMQ_OK;
+template <int ACT>
+int launch_quantize_act_impl(const __half *x, int64_t M, int64_t K, int64_t ldx, float clip, uint8_t *qact, __half *scale_h,
+                             hipStream_t s) {
     const int64_t nch = ceil_div(k_padded(K), 512);
 #define VDMQ_CASE(n) \
-    if (nch <= n) return launch_reg<n>(x, M, K, ldx, clip, qact, scale_h, s)
+    if (nch <= n) return launch_reg<n, ACT>(x, M, K, ldx, clip, qact, scale_h, s)
     VDMQ_CASE(1);
     VDMQ_CASE(2);
     VDMQ_CASE(3);
@@ -271,9 +309,31 @@ int launch_quantize_act(const __half *x, int64_t M, int64_t K, int64_t ldx, floa
     VDMQ_CASE(32);
 #undef VDMQ_CASE
     const unsigned grid = static_cast<unsigned>(ceil_div(M, kRowsPerBlock));
-    hipLaunchKernelGGL(quantize_rows_anyk_kernel, dim3(grid), dim3(kRowsPerBlock * kWaveSize), 0, s, x, ldx, static_cast<int>(M),
+    hipLaunchKernelGGL(quantize_rows_anyk_kernel<ACT>, dim3(grid), dim3(kRowsPerBlock * kWaveSize), 0, s, x, ldx, static_cast<int>(M),
                        static_cast<int>(K), static_cast<int>(k_padded(K)), clip, qact, scale_h);
     return check_launch("quantize_rows_anyk_kernel");
+}
+
+__global__ __launch_bounds__(256) void gelu_tanh_kernel(const uint32_t *__restrict__ x, uint32_t *__restrict__ y, int64_t pairs) {
+    const int64_t i = static_cast<int64_t>(blockIdx.x) * blockDim.x + threadIdx.x;
+    if (i < pairs) y[i] = gelu_tanh_pair(x[i]);
+}
+
+}  // namespace
+
+int launch_quantize_act(const __half *x, int64_t M, int64_t K, int64_t ldx, float clip, int act, uint8_t *qact, __half *scale_h,
+                        hipStream_t s) {
+    if (M == 0) return VDMQ_OK;
+    if (act == VDMQ_ACT_GELU_TANH) return launch_quantize_act_impl<VDMQ_ACT_GELU_TANH>(x, M, K, ldx, clip, qact, scale_h, s);
+    return launch_quantize_act_impl<VDMQ_ACT_NONE>(x, M, K, ldx, clip, qact, scale_h, s);
+}
+
+int launch_gelu_tanh(const __half *x, __half *y, int64_t n, hipStream_t s) {
+    const int64_t pairs = n / 2;
+    if (pairs == 0) return VDMQ_OK;
+    hipLaunchKernelGGL(gelu_tanh_kernel, dim3(static_cast<unsigned>(ceil_div(pairs, 256))), dim3(256), 0, s,
+                       reinterpret_cast<const uint32_t *>(x), reinterpret_cast<uint32_t *>(y), pairs);
+    return check_launch("gelu_tanh_kernel");
 }
 
 int launch_row_scale(const __half *x, int64_t rows, int64_t K, float clip, __half *scale_h, hipStream_t s) {

@@ -188,8 +188,17 @@ def quantize_weight_per_channel(weight: torch.Tensor):
     return pack_weight_with_scale(weight_h, scales)
 
 
+_ACTIVATIONS = {None: _lib.VDMQ_ACT_NONE, "none": _lib.VDMQ_ACT_NONE, "gelu_tanh": _lib.VDMQ_ACT_GELU_TANH}
+
+
+def _act_code(act: Optional[str]) -> int:
+    if act not in _ACTIVATIONS:
+        raise ValueError(f"unknown activation {act!r}; expected one of {sorted(k for k in _ACTIVATIONS if k)}")
+    return _ACTIVATIONS[act]
+
+
 def _linear_2d(x_2d: torch.Tensor, native_w: torch.Tensor, wscale: torch.Tensor, bias: Optional[torch.Tensor], clip_ratio: float,
-               out_dtype: torch.dtype = torch.float16) -> torch.Tensor:
+               out_dtype: torch.dtype = torch.float16, act: Optional[str] = None) -> torch.Tensor:
     lib = _load_ext()
     M, K = x_2d.shape
     N = native_w.shape[0]
@@ -205,8 +214,8 @@ def _linear_2d(x_2d: torch.Tensor, native_w: torch.Tensor, wscale: torch.Tensor,
             return out
         ws_bytes = int(lib.vdmq_workspace_bytes(M, K))
         workspace = torch.empty((ws_bytes,), dtype=torch.uint8, device=dev)
-        _lib.check(lib.vdmq_linear_w4a4(
-            x_2d.data_ptr(), M, K, x_2d.stride(0), float(clip_ratio), native_w.data_ptr(), wscale.data_ptr(),
+        _lib.check(lib.vdmq_linear_w4a4_ex(
+            x_2d.data_ptr(), M, K, x_2d.stride(0), float(clip_ratio), _act_code(act), native_w.data_ptr(), wscale.data_ptr(),
             None if bias is None else bias.data_ptr(), out.data_ptr(),
             _lib.VDMQ_OUT_F16 if out_dtype == torch.float16 else _lib.VDMQ_OUT_BF16, N, out.stride(0), workspace.data_ptr(),
             ws_bytes, _stream(dev)))
@@ -259,8 +268,9 @@ def quantize_activation_per_token(x: torch.Tensor, clip_ratio: float = 1.0):
     return qact, ascales, act_scales
 
 
-def quantize_activation_native(x: torch.Tensor, clip_ratio: float = 1.0):
-    """The quantizer's own output: ``(qact u8 [M, Kp/2] row-major, scales fp16 [M])``."""
+def quantize_activation_native(x: torch.Tensor, clip_ratio: float = 1.0, act: Optional[str] = None):
+    """The quantizer's own output: ``(qact u8 [M, Kp/2] row-major, scales fp16 [M])``.
+    ``act="gelu_tanh"`` quantizes ``gelu_tanh(x)`` instead of ``x`` in the same pass."""
     lib = _load_ext()
     x_2d, _ = _as_2d_half_contiguous(x)
     _check_device_tensor(x_2d, "input", torch.float16)
@@ -270,8 +280,8 @@ def quantize_activation_native(x: torch.Tensor, clip_ratio: float = 1.0):
     with torch.cuda.device(dev):
         native = torch.empty((M, k_padded(K) // 2), dtype=torch.uint8, device=dev)
         act_scales = torch.empty((M,), dtype=torch.float16, device=dev)
-        _lib.check(lib.vdmq_quantize_act(x_2d.data_ptr(), M, K, x_2d.stride(0), float(clip_ratio), native.data_ptr(),
-                                         act_scales.data_ptr(), _stream(dev)))
+        _lib.check(lib.vdmq_quantize_act_ex(x_2d.data_ptr(), M, K, x_2d.stride(0), float(clip_ratio), _act_code(act),
+                                            native.data_ptr(), act_scales.data_ptr(), _stream(dev)))
     return native, act_scales
 
 

@@ -130,8 +130,16 @@ class FeedForward(nn.Module):
         super().__init__()
         self.up, self.down = nn.Linear(dim, ffn_dim), nn.Linear(ffn_dim, dim)
 
+    fuse_gelu = False  # evaluate the GELU inside the second linear's activation quantizer
+
     def forward(self, x: torch.Tensor) -> torch.Tensor:
-        return self.down(F.gelu(self.up(x), approximate="tanh"))
+        down = self.down
+        if self.fuse_gelu and getattr(down, "use_vdm_kernel", False):
+            from . import fused_ops
+
+            return fused_ops.linear_gelu_vdm_w4a4(self.up(x), down.vdm_weight_packed, down.vdm_weight_scale_packed, down.bias,
+                                                  down.kernel_clip_ratio, bias_half=down._bias_half)
+        return down(F.gelu(self.up(x), approximate="tanh"))
 
 
 class Block(nn.Module):
@@ -317,23 +325,29 @@ class time_w4a4_calls:
         self.timers = timers
 
     def __enter__(self):
+        from . import fused_ops
         from .kernels import vdm_w4a4 as k
 
-        self._k, self._orig = k, k.linear_vdm_w4a4
-        timers, orig = self.timers, self._orig
+        timers = self.timers
 
-        def timed(*a, **kw):
-            timers.start("w4a4")
-            try:
-                return orig(*a, **kw)
-            finally:
-                timers.stop("w4a4")
+        def wrap(orig):
+            def timed(*a, **kw):
+                timers.start("w4a4")
+                try:
+                    return orig(*a, **kw)
+                finally:
+                    timers.stop("w4a4")
 
-        k.linear_vdm_w4a4 = timed
+            return timed
+
+        self._saved = [(k, "linear_vdm_w4a4", k.linear_vdm_w4a4), (fused_ops, "linear_gelu_vdm_w4a4", fused_ops.linear_gelu_vdm_w4a4)]
+        for mod, name, orig in self._saved:
+            setattr(mod, name, wrap(orig))
         return self
 
     def __exit__(self, *exc):
-        self._k.linear_vdm_w4a4 = self._orig
+        for mod, name, orig in self._saved:
+            setattr(mod, name, orig)
         return False
 
 

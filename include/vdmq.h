@@ -42,6 +42,10 @@ extern "C" {
 #define VDMQ_OUT_F16 0
 #define VDMQ_OUT_BF16 1
 
+/* elementwise activation applied to the input of a quantizer */
+#define VDMQ_ACT_NONE 0
+#define VDMQ_ACT_GELU_TANH 1
+
 /* Shape constants of the v1 layout (vdm_w4a4_kernel.cu:15-24, vdm_w4a4.py:23-25). */
 #define VDMQ_BLOCK_M 256
 #define VDMQ_BLOCK_N 128
@@ -66,6 +70,24 @@ int64_t vdmq_k_padded(int64_t K);
  * Preconditions: K % 64 == 0, M >= 0. */
 int vdmq_quantize_act(const void *x, int64_t M, int64_t K, int64_t ldx, float clip, void *qact, void *scale_h,
                       vdmq_stream_t stream);
+
+/* The same quantizer with the preceding elementwise activation fused in:
+ * row m is act(x[m, :]) evaluated in fp32 and rounded once to fp16, then
+ * quantized as above.  VDMQ_ACT_GELU_TANH is the FeedForward activation
+ * between the two FFN linears (activation_fn="gelu-approximate",
+ * vdm_infer/models/wan_vdm/modules/dit_block.py:56):
+ *   gelu(x) = 0.5 * x * (1 + tanh(sqrt(2/pi) * (x + 0.044715 * x^3))).
+ * Fusing it removes the activation kernel, its [M, K] fp16 write and the
+ * quantizer's re-read (the reference runs them separately: FeedForward ->
+ * QuantLinear.forward, quant_linear.py:162-172).  The fp16 activation values
+ * are those vdmq_gelu_tanh_f16 returns; given them, qact and scale_h are
+ * exactly vdmq_quantize_act's. */
+int vdmq_quantize_act_ex(const void *x, int64_t M, int64_t K, int64_t ldx, float clip, int act, void *qact, void *scale_h,
+                         vdmq_stream_t stream);
+
+/* y[i] = fp16_rn(gelu_tanh(float(x[i]))) for n fp16 values (n even, 4-byte
+ * aligned pointers): the activation of vdmq_quantize_act_ex on its own. */
+int vdmq_gelu_tanh_f16(const void *x, void *y, int64_t n, vdmq_stream_t stream);
 
 /* W4A4 GEMM with fused epilogue.  Replaces linear_w4a4_kernel
  * (vdm_w4a4_kernel.cu:627-686, launched at :819 and :907):
@@ -94,6 +116,12 @@ int64_t vdmq_workspace_bytes(int64_t M, int64_t K);
 int vdmq_linear_w4a4(const void *x, int64_t M, int64_t K, int64_t ldx, float clip, const void *wq, const void *wscale,
                      const void *bias, void *out, int out_dtype, int64_t N, int64_t ldo, void *workspace,
                      int64_t workspace_bytes, vdmq_stream_t stream);
+
+/* vdmq_linear_w4a4 with an activation fused into the quantizer (see
+ * vdmq_quantize_act_ex): out = linear(act(x)). */
+int vdmq_linear_w4a4_ex(const void *x, int64_t M, int64_t K, int64_t ldx, float clip, int act, const void *wq, const void *wscale,
+                        const void *bias, void *out, int out_dtype, int64_t N, int64_t ldo, void *workspace,
+                        int64_t workspace_bytes, vdmq_stream_t stream);
 
 /* One-time relayouts between the checkpoint's v1 buffers and native ones.
  * v1 weight layout: weight_quantize_per_channel_kernel + pack_wscales

@@ -195,6 +195,27 @@ def c_linear(x, qw, ws_h, bias_h=None, clip: float = 1.0):
 
 # ------------------------------------------------------------- numpy forms
 
+def np_gelu_tanh_f64(x) -> np.ndarray:
+    """GELU, tanh approximation, in float64.  The reference's FFN is diffusers'
+    FeedForward(activation_fn="gelu-approximate") (dit_block.py:56), i.e. torch's
+    GELU(approximate="tanh"), whose published definition is
+        0.5 * x * (1 + tanh(sqrt(2/pi) * (x + 0.044715 * x^3))).
+    0.5 * (1 + tanh(u)) is written as 1 / (1 + exp(-2u)) (the same function, without
+    the cancellation of 1 + tanh(u) for very negative u)."""
+    x = np.asarray(x, dtype=np.float64)
+    with np.errstate(over="ignore", invalid="ignore"):
+        u = np.sqrt(2.0 / np.pi) * (x + 0.044715 * x * x * x)
+        return x / (1.0 + np.exp(-2.0 * u))
+
+
+def np_gelu_tanh_f16(x_h: np.ndarray) -> np.ndarray:
+    """The correctly rounded fp16 GELU of fp16 inputs: what a framework's fp32
+    evaluation on an fp16 tensor approximates (one rounding to fp16)."""
+    assert x_h.dtype == np.float16
+    with np.errstate(over="ignore", invalid="ignore"):
+        return np_gelu_tanh_f64(x_h).astype(np.float16)
+
+
 def np_row_scale(x: np.ndarray, clip: float = 1.0) -> np.ndarray:
     """vdm_w4a4_kernel.cu:459-481 -- fp32 absmax ignoring NaN, /7, *clip, fp16."""
     a = np.abs(x.astype(np.float32))

@@ -73,6 +73,19 @@ def test_small_dit_structure_and_numerics():
     err = (y.float() - y_ref.float()).abs().max().item()
     assert err <= 2e-2 * y_ref.float().abs().max().item() + 1e-3, err
 
+    # GELU evaluated inside the FFN-down quantizer: same call count, same result up to the few fp16 ulp by which
+    # torch's GELU kernel and the fused one differ on isolated values
+    timers2 = W.KernelTimers()
+    W.FeedForward.fuse_gelu = True
+    try:
+        with torch.no_grad(), W.time_w4a4_calls(timers2):
+            y_fused = model(latent, t, ctx, timers2)
+    finally:
+        W.FeedForward.fuse_gelu = False
+    timers2.collect()
+    assert timers2.counts() == {"w4a4": 7 * args.num_layers, "attention": 2 * args.num_layers}
+    assert (y_fused.float() - y.float()).abs().max().item() <= 1e-2 * y.float().abs().max().item() + 1e-3
+
     # denoise loop: 2 forwards per step above the boundary, 1 below (guidance_scale_2 = 1)
     lat = torch.randn((1, 16, 3, 8, 12), generator=g, device=dev)
     _, n1 = W.denoise(model, lat, ctx, ctx, [900.0, 500.0], boundary_ratio=0.4)

@@ -304,6 +304,72 @@ def test_fused_qkv_is_bitwise_three_separate_calls():
     assert torch.equal(q2, sep[0]) and torch.equal(k2, sep[1]) and torch.equal(v2, sep[2])
 
 
+# ------------------------------------------------- GELU fused into the quantizer
+
+def gpu_gelu_table():
+    """fp16 -> fp16 GELU of the library for all 65 536 bit patterns."""
+    from dsaquant_amd import fused_ops
+
+    allh = np.arange(65536, dtype=np.uint16).view(np.float16)
+    return allh, fused_ops.gelu_tanh(t16(allh)).cpu().numpy()
+
+
+def test_gelu_table_within_one_ulp_of_the_correctly_rounded_value():
+    """Floating-point part of the fused path, tolerance stated here: for every fp16 input the library's GELU is
+    within 1 fp16 ulp of the correctly rounded float64 value (and equal to it for more than 99.5 % of them);
+    NaN exactly where the formula gives NaN (NaN inputs and -inf)."""
+    allh, got = gpu_gelu_table()
+    want = O.np_gelu_tanh_f16(allh)
+    assert np.array_equal(np.isnan(got), np.isnan(want))
+    ok = ~np.isnan(want)
+    assert np.array_equal(np.isinf(got[ok]), np.isinf(want[ok]))
+    fin = ok & ~np.isinf(want)
+    # ordered-integer distance; +0 and -0 count as equal
+    def key(h):
+        b = h.view(np.int16).astype(np.int32)
+        return np.where(b < 0, -(b & 0x7FFF), b)
+    ulp = np.abs(key(got[fin]) - key(want[fin]))
+    print("gelu table: max ulp", ulp.max(), "inexact", int((ulp != 0).sum()), flush=True)
+    assert ulp.max() <= 1
+    assert (ulp != 0).mean() < 0.005
+
+
+@pytest.mark.parametrize("M,K", [(515, 5120), (130, 13824), (257, 1536), (19, 16384 + 64)])
+def test_fused_gelu_quantizer_is_the_quantizer_of_the_gelu_values(M, K):
+    """Integer part, bit-exact: quantize(act='gelu_tanh')(x) == oracle quantizer applied to the library's own fp16
+    GELU values of x (looked up in its 65 536-entry table), scales included."""
+    v = vk()
+    _, table = gpu_gelu_table()
+    x = special_rows((3.0 * O.synth_linear(M, K, 128, seed=M + K)[0].astype(np.float32)).astype(np.float16))
+    print(f"fused gelu quantizer M={M} K={K}", flush=True)
+    for clip in (1.0, 0.95):
+        qn, sc = v.quantize_activation_native(t16(x), clip, act="gelu_tanh")
+        torch.cuda.synchronize()
+        g = table[x.view(np.uint16)]
+        want_s = O.np_row_scale(g, clip)
+        assert np.array_equal(sc.cpu().numpy().view(np.uint16), want_s.view(np.uint16))
+        assert np.array_equal(unpack_native(qn.cpu().numpy(), K), O.np_quantize_rows(g, want_s))
+
+
+def test_linear_gelu_equals_unfused_chain_and_oracle():
+    from dsaquant_amd import fused_ops
+
+    v = vk()
+    M, K, N = 1237, 8960, 1536
+    x, qw, ws, bias = O.synth_linear(M, K, N, seed=4)
+    x = (2.0 * x.astype(np.float32)).astype(np.float16)
+    qv1, sv1, b = t16(O.np_pack_wgt_v1(qw)), t16(O.np_pack_wscales_v1(ws, K)), t16(bias)
+    y = fused_ops.linear_gelu_vdm_w4a4(t16(x).reshape(1, M, K), qv1, sv1, b, clip_ratio=1.0)
+    assert tuple(y.shape) == (1, M, N) and y.dtype == torch.float16
+    y2 = v.linear_vdm_w4a4(fused_ops.gelu_tanh(t16(x)), qv1, sv1, b, clip_ratio=1.0)  # three kernels
+    assert torch.equal(y[0], y2)
+    _, table = gpu_gelu_table()
+    want = O.np_linear(table[x.view(np.uint16)], qw, ws, bias, 1.0)[0]
+    assert np.array_equal(y[0].cpu().numpy().view(np.uint16), want.view(np.uint16))
+    with pytest.raises(ValueError):
+        v.quantize_activation_native(t16(x), 1.0, act="relu")
+
+
 # --------------------------- large-tile configuration, strided C-ABI calls
 
 @pytest.mark.parametrize("M,N,K", [(4100, 8320, 640), (8200, 8320, 2304)])

@@ -362,3 +362,28 @@ def test_property_v1_roundtrip_and_gemm_invariance(mb, nb, kb, seed):
     uw = O.np_unpack_wgt_v1(O.np_pack_wgt_v1(qw), N, K)
     assert np.array_equal(ua, qa) and np.array_equal(uw, qw)
     assert np.array_equal(O.np_gemm_i32(ua, uw), qa.astype(np.int64) @ qw.astype(np.int64).T)
+
+
+# ----------------------------------------------------------- fused GELU oracle
+
+def test_gelu_oracle_is_pinned_by_torch_float64_and_by_its_identities():
+    """np_gelu_tanh_f16 on all 65 536 fp16 patterns: equal to torch's own GELU(approximate="tanh") evaluated in
+    float64 and rounded once (a library routine, not a retyped formula); gelu(x) - gelu(-x) = x; special values.
+    torch's fp32 evaluation of an fp16 tensor (what the reference runs) is itself only within 3 fp16 ulp of it."""
+    import torch
+
+    allh = np.arange(65536, dtype=np.uint16).view(np.float16)
+    g = O.np_gelu_tanh_f16(allh)
+    t64 = torch.nn.functional.gelu(torch.from_numpy(allh.astype(np.float64)), approximate="tanh").numpy().astype(np.float16)
+    both_nan = np.isnan(g) & np.isnan(t64)
+    assert np.array_equal(g.view(np.uint16)[~both_nan], t64.view(np.uint16)[~both_nan])
+    assert np.array_equal(np.isnan(g), np.isnan(t64))
+    x = allh[np.isfinite(allh)].astype(np.float64)
+    assert np.abs(O.np_gelu_tanh_f64(x) - O.np_gelu_tanh_f64(-x) - x).max() < 1e-11
+    sp = O.np_gelu_tanh_f16(np.array([np.inf, -np.inf, 0.0, 65504.0, -65504.0, 1.0], dtype=np.float16))
+    assert sp[0] == np.inf and np.isnan(sp[1]) and sp[2] == 0 and sp[3] == np.float16(65504.0) and sp[4] == 0
+    assert sp[5] == np.float16(0.8411919906082768)  # 0.5 * (1 + tanh(sqrt(2/pi) * 1.044715)), worked by hand
+    t32 = torch.nn.functional.gelu(torch.from_numpy(allh.astype(np.float32)), approximate="tanh").numpy().astype(np.float16)
+    ok = ~(np.isnan(g) | np.isnan(t32))
+    ulp = np.abs(g.view(np.int16).astype(np.int32)[ok] - t32.view(np.int16).astype(np.int32)[ok])
+    assert ulp.max() <= 3
