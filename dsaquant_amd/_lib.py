@@ -18,6 +18,8 @@ VDMQ_OUT_F16 = 0
 VDMQ_OUT_BF16 = 1
 VDMQ_ACT_NONE = 0
 VDMQ_ACT_GELU_TANH = 1
+VDMQ_LN_MODULATE = 1
+VDMQ_LN_AFFINE = 2
 
 # name -> (restype, argtypes); every symbol include/vdmq.h declares
 _i64, _p, _f32, _int = ctypes.c_int64, ctypes.c_void_p, ctypes.c_float, ctypes.c_int
@@ -28,6 +30,9 @@ SIGNATURES = {
     "vdmq_k_padded": (_i64, [_i64]),
     "vdmq_quantize_act": (_int, [_p, _i64, _i64, _i64, _f32, _p, _p, _p]),
     "vdmq_quantize_act_ex": (_int, [_p, _i64, _i64, _i64, _f32, _int, _p, _p, _p]),
+    "vdmq_quantize_act_ln": (_int, [_p, _i64, _i64, _i64, _f32, _int, _p, _p, _i64, _i64, _f32, _p, _p, _p]),
+    "vdmq_ln_f16": (_int, [_p, _i64, _i64, _i64, _f32, _int, _p, _p, _i64, _i64, _p, _i64, _p]),
+    "vdmq_linear_ln_w4a4": (_int, [_p, _i64, _i64, _i64, _f32, _int, _p, _p, _i64, _i64, _f32, _p, _p, _p, _p, _int, _i64, _i64, _p, _i64, _p]),
     "vdmq_gelu_tanh_f16": (_int, [_p, _p, _i64, _p]),
     "vdmq_gemm_w4a4": (_int, [_p, _p, _p, _p, _p, _p, _int, _i64, _i64, _i64, _i64, _p]),
     "vdmq_gemm_w4a4_acc": (_int, [_p, _p, _p, _i64, _i64, _i64, _p]),

@@ -103,6 +103,44 @@ int vdmq_gelu_tanh_f16(const void *x, void *y, int64_t n, vdmq_stream_t stream) 
     return launch_gelu_tanh(static_cast<const __half *>(x), static_cast<__half *>(y), n, as_stream(stream));
 }
 
+static int ln_checked(const void *x, int64_t M, int64_t K, int64_t ldx, int ln_mode, const void *a, const void *b, int64_t ldv,
+                      int64_t rows_per_vec) {
+    VDMQ_TRY(check_k(K));
+    VDMQ_TRY(check_m(M));
+    if (K > 16384) return fail(VDMQ_ESHAPE, "the fused LayerNorm needs K <= 16384 (got %lld)", (long long)K);
+    if (ln_mode != VDMQ_LN_MODULATE && ln_mode != VDMQ_LN_AFFINE) return fail(VDMQ_EINVAL, "unknown ln_mode %d", ln_mode);
+    if (rows_per_vec <= 0) return fail(VDMQ_ESHAPE, "rows_per_vec must be positive (got %lld)", (long long)rows_per_vec);
+    if (ldv < K || ldv % 8 != 0) return fail(VDMQ_ESHAPE, "ldv must be >= K and a multiple of 8 (got %lld)", (long long)ldv);
+    if (ldx < K || ldx % 8 != 0) return fail(VDMQ_ESHAPE, "ldx must be >= K and a multiple of 8 (got %lld)", (long long)ldx);
+    if (M == 0) return VDMQ_OK;
+    VDMQ_TRY(check_ptr(x, "x"));
+    VDMQ_TRY(check_ptr(a, "a"));
+    VDMQ_TRY(check_ptr(b, "b"));
+    return VDMQ_OK;
+}
+
+int vdmq_quantize_act_ln(const void *x, int64_t M, int64_t K, int64_t ldx, float eps, int ln_mode, const void *a, const void *b,
+                         int64_t ldv, int64_t rows_per_vec, float clip, void *qact, void *scale_h, vdmq_stream_t stream) {
+    VDMQ_TRY(ln_checked(x, M, K, ldx, ln_mode, a, b, ldv, rows_per_vec));
+    if (M == 0) return VDMQ_OK;
+    VDMQ_TRY(check_ptr(qact, "qact"));
+    VDMQ_TRY(check_ptr(scale_h, "scale_h", false));
+    return launch_ln_quantize(static_cast<const __half *>(x), M, K, ldx, eps, ln_mode, static_cast<const __half *>(a),
+                              static_cast<const __half *>(b), ldv, rows_per_vec, clip, static_cast<uint8_t *>(qact),
+                              static_cast<__half *>(scale_h), nullptr, 0, as_stream(stream));
+}
+
+int vdmq_ln_f16(const void *x, int64_t M, int64_t K, int64_t ldx, float eps, int ln_mode, const void *a, const void *b, int64_t ldv,
+                int64_t rows_per_vec, void *h, int64_t ldh, vdmq_stream_t stream) {
+    VDMQ_TRY(ln_checked(x, M, K, ldx, ln_mode, a, b, ldv, rows_per_vec));
+    if (M == 0) return VDMQ_OK;
+    VDMQ_TRY(check_ptr(h, "h"));
+    if (ldh < K || ldh % 8 != 0) return fail(VDMQ_ESHAPE, "ldh must be >= K and a multiple of 8 (got %lld)", (long long)ldh);
+    return launch_ln_quantize(static_cast<const __half *>(x), M, K, ldx, eps, ln_mode, static_cast<const __half *>(a),
+                              static_cast<const __half *>(b), ldv, rows_per_vec, 1.0f, nullptr, nullptr, static_cast<__half *>(h), ldh,
+                              as_stream(stream));
+}
+
 static int gemm_checked(const void *qact, const void *ascale, const void *wq, const void *wscale, const void *bias, void *out,
                         int out_dtype, int32_t *acc, int64_t M, int64_t N, int64_t K, int64_t ldo, vdmq_stream_t stream) {
     VDMQ_TRY(check_k(K));
@@ -156,6 +194,23 @@ int vdmq_linear_w4a4_ex(const void *x, int64_t M, int64_t K, int64_t ldx, float 
     uint8_t *qact = static_cast<uint8_t *>(workspace);
     void *scale = qact + (M * (k_padded(K) / 2) + 255) / 256 * 256;
     VDMQ_TRY(vdmq_quantize_act_ex(x, M, K, ldx, clip, act, qact, scale, stream));
+    return vdmq_gemm_w4a4(qact, scale, wq, wscale, bias, out, out_dtype, M, N, K, ldo, stream);
+}
+
+int vdmq_linear_ln_w4a4(const void *x, int64_t M, int64_t K, int64_t ldx, float eps, int ln_mode, const void *a, const void *b,
+                        int64_t ldv, int64_t rows_per_vec, float clip, const void *wq, const void *wscale, const void *bias, void *out,
+                        int out_dtype, int64_t N, int64_t ldo, void *workspace, int64_t workspace_bytes, vdmq_stream_t stream) {
+    VDMQ_TRY(check_k(K));
+    VDMQ_TRY(check_n(N));
+    VDMQ_TRY(check_m(M));
+    if (M == 0) return VDMQ_OK;
+    VDMQ_TRY(check_ptr(workspace, "workspace"));
+    if (workspace_bytes < vdmq_workspace_bytes(M, K))
+        return fail(VDMQ_ENOSPACE, "workspace has %lld bytes, %lld needed", (long long)workspace_bytes,
+                    (long long)vdmq_workspace_bytes(M, K));
+    uint8_t *qact = static_cast<uint8_t *>(workspace);
+    void *scale = qact + (M * (k_padded(K) / 2) + 255) / 256 * 256;
+    VDMQ_TRY(vdmq_quantize_act_ln(x, M, K, ldx, eps, ln_mode, a, b, ldv, rows_per_vec, clip, qact, scale, stream));
     return vdmq_gemm_w4a4(qact, scale, wq, wscale, bias, out, out_dtype, M, N, K, ldo, stream);
 }
 

@@ -26,6 +26,10 @@ inline bool aligned16(const void *p) { return (reinterpret_cast<uintptr_t>(p) & 
 int launch_quantize_act(const __half *x, int64_t M, int64_t K, int64_t ldx, float clip, int act, uint8_t *qact, __half *scale_h,
                         hipStream_t stream);
 int launch_gelu_tanh(const __half *x, __half *y, int64_t n, hipStream_t stream);
+// h_out == nullptr: quantize into qact/scale_h; otherwise write the normalised fp16 rows to h_out
+int launch_ln_quantize(const __half *x, int64_t M, int64_t K, int64_t ldx, float eps, int ln_mode, const __half *va, const __half *vb,
+                       int64_t ldv, int64_t rows_per_vec, float clip, uint8_t *qact, __half *scale_h, __half *h_out, int64_t ldh,
+                       hipStream_t stream);
 int launch_row_scale(const __half *x, int64_t rows, int64_t K, float clip, __half *scale_h, hipStream_t stream);
 int launch_quantize_given_scale(const __half *x, const __half *scale_h, int64_t rows, int64_t K, uint8_t *q, hipStream_t stream);
 int launch_gemm(const uint8_t *qact, const __half *ascale, const uint8_t *wq, const __half *wscale, const __half *bias,

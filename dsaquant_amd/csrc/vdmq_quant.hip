@@ -160,30 +160,11 @@ __device__ __forceinline__ void store_word(uint32_t *p, uint32_t w) {
         *p = w;
 }
 
-// NCH = number of 512-element chunks (one 128-bit load per lane each) that
-// cover the padded row.  STREAM_OUT: write the nibbles with non-temporal
-// stores -- measured faster once the output no longer fits the 256 MB
-// Infinity Cache (5.35 -> 5.9 TB/s at K = 13824, M = 75600), slower below.
-// ACT: an elementwise activation applied to the row (in fp32, rounded to fp16)
-// before it is quantized: the activation kernel between two linears, its write
-// and the quantizer's re-read of its output are saved.
-template <int NCH, bool STREAM_OUT, int ACT>
-__global__ __launch_bounds__(kRowsPerBlock * kWaveSize) void quantize_rows_kernel(const __half *__restrict__ x, int64_t ldx,
-                                                                                  int M, int K, int Kp, float clip,
-                                                                                  uint8_t *__restrict__ qact,
-                                                                                  __half *__restrict__ scale_h) {
-    const int lane = threadIdx.x & (kWaveSize - 1);
-    const int64_t row = static_cast<int64_t>(blockIdx.x) * kRowsPerBlock + (threadIdx.x >> 6);
-    if (row >= M) return;
-    const u32x4 *src = reinterpret_cast<const u32x4 *>(x + row * ldx);
-
-    u32x4 v[NCH];
-#pragma unroll
-    for (int c = 0; c < NCH; ++c) {
-        const int k0 = c * 512 + lane * 8;
-        v[c] = k0 < K ? apply_act<ACT>(__builtin_nontemporal_load(src + c * 64 + lane)) : u32x4{0u, 0u, 0u, 0u};
-    }
-
+// Quantize a row held in registers (v[c] = elements 512c + 8*lane ... +7, zero
+// beyond K): absmax, fp16 scale, nibbles, stores.
+template <int NCH, bool STREAM_OUT>
+__device__ __forceinline__ void quantize_held_row(const u32x4 (&v)[NCH], int lane, int64_t row, int Kp, float clip,
+                                                  uint8_t *__restrict__ qact, __half *__restrict__ scale_h) {
     uint32_t m2 = 0;
 #pragma unroll
     for (int c = 0; c < NCH; ++c) m2 = absmax_bits(v[c], m2);
@@ -219,6 +200,131 @@ __global__ __launch_bounds__(kRowsPerBlock * kWaveSize) void quantize_rows_kerne
         }
     }
     if (lane == 0) scale_h[row] = sh;
+}
+
+// NCH = number of 512-element chunks (one 128-bit load per lane each) that
+// cover the padded row.  STREAM_OUT: write the nibbles with non-temporal
+// stores -- measured faster once the output no longer fits the 256 MB
+// Infinity Cache (5.35 -> 5.9 TB/s at K = 13824, M = 75600), slower below.
+// ACT: an elementwise activation applied to the row (in fp32, rounded to fp16)
+// before it is quantized: the activation kernel between two linears, its write
+// and the quantizer's re-read of its output are saved.
+template <int NCH, bool STREAM_OUT, int ACT>
+__global__ __launch_bounds__(kRowsPerBlock * kWaveSize) void quantize_rows_kernel(const __half *__restrict__ x, int64_t ldx,
+                                                                                  int M, int K, int Kp, float clip,
+                                                                                  uint8_t *__restrict__ qact,
+                                                                                  __half *__restrict__ scale_h) {
+    const int lane = threadIdx.x & (kWaveSize - 1);
+    const int64_t row = static_cast<int64_t>(blockIdx.x) * kRowsPerBlock + (threadIdx.x >> 6);
+    if (row >= M) return;
+    const u32x4 *src = reinterpret_cast<const u32x4 *>(x + row * ldx);
+
+    u32x4 v[NCH];
+#pragma unroll
+    for (int c = 0; c < NCH; ++c) {
+        const int k0 = c * 512 + lane * 8;
+        v[c] = k0 < K ? apply_act<ACT>(__builtin_nontemporal_load(src + c * 64 + lane)) : u32x4{0u, 0u, 0u, 0u};
+    }
+
+    quantize_held_row<NCH, STREAM_OUT>(v, lane, row, Kp, clip, qact, scale_h);
+}
+
+__device__ __forceinline__ float wave_sum(float v) {
+#pragma unroll
+    for (int off = 32; off > 0; off >>= 1) v += __shfl_xor(v, off, 64);
+    return v;
+}
+
+// LayerNorm over the row (fp32 statistics, no affine) followed by the block's
+// modulation, fused in front of the quantizer -- the producer of the attn1 and
+// FFN-up inputs (dit_block.py:100, :110 of the reference):
+//   VDMQ_LN_MODULATE  h = (fp16(LN(x)) * (1 + a)) + b   with a = scale, b = shift, every
+//                     operation a correctly rounded fp16 operation, as the reference's
+//                     fp16 tensor arithmetic after FP32LayerNorm's cast back to fp16
+//   VDMQ_LN_AFFINE    h = fp16(LN(x) * a + b)           with a = weight, b = bias, in
+//                     fp32 with one rounding (FP32LayerNorm with elementwise_affine, norm2)
+// Row m takes vector row m / rows_per_vec of a and b (stride ldv elements): one
+// vector per batch element, or one per token.  EMIT_H writes h itself instead of
+// quantizing it (the same arithmetic: the checker's view of h).
+template <int NCH, int LNMODE, bool EMIT_H>
+__global__ __launch_bounds__(kRowsPerBlock * kWaveSize) void ln_quantize_rows_kernel(
+    const __half *__restrict__ x, int64_t ldx, int M, int K, int Kp, float eps, const __half *__restrict__ va,
+    const __half *__restrict__ vb, int64_t ldv, int rows_per_vec, float clip, uint8_t *__restrict__ qact,
+    __half *__restrict__ scale_h, __half *__restrict__ h_out, int64_t ldh) {
+    const int lane = threadIdx.x & (kWaveSize - 1);
+    const int64_t row = static_cast<int64_t>(blockIdx.x) * kRowsPerBlock + (threadIdx.x >> 6);
+    if (row >= M) return;
+    const u32x4 *src = reinterpret_cast<const u32x4 *>(x + row * ldx);
+    const int64_t vrow = (row / rows_per_vec) * ldv;
+    const u32x4 *pa = reinterpret_cast<const u32x4 *>(va + vrow), *pb = reinterpret_cast<const u32x4 *>(vb + vrow);
+
+    u32x4 v[NCH];
+    float sum = 0.0f;
+#pragma unroll
+    for (int c = 0; c < NCH; ++c) {
+        const int k0 = c * 512 + lane * 8;
+        v[c] = k0 < K ? __builtin_nontemporal_load(src + c * 64 + lane) : u32x4{0u, 0u, 0u, 0u};
+        const uint32_t w[4] = {v[c].x, v[c].y, v[c].z, v[c].w};
+#pragma unroll
+        for (int i = 0; i < 4; ++i) {
+            const f16x2 h = __builtin_bit_cast(f16x2, w[i]);
+            sum += static_cast<float>(h[0]) + static_cast<float>(h[1]); /* padding adds zeros */
+        }
+    }
+    const float mean = wave_sum(sum) / static_cast<float>(K);
+    float sq = 0.0f;
+#pragma unroll
+    for (int c = 0; c < NCH; ++c) {
+        const int k0 = c * 512 + lane * 8;
+        if (k0 < K) {
+            const uint32_t w[4] = {v[c].x, v[c].y, v[c].z, v[c].w};
+#pragma unroll
+            for (int i = 0; i < 4; ++i) {
+                const f16x2 h = __builtin_bit_cast(f16x2, w[i]);
+                const float d0 = static_cast<float>(h[0]) - mean, d1 = static_cast<float>(h[1]) - mean;
+                sq += d0 * d0 + d1 * d1;
+            }
+        }
+    }
+    const float rstd = 1.0f / __builtin_sqrtf(wave_sum(sq) / static_cast<float>(K) + eps);
+
+#pragma unroll
+    for (int c = 0; c < NCH; ++c) {
+        const int k0 = c * 512 + lane * 8;
+        if (k0 < K) {
+            const u32x4 a4 = pa[c * 64 + lane], b4 = pb[c * 64 + lane];
+            const uint32_t w[4] = {v[c].x, v[c].y, v[c].z, v[c].w};
+            const uint32_t aw[4] = {a4.x, a4.y, a4.z, a4.w}, bw[4] = {b4.x, b4.y, b4.z, b4.w};
+            uint32_t o[4];
+#pragma unroll
+            for (int i = 0; i < 4; ++i) {
+                const f16x2 h = __builtin_bit_cast(f16x2, w[i]);
+                const f16x2 a = __builtin_bit_cast(f16x2, aw[i]), b = __builtin_bit_cast(f16x2, bw[i]);
+                const float n0 = (static_cast<float>(h[0]) - mean) * rstd, n1 = (static_cast<float>(h[1]) - mean) * rstd;
+                f16x2 r;
+                if (LNMODE == VDMQ_LN_MODULATE) {
+                    const f16x2 ln = {static_cast<_Float16>(n0), static_cast<_Float16>(n1)};
+                    const f16x2 one = {static_cast<_Float16>(1.0f), static_cast<_Float16>(1.0f)};
+                    r = ln * (one + a) + b; /* three packed fp16 operations, each rounded (no contraction) */
+                } else {
+                    r[0] = static_cast<_Float16>(n0 * static_cast<float>(a[0]) + static_cast<float>(b[0]));
+                    r[1] = static_cast<_Float16>(n1 * static_cast<float>(a[1]) + static_cast<float>(b[1]));
+                }
+                o[i] = __builtin_bit_cast(uint32_t, r);
+            }
+            v[c] = u32x4{o[0], o[1], o[2], o[3]};
+        }
+    }
+    if (EMIT_H) {
+        u32x4 *dst = reinterpret_cast<u32x4 *>(h_out + row * ldh);
+#pragma unroll
+        for (int c = 0; c < NCH; ++c) {
+            const int k0 = c * 512 + lane * 8;
+            if (k0 < K) dst[c * 64 + lane] = v[c];
+        }
+        return;
+    }
+    quantize_held_row<NCH, false>(v, lane, row, Kp, clip, qact, scale_h);
 }
 
 // Any K: two passes over the row (the second one is served by the caches).
@@ -314,6 +420,41 @@ int launch_quantize_act_impl(const __half *x, int64_t M, int64_t K, int64_t ldx,
     return check_launch("quantize_rows_anyk_kernel");
 }
 
+template <int NCH, int LNMODE>
+int launch_ln_reg(const __half *x, int64_t M, int64_t K, int64_t ldx, float eps, const __half *va, const __half *vb, int64_t ldv,
+                  int64_t rows_per_vec, float clip, uint8_t *qact, __half *scale_h, __half *h_out, int64_t ldh, hipStream_t s) {
+    const dim3 grid(static_cast<unsigned>(ceil_div(M, kRowsPerBlock))), block(kRowsPerBlock * kWaveSize);
+    if (h_out != nullptr)
+        hipLaunchKernelGGL((ln_quantize_rows_kernel<NCH, LNMODE, true>), grid, block, 0, s, x, ldx, static_cast<int>(M), static_cast<int>(K),
+                           static_cast<int>(k_padded(K)), eps, va, vb, ldv, static_cast<int>(rows_per_vec), clip, qact, scale_h, h_out, ldh);
+    else
+        hipLaunchKernelGGL((ln_quantize_rows_kernel<NCH, LNMODE, false>), grid, block, 0, s, x, ldx, static_cast<int>(M), static_cast<int>(K),
+                           static_cast<int>(k_padded(K)), eps, va, vb, ldv, static_cast<int>(rows_per_vec), clip, qact, scale_h, h_out, ldh);
+    return check_launch("ln_quantize_rows_kernel");
+}
+
+template <int LNMODE>
+int launch_ln_impl(const __half *x, int64_t M, int64_t K, int64_t ldx, float eps, const __half *va, const __half *vb, int64_t ldv,
+                   int64_t rows_per_vec, float clip, uint8_t *qact, __half *scale_h, __half *h_out, int64_t ldh, hipStream_t s) {
+    const int64_t nch = ceil_div(k_padded(K), 512);
+#define VDMQ_CASE(n) \
+    if (nch <= n) return launch_ln_reg<n, LNMODE>(x, M, K, ldx, eps, va, vb, ldv, rows_per_vec, clip, qact, scale_h, h_out, ldh, s)
+    VDMQ_CASE(1);
+    VDMQ_CASE(2);
+    VDMQ_CASE(3);
+    VDMQ_CASE(4);
+    VDMQ_CASE(6);
+    VDMQ_CASE(8);
+    VDMQ_CASE(10);
+    VDMQ_CASE(12);
+    VDMQ_CASE(16);
+    VDMQ_CASE(20);
+    VDMQ_CASE(24);
+    VDMQ_CASE(32);
+#undef VDMQ_CASE
+    return fail(VDMQ_ESHAPE, "the fused LayerNorm needs K <= 16384 (got %lld)", (long long)K);
+}
+
 __global__ __launch_bounds__(256) void gelu_tanh_kernel(const uint32_t *__restrict__ x, uint32_t *__restrict__ y, int64_t pairs) {
     const int64_t i = static_cast<int64_t>(blockIdx.x) * blockDim.x + threadIdx.x;
     if (i < pairs) y[i] = gelu_tanh_pair(x[i]);
@@ -326,6 +467,15 @@ int launch_quantize_act(const __half *x, int64_t M, int64_t K, int64_t ldx, floa
     if (M == 0) return VDMQ_OK;
     if (act == VDMQ_ACT_GELU_TANH) return launch_quantize_act_impl<VDMQ_ACT_GELU_TANH>(x, M, K, ldx, clip, qact, scale_h, s);
     return launch_quantize_act_impl<VDMQ_ACT_NONE>(x, M, K, ldx, clip, qact, scale_h, s);
+}
+
+int launch_ln_quantize(const __half *x, int64_t M, int64_t K, int64_t ldx, float eps, int ln_mode, const __half *va, const __half *vb,
+                       int64_t ldv, int64_t rows_per_vec, float clip, uint8_t *qact, __half *scale_h, __half *h_out, int64_t ldh,
+                       hipStream_t s) {
+    if (M == 0) return VDMQ_OK;
+    if (ln_mode == VDMQ_LN_MODULATE)
+        return launch_ln_impl<VDMQ_LN_MODULATE>(x, M, K, ldx, eps, va, vb, ldv, rows_per_vec, clip, qact, scale_h, h_out, ldh, s);
+    return launch_ln_impl<VDMQ_LN_AFFINE>(x, M, K, ldx, eps, va, vb, ldv, rows_per_vec, clip, qact, scale_h, h_out, ldh, s);
 }
 
 int launch_gelu_tanh(const __half *x, __half *y, int64_t n, hipStream_t s) {

@@ -9,6 +9,11 @@ the first (FeedForward with activation_fn="gelu-approximate",
 vdm_infer/models/wan_vdm/modules/dit_block.py:56 of the reference).  The GELU is
 evaluated inside the activation quantizer, so the GELU kernel, its [M, ffn]
 fp16 write and the quantizer's re-read of it disappear.
+
+``LnInput`` + ``linear_ln_vdm_w4a4`` / ``qkv_projections_ln`` do the same for
+the block's ``norm(x) * (1 + scale) + shift`` (dit_block.py:100, :110) and for
+the affine ``norm2`` (:105): the LayerNorm, the modulation and the quantizer
+become one pass over ``x``.
 """
 from __future__ import annotations
 
@@ -57,3 +62,114 @@ def linear_gelu_vdm_w4a4(
         b = b.half().contiguous().view(-1)
     out = _k._linear_2d(x_2d, native_w, wscale, b, clip_ratio, act="gelu_tanh")
     return out.view(*orig_shape, -1)
+
+
+class LnInput:
+    """A linear's input that is still to be produced: ``LayerNorm(x)`` followed by
+    the modulation ``* (1 + a) + b`` (``mode="modulate"``, a = scale, b = shift,
+    fp16 arithmetic on the fp16 LayerNorm output) or by the affine ``* a + b``
+    (``mode="affine"``, a = weight, b = bias, fp32 arithmetic, one rounding).
+
+    ``x`` is ``[B, L, K]`` (or ``[L, K]``); ``a`` and ``b`` hold one vector per batch
+    element (``[B, K]``, ``[B, 1, K]`` or ``[K]``) or one per token (``[B, L, K]``).
+    """
+
+    def __init__(self, x: torch.Tensor, a: torch.Tensor, b: torch.Tensor, eps: float, mode: str = "modulate"):
+        if mode not in ("modulate", "affine"):
+            raise ValueError(f"unknown LayerNorm mode {mode!r}")
+        self.shape = tuple(x.shape)
+        K = x.shape[-1]
+        self.x = x.reshape(-1, K).half().contiguous()
+        M = self.x.shape[0]
+        a2, b2 = a.reshape(-1, K).half().contiguous(), b.reshape(-1, K).half().contiguous()
+        if a2.shape != b2.shape:
+            raise ValueError("the two LayerNorm vectors must have the same shape")
+        nvec = a2.shape[0]
+        if nvec == 0 or M % nvec != 0:
+            raise ValueError(f"{nvec} vectors do not divide {M} rows")
+        self.a, self.b, self.rows_per_vec = a2, b2, M // nvec
+        self.eps, self.mode = float(eps), mode
+        self.code = _lib.VDMQ_LN_MODULATE if mode == "modulate" else _lib.VDMQ_LN_AFFINE
+
+    def _args(self):
+        M, K = self.x.shape
+        return (self.x.data_ptr(), M, K, self.x.stride(0), self.eps, self.code, self.a.data_ptr(), self.b.data_ptr(), self.a.stride(0),
+                self.rows_per_vec)
+
+    def materialize(self) -> torch.Tensor:
+        """The fp16 tensor the fused quantizer sees (same kernel arithmetic), shaped like ``x``."""
+        lib = _k._load_ext()
+        _k._check_device_tensor(self.x, "input", torch.float16)
+        h = torch.empty_like(self.x)
+        if h.numel():
+            with torch.cuda.device(h.device):
+                _lib.check(lib.vdmq_ln_f16(*self._args(), h.data_ptr(), h.stride(0), _k._stream(h.device)))
+        return h.view(self.shape)
+
+    def quantize(self, clip_ratio: float = 1.0):
+        """``(qact native, scales)`` of the produced input, as ``quantize_activation_native`` returns them."""
+        lib = _k._load_ext()
+        _k._check_device_tensor(self.x, "input", torch.float16)
+        M, K = self.x.shape
+        dev = self.x.device
+        with torch.cuda.device(dev):
+            native = torch.empty((M, _k.k_padded(K) // 2), dtype=torch.uint8, device=dev)
+            scales = torch.empty((M,), dtype=torch.float16, device=dev)
+            if M:
+                _lib.check(lib.vdmq_quantize_act_ln(*self._args(), float(clip_ratio), native.data_ptr(), scales.data_ptr(), _k._stream(dev)))
+        return native, scales
+
+
+def linear_ln_vdm_w4a4(
+    pre: LnInput,
+    qweight: torch.Tensor,
+    wscales: torch.Tensor,
+    bias: Optional[torch.Tensor] = None,
+    clip_ratio: float = 1.0,
+    bias_half: Optional[torch.Tensor] = None,
+) -> torch.Tensor:
+    """``linear_vdm_w4a4(pre.materialize(), ...)`` without materializing: LayerNorm,
+    modulation and activation quantizer are one kernel, the GEMM the second."""
+    lib = _k._load_ext()
+    x_2d = pre.x
+    _k._check_linear_shapes(x_2d, qweight, wscales)
+    _k._require(x_2d.is_cuda, "input must be a CUDA tensor")
+    native_w, wscale = _k._native_weights(qweight.contiguous(), wscales.contiguous())
+    b = bias_half if bias_half is not None else bias
+    if b is not None:
+        b = b.half().contiguous().view(-1)
+        _k._check_device_tensor(b, "bias", torch.float16)
+        _k._require(b.numel() == native_w.shape[0], "bias length must equal N")
+    M, K = x_2d.shape
+    N = native_w.shape[0]
+    dev = x_2d.device
+    with torch.cuda.device(dev):
+        out = torch.empty((M, N), dtype=torch.float16, device=dev)
+        if M:
+            ws_bytes = int(lib.vdmq_workspace_bytes(M, K))
+            workspace = torch.empty((ws_bytes,), dtype=torch.uint8, device=dev)
+            _lib.check(lib.vdmq_linear_ln_w4a4(*pre._args(), float(clip_ratio), native_w.data_ptr(), wscale.data_ptr(),
+                                               None if b is None else b.data_ptr(), out.data_ptr(), _lib.VDMQ_OUT_F16, N, out.stride(0),
+                                               workspace.data_ptr(), ws_bytes, _k._stream(dev)))
+    return out.view(*pre.shape[:-1], N)
+
+
+def qkv_projections_ln(attn, pre: LnInput):
+    """Self-attention Q, K, V of ``pre`` through the cached concatenation Wq|Wk|Wv
+    (the fused branch of ``get_qkv_projections``, attention.py:41-68 of the
+    reference) with the LayerNorm fused into the one activation quantization."""
+    from .fused_qkv import _cat_cached
+
+    w, s, b = _cat_cached(attn, ["to_q", "to_k", "to_v"], "qkv")
+    out = linear_ln_vdm_w4a4(pre, w, s, None, attn.to_q.kernel_clip_ratio, bias_half=b)
+    n = attn.to_q.vdm_weight_packed.shape[0]
+    return out.split(n, dim=-1)
+
+
+def kv_projections(attn, encoder_hidden_states: torch.Tensor):
+    """Cross-attention K, V through the cached concatenation Wk|Wv (attention.py:70-107 of the reference)."""
+    from .fused_qkv import _cat_cached
+
+    w, s, b = _cat_cached(attn, ["to_k", "to_v"], "kv")
+    kv = _k.linear_vdm_w4a4(encoder_hidden_states, w, s, bias=None, clip_ratio=attn.to_k.kernel_clip_ratio, bias_half=b)
+    return kv.split(attn.to_k.vdm_weight_packed.shape[0], dim=-1)

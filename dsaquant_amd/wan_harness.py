@@ -112,7 +112,18 @@ class Attention(nn.Module):
         self.qkv_kernel_backend = None
 
     def forward(self, x: torch.Tensor, context: Optional[torch.Tensor], freqs: Optional[torch.Tensor], timers=None) -> torch.Tensor:
-        q, k, v = get_qkv_projections(self, x, context)
+        from . import fused_ops
+
+        if isinstance(x, fused_ops.LnInput):  # the LayerNorm in front of this module runs inside the quantizer
+            if context is None:
+                q, k, v = fused_ops.qkv_projections_ln(self, x)
+            else:
+                tq = self.to_q
+                q = fused_ops.linear_ln_vdm_w4a4(x, tq.vdm_weight_packed, tq.vdm_weight_scale_packed, tq.bias, tq.kernel_clip_ratio,
+                                                 bias_half=tq._bias_half)
+                k, v = fused_ops.kv_projections(self, context)
+        else:
+            q, k, v = get_qkv_projections(self, x, context)
         q, k = self.norm_q(q), self.norm_k(k)
         q, k, v = (t.unflatten(2, (self.heads, -1)) for t in (q, k, v))
         if freqs is not None:
@@ -133,13 +144,23 @@ class FeedForward(nn.Module):
     fuse_gelu = False  # evaluate the GELU inside the second linear's activation quantizer
 
     def forward(self, x: torch.Tensor) -> torch.Tensor:
+        from . import fused_ops
+
+        if isinstance(x, fused_ops.LnInput):
+            up = self.up
+            x = fused_ops.linear_ln_vdm_w4a4(x, up.vdm_weight_packed, up.vdm_weight_scale_packed, up.bias, up.kernel_clip_ratio,
+                                             bias_half=up._bias_half)
+            return self._second(x)
+        return self._second(self.up(x))
+
+    def _second(self, y: torch.Tensor) -> torch.Tensor:
         down = self.down
         if self.fuse_gelu and getattr(down, "use_vdm_kernel", False):
             from . import fused_ops
 
-            return fused_ops.linear_gelu_vdm_w4a4(self.up(x), down.vdm_weight_packed, down.vdm_weight_scale_packed, down.bias,
+            return fused_ops.linear_gelu_vdm_w4a4(y, down.vdm_weight_packed, down.vdm_weight_scale_packed, down.bias,
                                                   down.kernel_clip_ratio, bias_half=down._bias_half)
-        return down(F.gelu(self.up(x), approximate="tanh"))
+        return down(F.gelu(y, approximate="tanh"))
 
 
 class Block(nn.Module):
@@ -152,10 +173,18 @@ class Block(nn.Module):
         self.ffn = FeedForward(a.dim, a.ffn_dim)
         self.scale_shift_table = nn.Parameter(torch.randn(1, 6, a.dim) / a.dim ** 0.5)
 
+    fuse_ln = False  # run the three LayerNorms (+ modulation) inside the following linears' activation quantizers
+
     def forward(self, x, context, tproj, freqs, timers=None):
         # tproj: [1, 6, dim] (one timestep for the whole sequence; the reference repeats it per token)
         mod = (self.scale_shift_table.to(tproj.dtype) + tproj).unbind(dim=1)
         shift, scale, gate, c_shift, c_scale, c_gate = (m.unsqueeze(1) for m in mod)
+        if self.fuse_ln and getattr(self.ffn.up, "use_vdm_kernel", False) and self.attn1.use_fused_qkv_kernel:
+            from .fused_ops import LnInput
+
+            x = x + self.attn1(LnInput(x, scale, shift, self.eps, "modulate"), None, freqs, timers) * gate
+            x = x + self.attn2(LnInput(x, self.norm2.weight, self.norm2.bias, self.eps, "affine"), context, None, timers)
+            return x + self.ffn(LnInput(x, c_scale, c_shift, self.eps, "modulate")) * c_gate
         h = fp32_layer_norm(x, None, None, self.eps) * (1 + scale) + shift
         x = x + self.attn1(h, None, freqs, timers) * gate
         h = fp32_layer_norm(x, self.norm2.weight, self.norm2.bias, self.eps)
@@ -340,7 +369,8 @@ class time_w4a4_calls:
 
             return timed
 
-        self._saved = [(k, "linear_vdm_w4a4", k.linear_vdm_w4a4), (fused_ops, "linear_gelu_vdm_w4a4", fused_ops.linear_gelu_vdm_w4a4)]
+        self._saved = [(k, "linear_vdm_w4a4", k.linear_vdm_w4a4), (fused_ops, "linear_gelu_vdm_w4a4", fused_ops.linear_gelu_vdm_w4a4),
+                       (fused_ops, "linear_ln_vdm_w4a4", fused_ops.linear_ln_vdm_w4a4)]
         for mod, name, orig in self._saved:
             setattr(mod, name, wrap(orig))
         return self

@@ -46,6 +46,10 @@ extern "C" {
 #define VDMQ_ACT_NONE 0
 #define VDMQ_ACT_GELU_TANH 1
 
+/* what follows the LayerNorm fused in front of a quantizer */
+#define VDMQ_LN_MODULATE 1 /* fp16(LN(x)) * (1 + scale) + shift, fp16 arithmetic */
+#define VDMQ_LN_AFFINE 2   /* fp16(LN(x) * weight + bias), fp32 arithmetic */
+
 /* Shape constants of the v1 layout (vdm_w4a4_kernel.cu:15-24, vdm_w4a4.py:23-25). */
 #define VDMQ_BLOCK_M 256
 #define VDMQ_BLOCK_N 128
@@ -89,6 +93,26 @@ int vdmq_quantize_act_ex(const void *x, int64_t M, int64_t K, int64_t ldx, float
  * aligned pointers): the activation of vdmq_quantize_act_ex on its own. */
 int vdmq_gelu_tanh_f16(const void *x, void *y, int64_t n, vdmq_stream_t stream);
 
+/* The quantizer with the preceding LayerNorm (+ modulation) fused in: the
+ * producer of a Wan block's attn1 and FFN-up inputs,
+ *   norm(hidden_states) * (1 + scale) + shift
+ * (vdm_infer/models/wan_vdm/modules/dit_block.py:100, :110; norm = FP32LayerNorm
+ * without affine: statistics in fp32, result cast to fp16), or of the attn2 query
+ * input, norm2 with elementwise affine (:105).  Row m of x [M, K] is normalised
+ * over K (biased variance, eps inside the square root), then
+ *   VDMQ_LN_MODULATE: h = fp16(fp16(fp16(LN) * fp16(1 + a)) + b)   a = scale, b = shift
+ *   VDMQ_LN_AFFINE:   h = fp16(LN * a + b) in fp32                 a = weight, b = bias
+ * with a, b fp16 [*, K] (row stride ldv elements, ldv % 8 == 0, 16-byte
+ * aligned); row m uses vector row m / rows_per_vec (one vector per batch element:
+ * rows_per_vec = tokens per batch element; one per token: 1).  h is then
+ * quantized as vdmq_quantize_act does.  K <= 16384.
+ * vdmq_ln_f16 writes h itself (fp16 [M, K], row stride ldh) with the same
+ * arithmetic; given its h, qact and scale_h are exactly vdmq_quantize_act's. */
+int vdmq_quantize_act_ln(const void *x, int64_t M, int64_t K, int64_t ldx, float eps, int ln_mode, const void *a, const void *b,
+                         int64_t ldv, int64_t rows_per_vec, float clip, void *qact, void *scale_h, vdmq_stream_t stream);
+int vdmq_ln_f16(const void *x, int64_t M, int64_t K, int64_t ldx, float eps, int ln_mode, const void *a, const void *b, int64_t ldv,
+                int64_t rows_per_vec, void *h, int64_t ldh, vdmq_stream_t stream);
+
 /* W4A4 GEMM with fused epilogue.  Replaces linear_w4a4_kernel
  * (vdm_w4a4_kernel.cu:627-686, launched at :819 and :907):
  *   acc[m,n] = sum_k qact[m,k] * wq[n,k]                      (int32, exact)
@@ -122,6 +146,12 @@ int vdmq_linear_w4a4(const void *x, int64_t M, int64_t K, int64_t ldx, float cli
 int vdmq_linear_w4a4_ex(const void *x, int64_t M, int64_t K, int64_t ldx, float clip, int act, const void *wq, const void *wscale,
                         const void *bias, void *out, int out_dtype, int64_t N, int64_t ldo, void *workspace,
                         int64_t workspace_bytes, vdmq_stream_t stream);
+
+/* vdmq_linear_w4a4 with the LayerNorm (+ modulation) fused into the quantizer
+ * (see vdmq_quantize_act_ln): out = linear(h). */
+int vdmq_linear_ln_w4a4(const void *x, int64_t M, int64_t K, int64_t ldx, float eps, int ln_mode, const void *a, const void *b,
+                        int64_t ldv, int64_t rows_per_vec, float clip, const void *wq, const void *wscale, const void *bias, void *out,
+                        int out_dtype, int64_t N, int64_t ldo, void *workspace, int64_t workspace_bytes, vdmq_stream_t stream);
 
 /* One-time relayouts between the checkpoint's v1 buffers and native ones.
  * v1 weight layout: weight_quantize_per_channel_kernel + pack_wscales

@@ -216,6 +216,36 @@ def np_gelu_tanh_f16(x_h: np.ndarray) -> np.ndarray:
         return np_gelu_tanh_f64(x_h).astype(np.float16)
 
 
+def np_layer_norm_f64(x_h: np.ndarray, eps: float) -> np.ndarray:
+    """LayerNorm without affine over the last axis, float64: (x - mean) / sqrt(var + eps), biased variance
+    (FP32LayerNorm of the reference's blocks, dit_block.py:32,56: torch.nn.functional.layer_norm on x.float())."""
+    x = x_h.astype(np.float64)
+    mean = x.mean(axis=-1, keepdims=True)
+    var = ((x - mean) ** 2).mean(axis=-1, keepdims=True)
+    return (x - mean) / np.sqrt(var + eps)
+
+
+def np_ln_modulate_f16(x_h: np.ndarray, scale_h: np.ndarray, shift_h: np.ndarray, eps: float, rows_per_vec: int = 1):
+    """norm(x) * (1 + scale) + shift as the reference evaluates it on fp16 tensors (dit_block.py:100, :110): the
+    LayerNorm result is cast to fp16, then three fp16 tensor operations, each correctly rounded.  Returns
+    (h, aux) with aux = the intermediate fp16 tensors ln, s1 = 1 + scale and p = ln * s1 (an error bound for an
+    implementation whose LayerNorm is one ulp off needs their magnitudes)."""
+    ln = np_layer_norm_f64(x_h, eps).astype(np.float16)
+    a = np.repeat(scale_h.reshape(-1, x_h.shape[-1]), rows_per_vec, axis=0)
+    b = np.repeat(shift_h.reshape(-1, x_h.shape[-1]), rows_per_vec, axis=0)
+    s1 = (np.float16(1.0) + a).astype(np.float16)
+    p = (ln.astype(np.float32) * s1.astype(np.float32)).astype(np.float16)  # product of two fp16 is exact in fp32
+    h = (p.astype(np.float64) + b.astype(np.float64)).astype(np.float16)     # exact sum, one rounding
+    return h, {"ln": ln, "s1": s1, "p": p}
+
+
+def np_ln_affine_f16(x_h: np.ndarray, weight_h: np.ndarray, bias_h: np.ndarray, eps: float, rows_per_vec: int = 1) -> np.ndarray:
+    """FP32LayerNorm with elementwise affine (norm2, dit_block.py:53): LN(x) * w + b, one rounding to fp16."""
+    a = np.repeat(weight_h.reshape(-1, x_h.shape[-1]), rows_per_vec, axis=0).astype(np.float64)
+    b = np.repeat(bias_h.reshape(-1, x_h.shape[-1]), rows_per_vec, axis=0).astype(np.float64)
+    return (np_layer_norm_f64(x_h, eps) * a + b).astype(np.float16)
+
+
 def np_row_scale(x: np.ndarray, clip: float = 1.0) -> np.ndarray:
     """vdm_w4a4_kernel.cu:459-481 -- fp32 absmax ignoring NaN, /7, *clip, fp16."""
     a = np.abs(x.astype(np.float32))

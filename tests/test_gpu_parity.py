@@ -370,6 +370,89 @@ def test_linear_gelu_equals_unfused_chain_and_oracle():
         v.quantize_activation_native(t16(x), 1.0, act="relu")
 
 
+# ---------------------------------- LayerNorm + modulation fused into the quantizer
+
+def spacing16(v):
+    """fp16 ulp at magnitude v (subnormal spacing below 2^-14)."""
+    v = np.maximum(np.abs(v.astype(np.float64)), 2.0 ** -14)
+    return 2.0 ** (np.floor(np.log2(v)) - 10)
+
+
+LN_CASES = [
+    # (B, L, K, per_token)
+    (2, 300, 1536, False), (1, 515, 5120, False), (3, 77, 3072, True), (1, 33, 64, False), (1, 19, 16384, False), (2, 64, 8960, True)]
+
+
+@pytest.mark.parametrize("B,L,K,per_token", LN_CASES)
+@pytest.mark.parametrize("mode", ["modulate", "affine"])
+def test_fused_layer_norm_quantizer(B, L, K, per_token, mode):
+    """Floating-point part (tolerance stated here): the library's fp32 LayerNorm may land one fp16 ulp from the
+    oracle's (float64 statistics); carried through the reference's fp16 chain ln * (1 + scale) + shift that bounds
+    |h - oracle| by ulp(ln) * |1 + scale| + ulp(product) + ulp(h); in affine mode (fp32, one rounding) by 1 ulp(h) plus
+    2^-21 of the two terms' magnitudes (fp32 rounding where they cancel).  On more
+    than 99 % of the elements the two are equal.  Integer part, bit-exact:
+    the fused quantizer's output is the oracle quantizer's on the library's own h; the fused linear equals the
+    three-kernel chain."""
+    from dsaquant_amd import fused_ops
+
+    v = vk()
+    rng = np.random.default_rng(B * 1000 + L + K)
+    eps = 1e-6
+    x = (rng.standard_normal((B, L, K)) * 2.0 + 0.25).astype(np.float32)
+    x[..., rng.integers(0, K, max(1, K // 100))] *= 15.0
+    x = x.astype(np.float16)
+    nv = (B, L, K) if per_token else (B, 1, K)
+    a = (0.2 * rng.standard_normal(nv)).astype(np.float16)
+    b = (0.3 * rng.standard_normal(nv)).astype(np.float16)
+    if mode == "affine":
+        a = (1.0 + a.astype(np.float32)).astype(np.float16)
+    print(f"fused LN {mode} B={B} L={L} K={K} per_token={per_token}", flush=True)
+    pre = fused_ops.LnInput(t16(x), t16(a), t16(b), eps, mode)
+    h_gpu = pre.materialize().cpu().numpy()
+    rpv = 1 if per_token else L
+    x2 = x.reshape(-1, K)
+    if mode == "modulate":
+        want, aux = O.np_ln_modulate_f16(x2, a.reshape(-1, K), b.reshape(-1, K), eps, rpv)
+        tol = spacing16(aux["ln"]) * np.abs(aux["s1"].astype(np.float64)) + spacing16(aux["p"]) + spacing16(want)
+    else:
+        want = O.np_ln_affine_f16(x2, a.reshape(-1, K), b.reshape(-1, K), eps, rpv)
+        # one rounding to fp16, plus the fp32 rounding of the two terms where they cancel
+        terms = np.abs(O.np_layer_norm_f64(x2, eps) * np.repeat(a.reshape(-1, K), rpv, axis=0)) + np.abs(np.repeat(b.reshape(-1, K), rpv, axis=0))
+        tol = spacing16(want) + 2.0 ** -21 * terms
+    got = h_gpu.reshape(-1, K)
+    err = np.abs(got.astype(np.float64) - want.astype(np.float64))
+    assert (err <= tol).all(), float((err / tol).max())
+    assert (got.view(np.uint16) != want.view(np.uint16)).mean() < 0.01
+    for clip in (1.0, 0.95):
+        qn, sc = pre.quantize(clip)
+        want_s = O.np_row_scale(got, clip)
+        assert np.array_equal(sc.cpu().numpy().view(np.uint16), want_s.view(np.uint16))
+        assert np.array_equal(unpack_native(qn.cpu().numpy(), K), O.np_quantize_rows(got, want_s))
+    if K <= 5120:
+        N = 256
+        _, qw, ws, bias = O.synth_linear(1, K, N, seed=K)
+        qv1, sv1, bb = t16(O.np_pack_wgt_v1(qw)), t16(O.np_pack_wscales_v1(ws, K)), t16(bias)
+        y = fused_ops.linear_ln_vdm_w4a4(pre, qv1, sv1, bb, clip_ratio=0.95)
+        y3 = v.linear_vdm_w4a4(pre.materialize(), qv1, sv1, bb, clip_ratio=0.95)
+        assert tuple(y.shape) == (B, L, N) and torch.equal(y, y3)
+
+
+def test_fused_layer_norm_argument_errors():
+    from dsaquant_amd import fused_ops
+
+    x = torch.randn(2, 10, 128, device=DEV).half()
+    with pytest.raises(ValueError):
+        fused_ops.LnInput(x, torch.zeros(3, 128, device=DEV), torch.zeros(3, 128, device=DEV), 1e-6)  # 3 does not divide 20
+    with pytest.raises(ValueError):
+        fused_ops.LnInput(x, torch.zeros(2, 128, device=DEV), torch.zeros(1, 128, device=DEV), 1e-6)
+    with pytest.raises(ValueError):
+        fused_ops.LnInput(x, torch.zeros(2, 128, device=DEV), torch.zeros(2, 128, device=DEV), 1e-6, mode="rms")
+    big = torch.randn(4, 16384 + 64, device=DEV).half()
+    pre = fused_ops.LnInput(big, torch.zeros(1, 16384 + 64, device=DEV), torch.zeros(1, 16384 + 64, device=DEV), 1e-6)
+    with pytest.raises(RuntimeError):
+        pre.quantize()
+
+
 # --------------------------- large-tile configuration, strided C-ABI calls
 
 @pytest.mark.parametrize("M,N,K", [(4100, 8320, 640), (8200, 8320, 2304)])

@@ -387,3 +387,35 @@ def test_gelu_oracle_is_pinned_by_torch_float64_and_by_its_identities():
     ok = ~(np.isnan(g) | np.isnan(t32))
     ulp = np.abs(g.view(np.int16).astype(np.int32)[ok] - t32.view(np.int16).astype(np.int32)[ok])
     assert ulp.max() <= 3
+
+
+def test_layer_norm_oracles_are_pinned_by_torch():
+    """np_ln_modulate_f16 / np_ln_affine_f16 against torch's own layer_norm (float64) followed by torch's fp16 CPU
+    tensor arithmetic -- the operations the reference's block runs (dit_block.py:100), not a retyped formula --
+    plus the invariances that fix the statistics: shift and positive-scale invariance of LN, zero mean, unit
+    variance."""
+    import torch
+    import torch.nn.functional as F
+
+    rng = np.random.default_rng(0)
+    M, K, eps = 37, 320, 1e-6
+    x = (rng.standard_normal((M, K)) * 3 + 1.5).astype(np.float16)
+    a = (0.3 * rng.standard_normal((M, K))).astype(np.float16)
+    b = (0.5 * rng.standard_normal((M, K))).astype(np.float16)
+    h, aux = O.np_ln_modulate_f16(x, a, b, eps)
+    assert set(aux) == {"ln", "s1", "p"}
+    xt, at, bt = torch.from_numpy(x), torch.from_numpy(a), torch.from_numpy(b)
+    ht = F.layer_norm(xt.double(), (K,), None, None, eps).half() * (1 + at) + bt
+    assert ht.dtype == torch.float16
+    assert np.array_equal(h.view(np.uint16), ht.numpy().view(np.uint16))
+    # one vector per 37 rows
+    h1, _ = O.np_ln_modulate_f16(x, a[:1], b[:1], eps, rows_per_vec=M)
+    ht1 = F.layer_norm(xt.double(), (K,), None, None, eps).half() * (1 + at[:1]) + bt[:1]
+    assert np.array_equal(h1.view(np.uint16), ht1.numpy().view(np.uint16))
+    ha = O.np_ln_affine_f16(x, a[:1], b[:1], eps, rows_per_vec=M)
+    hta = F.layer_norm(xt.double(), (K,), at[0].double(), bt[0].double(), eps).half()
+    assert np.array_equal(ha.view(np.uint16), hta.numpy().view(np.uint16))
+    n = O.np_layer_norm_f64(x, 0.0)
+    assert np.abs(n.mean(axis=1)).max() < 1e-12 and np.abs((n ** 2).mean(axis=1) - 1).max() < 1e-12
+    xf = x.astype(np.float64)
+    assert np.abs(O.np_layer_norm_f64(4.0 * xf + 8.0, 0.0) - O.np_layer_norm_f64(xf, 0.0)).max() < 1e-12
