@@ -31,6 +31,7 @@ def main():
     ap.add_argument("--boundary-ratio", type=float, default=0.4)
     ap.add_argument("--model", default="1.3B", choices=["1.3B", "14B"])
     ap.add_argument("--fuse-ln", action="store_true", help="run the blocks' LayerNorm + modulation inside the following activation quantizers")
+    ap.add_argument("--fuse-residual", action="store_true", help="run the blocks' gated residual updates in the preceding GEMM epilogues")
     ap.add_argument("--fuse-gelu", action="store_true", help="evaluate the FFN's GELU inside the second linear's activation quantizer")
     args = ap.parse_args()
 
@@ -50,6 +51,7 @@ def main():
     build_s = time.perf_counter() - t0
     W.FeedForward.fuse_gelu = bool(args.fuse_gelu)
     W.Block.fuse_ln = bool(args.fuse_ln)
+    W.Block.fuse_residual = bool(args.fuse_residual)
     n_quant = sum(isinstance(m, QuantLinear) for m in model.modules())
     n_fused = sum(isinstance(m, W.Attention) and m.use_fused_qkv_kernel for m in model.modules())
 
@@ -81,7 +83,7 @@ def main():
         "w4a4_ms_per_forward": round(tot.get("w4a4", 0.0) / forwards, 2), "attention_ms_per_forward": round(tot.get("attention", 0.0) / forwards, 2),
         "w4a4_calls_per_forward": cnt.get("w4a4", 0) // forwards, "attention_calls_per_forward": cnt.get("attention", 0) // forwards,
         "tokens_per_forward": tokens, "timesteps": ts, "quant_linears": n_quant, "fused_attention_modules": n_fused,
-        "layers": args.layers, "fuse_gelu": bool(args.fuse_gelu), "fuse_ln": bool(args.fuse_ln), "build_s": round(build_s, 1), "data": "synthetic", "n_gpus": 1,
+        "layers": args.layers, "fuse_gelu": bool(args.fuse_gelu), "fuse_ln": bool(args.fuse_ln), "fuse_residual": bool(args.fuse_residual), "build_s": round(build_s, 1), "data": "synthetic", "n_gpus": 1,
     }))
 
 

@@ -35,6 +35,7 @@ SIGNATURES = {
     "vdmq_linear_ln_w4a4": (_int, [_p, _i64, _i64, _i64, _f32, _int, _p, _p, _i64, _i64, _f32, _p, _p, _p, _p, _int, _i64, _i64, _p, _i64, _p]),
     "vdmq_gelu_tanh_f16": (_int, [_p, _p, _i64, _p]),
     "vdmq_gemm_w4a4": (_int, [_p, _p, _p, _p, _p, _p, _int, _i64, _i64, _i64, _i64, _p]),
+    "vdmq_gemm_w4a4_ex": (_int, [_p, _p, _p, _p, _p, _p, _i64, _i64, _p, _i64, _p, _int, _i64, _i64, _i64, _i64, _p]),
     "vdmq_gemm_w4a4_acc": (_int, [_p, _p, _p, _i64, _i64, _i64, _p]),
     "vdmq_workspace_bytes": (_i64, [_i64, _i64]),
     "vdmq_linear_w4a4": (_int, [_p, _i64, _i64, _i64, _f32, _p, _p, _p, _p, _int, _i64, _i64, _p, _i64, _p]),

@@ -142,7 +142,8 @@ int vdmq_ln_f16(const void *x, int64_t M, int64_t K, int64_t ldx, float eps, int
 }
 
 static int gemm_checked(const void *qact, const void *ascale, const void *wq, const void *wscale, const void *bias, void *out,
-                        int out_dtype, int32_t *acc, int64_t M, int64_t N, int64_t K, int64_t ldo, vdmq_stream_t stream) {
+                        int out_dtype, int32_t *acc, int64_t M, int64_t N, int64_t K, int64_t ldo, const GemmTail &tail,
+                        vdmq_stream_t stream) {
     VDMQ_TRY(check_k(K));
     VDMQ_TRY(check_n(N));
     VDMQ_TRY(check_m(M));
@@ -156,22 +157,47 @@ static int gemm_checked(const void *qact, const void *ascale, const void *wq, co
         if (bias != nullptr) VDMQ_TRY(check_ptr(bias, "bias"));
         if (out_dtype != VDMQ_OUT_F16 && out_dtype != VDMQ_OUT_BF16) return fail(VDMQ_EINVAL, "unknown out_dtype %d", out_dtype);
         if (ldo < N || ldo % 8 != 0) return fail(VDMQ_ESHAPE, "ldo must be >= N and a multiple of 8 (got %lld)", (long long)ldo);
+        if (tail.gate != nullptr || tail.residual != nullptr) {
+            if (out_dtype != VDMQ_OUT_F16) return fail(VDMQ_EINVAL, "gate and residual need an fp16 output");
+            if (tail.gate != nullptr) {
+                VDMQ_TRY(check_ptr(tail.gate, "gate"));
+                if (tail.ldg < N || tail.ldg % 8 != 0) return fail(VDMQ_ESHAPE, "ldg must be >= N and a multiple of 8 (got %lld)", (long long)tail.ldg);
+                if (tail.rows_per_gate <= 0) return fail(VDMQ_ESHAPE, "rows_per_gate must be positive");
+            }
+            if (tail.residual != nullptr) {
+                VDMQ_TRY(check_ptr(tail.residual, "residual"));
+                if (tail.ldr < N || tail.ldr % 8 != 0) return fail(VDMQ_ESHAPE, "ldr must be >= N and a multiple of 8 (got %lld)", (long long)tail.ldr);
+            }
+        }
     } else {
         VDMQ_TRY(check_ptr(acc, "acc"));
     }
     return launch_gemm(static_cast<const uint8_t *>(qact), static_cast<const __half *>(ascale), static_cast<const uint8_t *>(wq),
-                       static_cast<const __half *>(wscale), static_cast<const __half *>(bias), out, out_dtype, acc, M, N, K, ldo,
+                       static_cast<const __half *>(wscale), static_cast<const __half *>(bias), out, out_dtype, acc, M, N, K, ldo, tail,
                        as_stream(stream));
 }
 
 int vdmq_gemm_w4a4(const void *qact, const void *ascale, const void *wq, const void *wscale, const void *bias, void *out,
                    int out_dtype, int64_t M, int64_t N, int64_t K, int64_t ldo, vdmq_stream_t stream) {
-    return gemm_checked(qact, ascale, wq, wscale, bias, out, out_dtype, nullptr, M, N, K, ldo, stream);
+    return gemm_checked(qact, ascale, wq, wscale, bias, out, out_dtype, nullptr, M, N, K, ldo, GemmTail{}, stream);
+}
+
+int vdmq_gemm_w4a4_ex(const void *qact, const void *ascale, const void *wq, const void *wscale, const void *bias, const void *gate,
+                      int64_t ldg, int64_t rows_per_gate, const void *residual, int64_t ldr, void *out, int out_dtype, int64_t M,
+                      int64_t N, int64_t K, int64_t ldo, vdmq_stream_t stream) {
+    if (rows_per_gate > (int64_t(1) << 30)) rows_per_gate = int64_t(1) << 30; /* "one gate vector for every row" */
+    GemmTail tail;
+    tail.gate = static_cast<const __half *>(gate);
+    tail.ldg = ldg;
+    tail.rows_per_gate = static_cast<int>(rows_per_gate);
+    tail.residual = static_cast<const __half *>(residual);
+    tail.ldr = ldr;
+    return gemm_checked(qact, ascale, wq, wscale, bias, out, out_dtype, nullptr, M, N, K, ldo, tail, stream);
 }
 
 int vdmq_gemm_w4a4_acc(const void *qact, const void *wq, int32_t *acc, int64_t M, int64_t N, int64_t K, vdmq_stream_t stream) {
     if (acc == nullptr && M != 0) return fail(VDMQ_EINVAL, "acc is null");
-    return gemm_checked(qact, nullptr, wq, nullptr, nullptr, nullptr, VDMQ_OUT_F16, acc, M, N, K, N, stream);
+    return gemm_checked(qact, nullptr, wq, nullptr, nullptr, nullptr, VDMQ_OUT_F16, acc, M, N, K, N, GemmTail{}, stream);
 }
 
 int64_t vdmq_workspace_bytes(int64_t M, int64_t K) {

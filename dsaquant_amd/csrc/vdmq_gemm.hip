@@ -199,15 +199,17 @@ __device__ __forceinline__ bool map_tile(const TileMap &tm, int bid, int &tile_m
     return tile_m < tm.tiles_m && tile_n < tm.tiles_n;
 }
 
-// OUT_MODE: 0 = scaled output, 1 = scaled output with non-temporal stores, 2 = raw int32 accumulators
+// OUT_MODE: 0 = scaled output, 1 = scaled output with non-temporal stores, 2 = raw int32 accumulators,
+// 3 / 4 = 0 / 1 followed by the gated residual update (a separate instantiation: carrying the tail's
+// branches and registers costs the plain kernel 1 %)
 template <typename Cfg, int OUT_MODE>
 __global__ __launch_bounds__(Cfg::kThreads, Cfg::kOccupancy * Cfg::kWaves / 4) void gemm_w4a4_kernel(const uint8_t *__restrict__ A, const uint8_t *__restrict__ W,
                                                                   const __half *__restrict__ ascale, const __half *__restrict__ wscale,
-                                                                  const __half *__restrict__ bias, void *__restrict__ out, int out_dtype,
+                                                                  const __half *__restrict__ bias, void *out, int out_dtype,
                                                                   int32_t *__restrict__ acc_out, int M, int N, int ldk, int64_t ldo,
-                                                                  TileMap tmap) {
+                                                                  TileMap tmap, GemmTail tail) {
     constexpr int BM = Cfg::BM, BN = Cfg::BN, S = Cfg::STAGES, L = Cfg::kLoads;
-    constexpr bool ACC_OUT = OUT_MODE == 2, STREAM_OUT = OUT_MODE == 1;
+    constexpr bool ACC_OUT = OUT_MODE == 2, STREAM_OUT = OUT_MODE == 1 || OUT_MODE == 4, TAIL = OUT_MODE >= 3;
     extern __shared__ __attribute__((aligned(1024))) uint8_t lds[];
 
     int tile_m, tile_n;
@@ -385,6 +387,18 @@ __global__ __launch_bounds__(Cfg::kThreads, Cfg::kOccupancy * Cfg::kWaves / 4) v
             //   float(256*acc) * fl((as/256) * ws) == fl(float(acc) * fl(as * ws))   bit for bit
             // (no under- or overflow: as*ws/256 >= 2^-56, |256*acc| < 2^31).
             const float as = static_cast<float>(as_p[min(m, M - 1)]) * 0.00390625f;
+            // gate and residual pieces of this strip, requested before the strip is converted and
+            // staged so that their latency runs under that work
+            f16x8 gv[PR / 2], rv[PR / 2];
+#pragma unroll
+            for (int it = 0; TAIL && it < PR / 2; ++it) {
+                const int mrow = m0 + wm0 + mi * 32 + it * (64 / PR) + lane / PR;
+                const bool live = mrow < M && ncol < N;
+                if (tail.gate != nullptr && live)
+                    gv[it] = *reinterpret_cast<const f16x8 *>(tail.gate + static_cast<int64_t>(mrow / tail.rows_per_gate) * tail.ldg + ncol);
+                if (tail.residual != nullptr && live)
+                    rv[it] = *reinterpret_cast<const f16x8 *>(tail.residual + static_cast<int64_t>(mrow) * tail.ldr + ncol);
+            }
 #pragma unroll
             for (int ni = 0; ni < Cfg::kNI; ++ni)
 #pragma unroll
@@ -403,6 +417,10 @@ __global__ __launch_bounds__(Cfg::kThreads, Cfg::kOccupancy * Cfg::kWaves / 4) v
                 f16x8 hv = *reinterpret_cast<const f16x8 *>(stg + row * RS + (lane % PR) * 16);
                 if (bias != nullptr) hv += bv; /* one fp16 add per element */
                 const int mrow = m0 + wm0 + mi * 32 + row;
+                // out = residual + y * gate: the block's gated residual update, two more fp16
+                // operations per element, each rounded like the fp16 tensor operations they replace
+                if (TAIL && tail.gate != nullptr && mrow < M && ncol < N) hv *= gv[it];
+                if (TAIL && tail.residual != nullptr && mrow < M && ncol < N) hv = rv[it] + hv;
 #ifdef VDMQ_DBG_NOSTORE
                 if (mrow < 0 && ncol < N) {
 #else
@@ -467,7 +485,7 @@ __global__ __launch_bounds__(Cfg::kThreads, Cfg::kOccupancy * Cfg::kWaves / 4) v
 
 template <typename Cfg>
 int launch_cfg(const uint8_t *qact, const __half *ascale, const uint8_t *wq, const __half *wscale, const __half *bias, void *out,
-               int out_dtype, int32_t *acc_out, int64_t M, int64_t N, int64_t K, int64_t ldo, hipStream_t s) {
+               int out_dtype, int32_t *acc_out, int64_t M, int64_t N, int64_t K, int64_t ldo, const GemmTail &tail, hipStream_t s) {
     TileMap tm;
     tm.tiles_m = static_cast<int>(ceil_div(M, Cfg::BM));
     tm.tiles_n = static_cast<int>(ceil_div(N, Cfg::BN));
@@ -489,13 +507,15 @@ int launch_cfg(const uint8_t *qact, const __half *ascale, const uint8_t *wq, con
 #else
     const bool stream_out = M * N * 2 > (int64_t(224) << 20);
 #endif
-    const int which = acc_out != nullptr ? 2 : (stream_out ? 1 : 0);
+    const bool has_tail = tail.gate != nullptr || tail.residual != nullptr;
+    const int which = acc_out != nullptr ? 2 : (stream_out ? 1 : 0) + (has_tail ? 3 : 0);
     using Kernel = void (*)(const uint8_t *, const uint8_t *, const __half *, const __half *, const __half *, void *, int, int32_t *, int,
-                            int, int, int64_t, TileMap);
-    const Kernel kernels[3] = {gemm_w4a4_kernel<Cfg, 0>, gemm_w4a4_kernel<Cfg, 1>, gemm_w4a4_kernel<Cfg, 2>};
+                            int, int, int64_t, TileMap, GemmTail);
+    const Kernel kernels[5] = {gemm_w4a4_kernel<Cfg, 0>, gemm_w4a4_kernel<Cfg, 1>, gemm_w4a4_kernel<Cfg, 2>, gemm_w4a4_kernel<Cfg, 3>,
+                               gemm_w4a4_kernel<Cfg, 4>};
     // LDS above 64 KiB has to be requested once per kernel and device
     constexpr int kMaxDevices = 64;
-    static bool attr_done[kMaxDevices][3] = {};
+    static bool attr_done[kMaxDevices][5] = {};
     int dev = 0;
     if (hipGetDevice(&dev) != hipSuccess || dev < 0 || dev >= kMaxDevices) return fail(VDMQ_ELAUNCH, "no current HIP device");
     if (!attr_done[dev][which]) {
@@ -505,14 +525,14 @@ int launch_cfg(const uint8_t *qact, const __half *ascale, const uint8_t *wq, con
         attr_done[dev][which] = true;
     }
     hipLaunchKernelGGL(kernels[which], grid, block, Cfg::kLdsBytes, s, qact, wq, ascale, wscale, bias, out, out_dtype, acc_out,
-                       static_cast<int>(M), static_cast<int>(N), ldk, ldo, tm);
+                       static_cast<int>(M), static_cast<int>(N), ldk, ldo, tm, tail);
     return check_launch("gemm_w4a4_kernel");
 }
 
 }  // namespace
 
 int launch_gemm(const uint8_t *qact, const __half *ascale, const uint8_t *wq, const __half *wscale, const __half *bias, void *out,
-                int out_dtype, int32_t *acc_out, int64_t M, int64_t N, int64_t K, int64_t ldo, hipStream_t s) {
+                int out_dtype, int32_t *acc_out, int64_t M, int64_t N, int64_t K, int64_t ldo, const GemmTail &tail, hipStream_t s) {
     if (M == 0 || N == 0) return VDMQ_OK;
 #ifndef VDMQ_GEMM_CFG
 #define VDMQ_GEMM_CFG 256, 256, 2, 4, 2, 1, 256
@@ -531,11 +551,11 @@ int launch_gemm(const uint8_t *qact, const __half *ascale, const uint8_t *wq, co
     using Big = GemmCfg<VDMQ_GEMM_CFG>;
     const int64_t big_tiles = ceil_div(M, Big::BM) * ceil_div(N, Big::BN);
 #ifndef VDMQ_DBG_ONE_CFG
-    if (big_tiles < 512) return launch_cfg<GemmCfg<VDMQ_GEMM_SMALL_CFG>>(qact, ascale, wq, wscale, bias, out, out_dtype, acc_out, M, N, K, ldo, s);
+    if (big_tiles < 512) return launch_cfg<GemmCfg<VDMQ_GEMM_SMALL_CFG>>(qact, ascale, wq, wscale, bias, out, out_dtype, acc_out, M, N, K, ldo, tail, s);
     if (big_tiles < 1024 || (K < 2048 && big_tiles < 4096))
-        return launch_cfg<GemmCfg<VDMQ_GEMM_MID_CFG>>(qact, ascale, wq, wscale, bias, out, out_dtype, acc_out, M, N, K, ldo, s);
+        return launch_cfg<GemmCfg<VDMQ_GEMM_MID_CFG>>(qact, ascale, wq, wscale, bias, out, out_dtype, acc_out, M, N, K, ldo, tail, s);
 #endif
-    return launch_cfg<Big>(qact, ascale, wq, wscale, bias, out, out_dtype, acc_out, M, N, K, ldo, s);
+    return launch_cfg<Big>(qact, ascale, wq, wscale, bias, out, out_dtype, acc_out, M, N, K, ldo, tail, s);
 }
 
 }  // namespace vdmq

@@ -32,7 +32,17 @@ int launch_ln_quantize(const __half *x, int64_t M, int64_t K, int64_t ldx, float
                        hipStream_t stream);
 int launch_row_scale(const __half *x, int64_t rows, int64_t K, float clip, __half *scale_h, hipStream_t stream);
 int launch_quantize_given_scale(const __half *x, const __half *scale_h, int64_t rows, int64_t K, uint8_t *q, hipStream_t stream);
+// Optional tail of the GEMM epilogue: out = residual + y * gate (fp16 operations), see vdmq_gemm_w4a4_ex.
+struct GemmTail {
+    const __half *gate = nullptr;     /* fp16 [*, N], row m uses row m / rows_per_gate */
+    int64_t ldg = 0;
+    int rows_per_gate = 1;
+    const __half *residual = nullptr; /* fp16 [M, N], row stride ldr */
+    int64_t ldr = 0;
+};
+
 int launch_gemm(const uint8_t *qact, const __half *ascale, const uint8_t *wq, const __half *wscale, const __half *bias,
-                void *out, int out_dtype, int32_t *acc_out, int64_t M, int64_t N, int64_t K, int64_t ldo, hipStream_t stream);
+                void *out, int out_dtype, int32_t *acc_out, int64_t M, int64_t N, int64_t K, int64_t ldo, const GemmTail &tail,
+                hipStream_t stream);
 
 }  // namespace vdmq

@@ -13,7 +13,8 @@ fp16 write and the quantizer's re-read of it disappear.
 ``LnInput`` + ``linear_ln_vdm_w4a4`` / ``qkv_projections_ln`` do the same for
 the block's ``norm(x) * (1 + scale) + shift`` (dit_block.py:100, :110) and for
 the affine ``norm2`` (:105): the LayerNorm, the modulation and the quantizer
-become one pass over ``x``.
+become one pass over ``x``.  ``linear_fused`` adds the consumer side: the gated
+residual update ``hidden_states + y * gate`` (:102, :107, :112) in the GEMM epilogue.
 """
 from __future__ import annotations
 
@@ -52,16 +53,7 @@ def linear_gelu_vdm_w4a4(
     """``linear_vdm_w4a4(gelu_tanh(x), qweight, wscales, bias, clip_ratio, bias_half)``
     in two kernels instead of three; same argument conventions and errors as
     ``linear_vdm_w4a4`` (vdm_w4a4.py:222-244 of the reference)."""
-    _k._load_ext()
-    x_2d, orig_shape = _k._as_2d_half_contiguous(x)
-    _k._check_linear_shapes(x_2d, qweight, wscales)
-    _k._require(x_2d.is_cuda, "input must be a CUDA tensor")
-    native_w, wscale = _k._native_weights(qweight.contiguous(), wscales.contiguous())
-    b = bias_half if bias_half is not None else bias
-    if b is not None:
-        b = b.half().contiguous().view(-1)
-    out = _k._linear_2d(x_2d, native_w, wscale, b, clip_ratio, act="gelu_tanh")
-    return out.view(*orig_shape, -1)
+    return linear_fused(x, qweight, wscales, bias, clip_ratio, bias_half, act="gelu_tanh")
 
 
 class LnInput:
@@ -130,28 +122,81 @@ def linear_ln_vdm_w4a4(
 ) -> torch.Tensor:
     """``linear_vdm_w4a4(pre.materialize(), ...)`` without materializing: LayerNorm,
     modulation and activation quantizer are one kernel, the GEMM the second."""
+    return linear_fused(pre, qweight, wscales, bias, clip_ratio, bias_half)
+
+
+def linear_fused(
+    x,
+    qweight: torch.Tensor,
+    wscales: torch.Tensor,
+    bias: Optional[torch.Tensor] = None,
+    clip_ratio: float = 1.0,
+    bias_half: Optional[torch.Tensor] = None,
+    *,
+    act: Optional[str] = None,
+    residual: Optional[torch.Tensor] = None,
+    gate: Optional[torch.Tensor] = None,
+) -> torch.Tensor:
+    """``residual + linear_vdm_w4a4(act(x), ...) * gate`` in two kernels.
+
+    ``x`` is a tensor (optionally with ``act="gelu_tanh"`` applied to it inside the
+    quantizer) or an ``LnInput``.  ``gate`` (fp16, one ``[N]`` vector per batch element
+    or per token) and ``residual`` (fp16, shaped like the output) are folded into the
+    GEMM epilogue as the two fp16 tensor operations of the reference's
+    ``hidden_states + attn_output * gate`` (dit_block.py:102, :107, :112); either may
+    be omitted.  Returns a new tensor; nothing is updated in place."""
     lib = _k._load_ext()
-    x_2d = pre.x
+    if isinstance(x, LnInput):
+        if act is not None:
+            raise ValueError("an activation cannot be combined with a LayerNorm input")
+        pre, x_2d, lead = x, x.x, x.shape[:-1]
+    else:
+        pre = None
+        x_2d, lead = _k._as_2d_half_contiguous(x)
     _k._check_linear_shapes(x_2d, qweight, wscales)
     _k._require(x_2d.is_cuda, "input must be a CUDA tensor")
+    act_code = _k._act_code(act)
     native_w, wscale = _k._native_weights(qweight.contiguous(), wscales.contiguous())
+    M, K = x_2d.shape
+    N = native_w.shape[0]
+    dev = x_2d.device
     b = bias_half if bias_half is not None else bias
     if b is not None:
         b = b.half().contiguous().view(-1)
         _k._check_device_tensor(b, "bias", torch.float16)
-        _k._require(b.numel() == native_w.shape[0], "bias length must equal N")
-    M, K = x_2d.shape
-    N = native_w.shape[0]
-    dev = x_2d.device
+        _k._require(b.numel() == N, "bias length must equal N")
+    g2 = r2 = None
+    rows_per_gate = 1
+    if gate is not None:
+        if gate.shape[-1] != N:
+            raise ValueError(f"gate must have {N} channels")
+        g2 = gate.reshape(-1, N).half().contiguous()
+        _k._check_device_tensor(g2, "gate", torch.float16)
+        if g2.shape[0] == 0 or (M and M % g2.shape[0] != 0):
+            raise ValueError(f"{g2.shape[0]} gate vectors do not divide {M} rows")
+        rows_per_gate = max(1, M // g2.shape[0])
+    if residual is not None:
+        if tuple(residual.shape) != tuple(lead) + (N,):
+            raise ValueError(f"residual must have shape {tuple(lead) + (N,)}, got {tuple(residual.shape)}")
+        r2 = residual.reshape(-1, N).half().contiguous()
+        _k._check_device_tensor(r2, "residual", torch.float16)
     with torch.cuda.device(dev):
         out = torch.empty((M, N), dtype=torch.float16, device=dev)
         if M:
-            ws_bytes = int(lib.vdmq_workspace_bytes(M, K))
-            workspace = torch.empty((ws_bytes,), dtype=torch.uint8, device=dev)
-            _lib.check(lib.vdmq_linear_ln_w4a4(*pre._args(), float(clip_ratio), native_w.data_ptr(), wscale.data_ptr(),
-                                               None if b is None else b.data_ptr(), out.data_ptr(), _lib.VDMQ_OUT_F16, N, out.stride(0),
-                                               workspace.data_ptr(), ws_bytes, _k._stream(dev)))
-    return out.view(*pre.shape[:-1], N)
+            s = _k._stream(dev)
+            qact = torch.empty((M, _k.k_padded(K) // 2), dtype=torch.uint8, device=dev)
+            scales = torch.empty((M,), dtype=torch.float16, device=dev)
+            if pre is not None:
+                _lib.check(lib.vdmq_quantize_act_ln(*pre._args(), float(clip_ratio), qact.data_ptr(), scales.data_ptr(), s))
+            else:
+                _lib.check(lib.vdmq_quantize_act_ex(x_2d.data_ptr(), M, K, x_2d.stride(0), float(clip_ratio), act_code, qact.data_ptr(),
+                                                    scales.data_ptr(), s))
+            _lib.check(lib.vdmq_gemm_w4a4_ex(
+                qact.data_ptr(), scales.data_ptr(), native_w.data_ptr(), wscale.data_ptr(), None if b is None else b.data_ptr(),
+                None if g2 is None else g2.data_ptr(), 0 if g2 is None else g2.stride(0), rows_per_gate,
+                None if r2 is None else r2.data_ptr(), 0 if r2 is None else r2.stride(0), out.data_ptr(), _lib.VDMQ_OUT_F16, M, N, K,
+                out.stride(0), s))
+    return out.view(*lead, N)
 
 
 def qkv_projections_ln(attn, pre: LnInput):

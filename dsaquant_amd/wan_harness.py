@@ -111,7 +111,9 @@ class Attention(nn.Module):
         self.use_fused_qkv_kernel = False
         self.qkv_kernel_backend = None
 
-    def forward(self, x: torch.Tensor, context: Optional[torch.Tensor], freqs: Optional[torch.Tensor], timers=None) -> torch.Tensor:
+    def forward(self, x, context: Optional[torch.Tensor], freqs: Optional[torch.Tensor], timers=None, residual=None, gate=None) -> torch.Tensor:
+        """Returns the attention output, or ``residual + output * gate`` when ``residual`` is given (the update
+        then runs in the output projection's GEMM epilogue if that projection is in kernel mode)."""
         from . import fused_ops
 
         if isinstance(x, fused_ops.LnInput):  # the LayerNorm in front of this module runs inside the quantizer
@@ -133,7 +135,23 @@ class Attention(nn.Module):
         o = F.scaled_dot_product_attention(q.transpose(1, 2), k.transpose(1, 2), v.transpose(1, 2), dropout_p=0.0, is_causal=False)
         if timers is not None:
             timers.stop("attention")
-        return self.to_out[0](o.transpose(1, 2).flatten(2, 3))
+        return _project_and_update(self.to_out[0], o.transpose(1, 2).flatten(2, 3), None, residual, gate)
+
+
+def _project_and_update(layer, y: torch.Tensor, act: Optional[str], residual, gate) -> torch.Tensor:
+    """``residual + layer(act(y)) * gate`` -- in one fused linear when ``layer`` is a QuantLinear in kernel mode and
+    something can be fused, otherwise as separate tensor operations (dit_block.py:102, :107, :112)."""
+    if getattr(layer, "use_vdm_kernel", False) and (act is not None or residual is not None):
+        from . import fused_ops
+
+        return fused_ops.linear_fused(y, layer.vdm_weight_packed, layer.vdm_weight_scale_packed, layer.bias, layer.kernel_clip_ratio,
+                                      bias_half=layer._bias_half, act=act, residual=residual, gate=gate)
+    if act == "gelu_tanh":
+        y = F.gelu(y, approximate="tanh")
+    out = layer(y)
+    if residual is None:
+        return out
+    return residual + (out if gate is None else out * gate)
 
 
 class FeedForward(nn.Module):
@@ -143,24 +161,18 @@ class FeedForward(nn.Module):
 
     fuse_gelu = False  # evaluate the GELU inside the second linear's activation quantizer
 
-    def forward(self, x: torch.Tensor) -> torch.Tensor:
+    def forward(self, x, residual=None, gate=None) -> torch.Tensor:
         from . import fused_ops
 
         if isinstance(x, fused_ops.LnInput):
             up = self.up
-            x = fused_ops.linear_ln_vdm_w4a4(x, up.vdm_weight_packed, up.vdm_weight_scale_packed, up.bias, up.kernel_clip_ratio,
+            y = fused_ops.linear_ln_vdm_w4a4(x, up.vdm_weight_packed, up.vdm_weight_scale_packed, up.bias, up.kernel_clip_ratio,
                                              bias_half=up._bias_half)
-            return self._second(x)
-        return self._second(self.up(x))
-
-    def _second(self, y: torch.Tensor) -> torch.Tensor:
-        down = self.down
-        if self.fuse_gelu and getattr(down, "use_vdm_kernel", False):
-            from . import fused_ops
-
-            return fused_ops.linear_gelu_vdm_w4a4(y, down.vdm_weight_packed, down.vdm_weight_scale_packed, down.bias,
-                                                  down.kernel_clip_ratio, bias_half=down._bias_half)
-        return down(F.gelu(y, approximate="tanh"))
+        else:
+            y = self.up(x)
+        if self.fuse_gelu:
+            return _project_and_update(self.down, y, "gelu_tanh", residual, gate)
+        return _project_and_update(self.down, F.gelu(y, approximate="tanh"), None, residual, gate)
 
 
 class Block(nn.Module):
@@ -174,17 +186,30 @@ class Block(nn.Module):
         self.scale_shift_table = nn.Parameter(torch.randn(1, 6, a.dim) / a.dim ** 0.5)
 
     fuse_ln = False  # run the three LayerNorms (+ modulation) inside the following linears' activation quantizers
+    fuse_residual = False  # run the three residual updates (x + y * gate) in the preceding linears' GEMM epilogues
 
     def forward(self, x, context, tproj, freqs, timers=None):
         # tproj: [1, 6, dim] (one timestep for the whole sequence; the reference repeats it per token)
         mod = (self.scale_shift_table.to(tproj.dtype) + tproj).unbind(dim=1)
         shift, scale, gate, c_shift, c_scale, c_gate = (m.unsqueeze(1) for m in mod)
-        if self.fuse_ln and getattr(self.ffn.up, "use_vdm_kernel", False) and self.attn1.use_fused_qkv_kernel:
+        kernel_mode = getattr(self.ffn.up, "use_vdm_kernel", False) and self.attn1.use_fused_qkv_kernel
+        if kernel_mode and (self.fuse_ln or self.fuse_residual):
             from .fused_ops import LnInput
 
-            x = x + self.attn1(LnInput(x, scale, shift, self.eps, "modulate"), None, freqs, timers) * gate
-            x = x + self.attn2(LnInput(x, self.norm2.weight, self.norm2.bias, self.eps, "affine"), context, None, timers)
-            return x + self.ffn(LnInput(x, c_scale, c_shift, self.eps, "modulate")) * c_gate
+            def ln(x, a, b, mode):
+                if self.fuse_ln:
+                    return LnInput(x, a, b, self.eps, mode)
+                if mode == "affine":
+                    return fp32_layer_norm(x, a, b, self.eps)
+                return fp32_layer_norm(x, None, None, self.eps) * (1 + a) + b
+
+            if self.fuse_residual:
+                x = self.attn1(ln(x, scale, shift, "modulate"), None, freqs, timers, residual=x, gate=gate)
+                x = self.attn2(ln(x, self.norm2.weight, self.norm2.bias, "affine"), context, None, timers, residual=x)
+                return self.ffn(ln(x, c_scale, c_shift, "modulate"), residual=x, gate=c_gate)
+            x = x + self.attn1(ln(x, scale, shift, "modulate"), None, freqs, timers) * gate
+            x = x + self.attn2(ln(x, self.norm2.weight, self.norm2.bias, "affine"), context, None, timers)
+            return x + self.ffn(ln(x, c_scale, c_shift, "modulate")) * c_gate
         h = fp32_layer_norm(x, None, None, self.eps) * (1 + scale) + shift
         x = x + self.attn1(h, None, freqs, timers) * gate
         h = fp32_layer_norm(x, self.norm2.weight, self.norm2.bias, self.eps)
@@ -369,8 +394,7 @@ class time_w4a4_calls:
 
             return timed
 
-        self._saved = [(k, "linear_vdm_w4a4", k.linear_vdm_w4a4), (fused_ops, "linear_gelu_vdm_w4a4", fused_ops.linear_gelu_vdm_w4a4),
-                       (fused_ops, "linear_ln_vdm_w4a4", fused_ops.linear_ln_vdm_w4a4)]
+        self._saved = [(k, "linear_vdm_w4a4", k.linear_vdm_w4a4), (fused_ops, "linear_fused", fused_ops.linear_fused)]
         for mod, name, orig in self._saved:
             setattr(mod, name, wrap(orig))
         return self

@@ -125,6 +125,20 @@ int vdmq_ln_f16(const void *x, int64_t M, int64_t K, int64_t ldx, float eps, int
 int vdmq_gemm_w4a4(const void *qact, const void *ascale, const void *wq, const void *wscale, const void *bias, void *out,
                    int out_dtype, int64_t M, int64_t N, int64_t K, int64_t ldo, vdmq_stream_t stream);
 
+/* The same GEMM with the block's gated residual update folded into the
+ * epilogue (vdm_infer/models/wan_vdm/modules/dit_block.py:102, :107, :112:
+ * hidden_states = hidden_states + attn_output * gate), y being the output of
+ * vdmq_gemm_w4a4 (bias included):
+ *   out[m,n] = fp16(residual[m,n] + fp16(y[m,n] * gate[m / rows_per_gate, n]))
+ * -- the two fp16 tensor operations the reference runs as separate kernels,
+ * each correctly rounded.  gate fp16 [*, N] (row stride ldg) or NULL (no
+ * multiplication: the attn2 update); residual fp16 [M, N] (row stride ldr) or
+ * NULL; `out` may be `residual` itself (in-place update).  16-byte aligned,
+ * strides multiples of 8; fp16 output only. */
+int vdmq_gemm_w4a4_ex(const void *qact, const void *ascale, const void *wq, const void *wscale, const void *bias, const void *gate,
+                      int64_t ldg, int64_t rows_per_gate, const void *residual, int64_t ldr, void *out, int out_dtype, int64_t M,
+                      int64_t N, int64_t K, int64_t ldo, vdmq_stream_t stream);
+
 /* Same GEMM, but writes the raw int32 accumulators acc [M, N] (row stride N)
  * instead of the scaled output: the checker's view of the value the reference
  * holds in `ipsum` before finalize_int_accum (vdm_w4a4_kernel.cu:650, :684). */

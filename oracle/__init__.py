@@ -285,6 +285,20 @@ def np_epilogue(acc, as_h, ws_h, bias_h=None) -> np.ndarray:
     return h
 
 
+def np_gated_residual(y_h: np.ndarray, gate_h, res_h, rows_per_gate: int = 1) -> np.ndarray:
+    """hidden_states + attn_output * gate on fp16 tensors (dit_block.py:102, :107, :112): the product rounded to
+    fp16, then the sum rounded to fp16.  gate_h [*, N] (row m uses row m // rows_per_gate) or None; res_h or None."""
+    out = y_h
+    if gate_h is not None:
+        g = np.repeat(gate_h.reshape(-1, y_h.shape[-1]), rows_per_gate, axis=0)
+        with np.errstate(over="ignore", invalid="ignore"):
+            out = (out.astype(np.float32) * g.astype(np.float32)).astype(np.float16)  # exact product, one rounding
+    if res_h is not None:
+        with np.errstate(over="ignore", invalid="ignore"):
+            out = (res_h.astype(np.float64) + out.astype(np.float64)).astype(np.float16)  # exact sum, one rounding
+    return out
+
+
 def np_linear(x, qw, ws_h, bias_h=None, clip: float = 1.0):
     as_h = np_row_scale(x, clip)
     qx = np_quantize_rows(x, as_h)

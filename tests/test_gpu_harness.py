@@ -78,12 +78,14 @@ def test_small_dit_structure_and_numerics():
     timers2 = W.KernelTimers()
     W.FeedForward.fuse_gelu = True
     W.Block.fuse_ln = True  # and the three LayerNorms (+ modulation) of a block inside the following quantizers
+    W.Block.fuse_residual = True  # and the three residual updates in the preceding GEMM epilogues
     try:
         with torch.no_grad(), W.time_w4a4_calls(timers2):
             y_fused = model(latent, t, ctx, timers2)
     finally:
         W.FeedForward.fuse_gelu = False
         W.Block.fuse_ln = False
+        W.Block.fuse_residual = False
     timers2.collect()
     assert timers2.counts() == {"w4a4": 7 * args.num_layers, "attention": 2 * args.num_layers}
     assert (y_fused.float() - y.float()).abs().max().item() <= 1e-2 * y.float().abs().max().item() + 1e-3

@@ -453,6 +453,69 @@ def test_fused_layer_norm_argument_errors():
         pre.quantize()
 
 
+# ------------------------------------- gated residual update in the GEMM epilogue
+
+@pytest.mark.parametrize("B,L,K,N,gate_kind", [
+    (2, 150, 1536, 1536, "batch"),      # 128 x 128 tiles
+    (1, 8197, 1536, 4224, "batch"),     # 256 x 128 tiles
+    (1, 8197, 2048, 8448, "token"),     # 256 x 256 tiles, one gate vector per token
+    (3, 100, 320, 256, "none"),         # residual only (the attn2 update)
+    (1, 257, 640, 384, "gate_only"),
+])
+def test_gated_residual_epilogue_bit_exact(B, L, K, N, gate_kind):
+    from dsaquant_amd import fused_ops
+
+    M = B * L
+    x, qw, ws, bias = O.synth_linear(M, K, N, seed=B + L)
+    rng = np.random.default_rng(K + N)
+    res = (2.0 * rng.standard_normal((B, L, N))).astype(np.float16)
+    gate = {"batch": (B, 1, N), "token": (B, L, N), "none": None, "gate_only": (B, 1, N)}[gate_kind]
+    g = None if gate is None else rng.standard_normal(gate).astype(np.float16)
+    r = None if gate_kind == "gate_only" else res
+    qv1, sv1, bb = t16(O.np_pack_wgt_v1(qw)), t16(O.np_pack_wscales_v1(ws, K)), t16(bias)
+    print(f"gated residual B={B} L={L} K={K} N={N} gate={gate_kind}", flush=True)
+    out = fused_ops.linear_fused(t16(x).reshape(B, L, K), qv1, sv1, bb, 0.95, residual=None if r is None else t16(r),
+                                 gate=None if g is None else t16(g))
+    torch.cuda.synchronize()
+    assert tuple(out.shape) == (B, L, N)
+    y = O.np_linear(x, qw, ws, bias, 0.95)[0]
+    rpg = 1 if gate_kind == "token" else L
+    want = O.np_gated_residual(y, None if g is None else g.reshape(-1, N), None if r is None else r.reshape(-1, N), rpg)
+    assert np.array_equal(out.cpu().numpy().reshape(-1, N).view(np.uint16), want.view(np.uint16))
+
+
+def test_gated_residual_in_place_through_the_c_abi_and_errors():
+    """out == residual (the in-place hidden-state update) through vdmq_gemm_w4a4_ex; argument errors."""
+    from dsaquant_amd import _lib, fused_ops
+
+    v = vk()
+    lib = _lib.load()
+    M, K, N = 700, 512, 640
+    x, qw, ws, bias = O.synth_linear(M, K, N, seed=9)
+    rng = np.random.default_rng(2)
+    res = rng.standard_normal((M, N)).astype(np.float16)
+    g = rng.standard_normal((1, N)).astype(np.float16)
+    qn, sc = v.quantize_activation_native(t16(x), 1.0)
+    wn, wsd, bd, gd = t16(pack_native(qw, v.k_padded(K))), t16(ws), t16(bias), t16(g)
+    hidden = t16(res).clone()
+    s = torch.cuda.current_stream().cuda_stream
+    _lib.check(lib.vdmq_gemm_w4a4_ex(qn.data_ptr(), sc.data_ptr(), wn.data_ptr(), wsd.data_ptr(), bd.data_ptr(), gd.data_ptr(), N, M,
+                                     hidden.data_ptr(), N, hidden.data_ptr(), 0, M, N, K, N, s))
+    torch.cuda.synchronize()
+    want = O.np_gated_residual(O.np_linear(x, qw, ws, bias, 1.0)[0], g, res, M)
+    assert np.array_equal(hidden.cpu().numpy().view(np.uint16), want.view(np.uint16))
+    # bf16 output with a tail, bad strides
+    assert lib.vdmq_gemm_w4a4_ex(qn.data_ptr(), sc.data_ptr(), wn.data_ptr(), wsd.data_ptr(), None, gd.data_ptr(), N, M, None, 0,
+                                 hidden.data_ptr(), 1, M, N, K, N, s) == -1
+    assert lib.vdmq_gemm_w4a4_ex(qn.data_ptr(), sc.data_ptr(), wn.data_ptr(), wsd.data_ptr(), None, gd.data_ptr(), N - 8, M, None, 0,
+                                 hidden.data_ptr(), 0, M, N, K, N, s) == -2
+    xt = t16(x)
+    with pytest.raises(ValueError):
+        fused_ops.linear_fused(xt, t16(O.np_pack_wgt_v1(qw)), t16(O.np_pack_wscales_v1(ws, K)), residual=xt)  # wrong shape
+    with pytest.raises(ValueError):
+        fused_ops.linear_fused(xt, t16(O.np_pack_wgt_v1(qw)), t16(O.np_pack_wscales_v1(ws, K)), gate=torch.zeros(3, N, device=DEV))
+
+
 # --------------------------- large-tile configuration, strided C-ABI calls
 
 @pytest.mark.parametrize("M,N,K", [(4100, 8320, 640), (8200, 8320, 2304)])

@@ -419,3 +419,23 @@ def test_layer_norm_oracles_are_pinned_by_torch():
     assert np.abs(n.mean(axis=1)).max() < 1e-12 and np.abs((n ** 2).mean(axis=1) - 1).max() < 1e-12
     xf = x.astype(np.float64)
     assert np.abs(O.np_layer_norm_f64(4.0 * xf + 8.0, 0.0) - O.np_layer_norm_f64(xf, 0.0)).max() < 1e-12
+
+
+def test_gated_residual_oracle_equals_torch_fp16_tensor_arithmetic():
+    import torch
+
+    rng = np.random.default_rng(1)
+    y = (rng.standard_normal((64, 256)) * 3).astype(np.float16)
+    y[0, :8] = [65504, -65504, 0, 1e-7, 6e-8, np.inf, -np.inf, np.nan]
+    g = rng.standard_normal((2, 256)).astype(np.float16)
+    r = (rng.standard_normal((64, 256)) * 5).astype(np.float16)
+    want = (torch.from_numpy(r) + torch.from_numpy(y) * torch.from_numpy(g).repeat_interleave(32, dim=0)).numpy()
+    got = O.np_gated_residual(y, g, r, rows_per_gate=32)
+    both_nan = np.isnan(want) & np.isnan(got)
+    assert np.array_equal(got.view(np.uint16)[~both_nan], want.view(np.uint16)[~both_nan])
+    assert np.array_equal(np.isnan(got), np.isnan(want))
+    assert np.array_equal(O.np_gated_residual(y, None, None).view(np.uint16), y.view(np.uint16))
+    want2 = (torch.from_numpy(r) + torch.from_numpy(y)).numpy()
+    got2 = O.np_gated_residual(y, None, r)
+    ok = ~np.isnan(want2)
+    assert np.array_equal(got2.view(np.uint16)[ok], want2.view(np.uint16)[ok])
