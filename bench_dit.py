@@ -1,6 +1,6 @@
 #!/usr/bin/env python3
 """End-to-end harness: Wan-2.1 1.3B W4A4 DiT denoise steps with random-init
-packed weights (BASELINE config 4), reporting the share of step time spent in
+packed weights (the fifth benchmark configuration: 480p, 81 frames, 5 steps), reporting the share of step time spent in
 the W4A4 kernels.
 
 Latent [2 (CFG pair), 16, 21, 60, 104] ~ N(0,1): the pipeline runs classifier-free
