@@ -170,7 +170,7 @@ __device__ __forceinline__ void schedule_region() {
 // L2), so workgroup b runs on XCD b%8 as its (b/8)-th.  Each XCD walks
 // "super-tiles" of kGroupM x kGroupN tiles (32 = its CU count): the tiles that are
 // resident on an XCD together share kGroupM token row-blocks and kGroupN weight
-// row-blocks, and the 8 XCDs work on neighbouring super-tiles at any moment.
+// row-blocks.
 #ifndef VDMQ_GROUP_M
 #define VDMQ_GROUP_M 8
 #define VDMQ_GROUP_N 4
@@ -178,18 +178,31 @@ __device__ __forceinline__ void schedule_region() {
 constexpr int kXcds = 8, kGroupM = VDMQ_GROUP_M, kGroupN = VDMQ_GROUP_N;
 
 struct TileMap {
-    int tiles_m, tiles_n, super_n, total_super;
+    int tiles_m, tiles_n, super_n;
+    int start[kXcds + 1]; /* XCD x walks super-tiles [start[x], start[x+1]) */
+    int contig;           /* 1: those contiguous runs; 0: super-tiles dealt round-robin (start[kXcds] = their number) */
 };
 
 __device__ __forceinline__ bool map_tile(const TileMap &tm, int bid, int &tile_m, int &tile_n) {
     const int xcd = bid % kXcds, slot = bid / kXcds;
     const int per = kGroupM * kGroupN;
-    const int st = (slot / per) * kXcds + xcd;
     const int j = slot % per;
-    if (st >= tm.total_super) return false;
+    int st;
+    if (tm.contig) {
+        // An XCD walks a contiguous run of super-tiles, n fastest: consecutive ones share their token
+        // slab, and with the K walk reversed on every other one (see the kernel) the part of that slab
+        // read last is still in this XCD's L2 when the next super-tile starts there.  The runs hold
+        // equal numbers of tiles, not of super-tiles (those on the ragged edges are partly empty).
+        st = tm.start[xcd] + slot / per;
+        if (st >= tm.start[xcd + 1]) return false;
+    } else {
+        // super-tiles dealt round-robin: the 8 XCDs work on neighbouring super-tiles at any moment
+        st = (slot / per) * kXcds + xcd;
+        if (st >= tm.start[kXcds]) return false;
+    }
 #ifdef VDMQ_ORDER_M_FIRST
     // consecutive super-tiles run down the token axis: an XCD keeps its weight super-column in L2
-    const int super_m = tm.total_super / tm.super_n;
+    const int super_m = tm.start[kXcds] / tm.super_n;
     tile_m = (st % super_m) * kGroupM + j / kGroupN;
     tile_n = (st / super_m) * kGroupN + j % kGroupN;
 #else
@@ -269,11 +282,17 @@ __global__ __launch_bounds__(Cfg::kThreads, Cfg::kOccupancy * Cfg::kWaves / 4) v
             for (int r = 0; r < 16; ++r) acc[ni][mi][r] = 0;
 
     const int ksteps = ldk / RB;
+    // Every other workgroup of a CU slot walks K backwards: the end of the previous tile's operand
+    // slabs is still in L2 when the next tile, which shares the token slab, starts there (measured:
+    // 18 % fewer bytes fetched from beyond L2, 23 % for the widest shape).  Integer accumulation is
+    // exact in any order.
+    const bool k_reverse = tmap.contig && ((blockIdx.x / (kXcds * kGroupM * kGroupN)) & 1) != 0;
+    auto kpos = [&](int kt) { return k_reverse ? ksteps - 1 - kt : kt; };
 
     // prologue: fill the ring (as far as K reaches), wait for stage 0
 #pragma unroll
     for (int s = 0; s < S; ++s)
-        if (s < ksteps) issue_stage<Cfg>(wbase + s * RB, xbase + s * RB, goff, lds + s * Cfg::kStageBytes, wave);
+        if (s < ksteps) issue_stage<Cfg>(wbase + kpos(s) * RB, xbase + kpos(s) * RB, goff, lds + s * Cfg::kStageBytes, wave);
     if (ksteps >= S)
         __builtin_amdgcn_s_waitcnt(waitcnt_imm(L * (S - 1), 15));
     else
@@ -326,7 +345,7 @@ __global__ __launch_bounds__(Cfg::kThreads, Cfg::kOccupancy * Cfg::kWaves / 4) v
             mma_step<Cfg>(acc, lo);
             schedule_region<Cfg, Cfg::kNI + Cfg::kMI, 0>();
 #ifndef VDMQ_DBG_NOLOAD
-            if (STEADY && j + 1 == R) issue_stage<Cfg>(wbase + (kt + S) * RB, xbase + (kt + S) * RB, goff, lds + cur * Cfg::kStageBytes, wave);
+            if (STEADY && j + 1 == R) issue_stage<Cfg>(wbase + kpos(kt + S) * RB, xbase + kpos(kt + S) * RB, goff, lds + cur * Cfg::kStageBytes, wave);
 #endif
             widen_frags<Cfg, 0>(lo, wn, xn);
             mma_step<Cfg>(acc, hi);
@@ -492,10 +511,34 @@ int launch_cfg(const uint8_t *qact, const __half *ascale, const uint8_t *wq, con
     const int super_m = static_cast<int>(ceil_div(tm.tiles_m, kGroupM));
     tm.super_n = static_cast<int>(ceil_div(tm.tiles_n, kGroupN));
     const int64_t total_super = static_cast<int64_t>(super_m) * tm.super_n;
-    if (total_super * kGroupM * kGroupN + kXcds * kGroupM * kGroupN > (int64_t(1) << 31) - 1)
+    if (total_super * kGroupM * kGroupN + kXcds * kGroupM * kGroupN > (int64_t(1) << 30))
         return fail(VDMQ_ESHAPE, "M x N = %lld x %lld needs more workgroups than one launch can hold", (long long)M, (long long)N);
-    tm.total_super = static_cast<int>(total_super);
-    const int rounds = static_cast<int>(ceil_div(tm.total_super, kXcds));
+    // Split the super-tile sequence (n fastest) into kXcds runs of equal tile counts.  tiles_before(st)
+    // is monotone, so each boundary is a binary search.
+    const int64_t last_m = tm.tiles_m - static_cast<int64_t>(super_m - 1) * kGroupM; /* tile rows of the last super-row */
+    auto tiles_before = [&](int64_t st) {
+        const int64_t sm = st / tm.super_n, sn = st % tm.super_n;
+        const int64_t rows_here = sm == super_m - 1 ? last_m : kGroupM;
+        const int64_t cols_done = sn * kGroupN < tm.tiles_n ? sn * kGroupN : tm.tiles_n;
+        return sm * kGroupM * tm.tiles_n + rows_here * cols_done;
+    };
+    const int64_t all_tiles = static_cast<int64_t>(tm.tiles_m) * tm.tiles_n;
+    tm.start[0] = 0;
+    int rounds = 0;
+    for (int x = 1; x <= kXcds; ++x) {
+        const int64_t want = (all_tiles * x + kXcds - 1) / kXcds;
+        int64_t lo = tm.start[x - 1], hi = total_super; /* first st with tiles_before(st) >= want */
+        while (lo < hi) {
+            const int64_t mid = (lo + hi) / 2;
+            if (tiles_before(mid) >= want) hi = mid; else lo = mid + 1;
+        }
+        tm.start[x] = x == kXcds ? static_cast<int>(total_super) : static_cast<int>(lo);
+        rounds = rounds > tm.start[x] - tm.start[x - 1] ? rounds : tm.start[x] - tm.start[x - 1];
+    }
+    // measured: the contiguous order wins with one workgroup per CU and K >= 3072 (+1 %, 18 % less traffic
+    // beyond L2), loses with two workgroups per CU (-3 %) and at K = 1536 (-4 %)
+    tm.contig = Cfg::kOccupancy == 1 && K >= 2048;
+    if (!tm.contig) rounds = static_cast<int>(ceil_div(total_super, kXcds));
     const dim3 grid(static_cast<unsigned>(rounds) * kXcds * kGroupM * kGroupN), block(Cfg::kThreads);
     const int ldk = static_cast<int>(k_padded(K) / 2);
 
