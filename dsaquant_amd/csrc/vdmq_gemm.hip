@@ -212,6 +212,17 @@ __device__ __forceinline__ bool map_tile(const TileMap &tm, int bid, int &tile_m
     return tile_m < tm.tiles_m && tile_n < tm.tiles_n;
 }
 
+#ifdef VDMQ_DBG_TIMELINE
+// debug build only: per-workgroup cycle stamps (entry, first stage landed, K loop done, epilogue done)
+__device__ unsigned long long g_timeline[4 * 32768];
+#define VDMQ_STAMP(i)                                                                                         \
+    do {                                                                                                      \
+        if (threadIdx.x == 0 && blockIdx.x < 32768) g_timeline[blockIdx.x * 4 + (i)] = __builtin_readcyclecounter(); \
+    } while (0)
+#else
+#define VDMQ_STAMP(i)
+#endif
+
 // OUT_MODE: 0 = scaled output, 1 = scaled output with non-temporal stores, 2 = raw int32 accumulators,
 // 3 / 4 = 0 / 1 followed by the gated residual update (a separate instantiation: carrying the tail's
 // branches and registers costs the plain kernel 1 %)
@@ -227,6 +238,7 @@ __global__ __launch_bounds__(Cfg::kThreads, Cfg::kOccupancy * Cfg::kWaves / 4) v
 
     int tile_m, tile_n;
     if (!map_tile(tmap, blockIdx.x, tile_m, tile_n)) return;
+    VDMQ_STAMP(0);
 #ifdef VDMQ_STAGGER
     // Two workgroups share a CU.  The first grid-wide wave of workgroups fills slot
     // one of every CU, the next one slot two: hold the latter back by about half a
@@ -298,6 +310,7 @@ __global__ __launch_bounds__(Cfg::kThreads, Cfg::kOccupancy * Cfg::kWaves / 4) v
     else
         __builtin_amdgcn_s_waitcnt(waitcnt_imm(0, 15));
     lds_barrier();
+    VDMQ_STAMP(1);
 
     // Software pipeline.  fa/fb hold the raw LDS fragments of the 128-bit read
     // being consumed and of the next one; `lo` holds the widened first half of
@@ -359,6 +372,7 @@ __global__ __launch_bounds__(Cfg::kThreads, Cfg::kOccupancy * Cfg::kWaves / 4) v
     int kt = 0;
     for (; kt + S < ksteps; ++kt) k_step(kt, std::true_type{});
     for (; kt < ksteps; ++kt) k_step(kt, std::false_type{});
+    VDMQ_STAMP(2);
 
     // Epilogue.  Accumulator register r of a 32x32 tile holds
     // n = 8*(r/4) + 4*(lane/32) + r%4, m = lane%32.
@@ -456,6 +470,7 @@ __global__ __launch_bounds__(Cfg::kThreads, Cfg::kOccupancy * Cfg::kWaves / 4) v
                 }
             }
         }
+        VDMQ_STAMP(3);
         return;
     }
 #pragma unroll
@@ -602,3 +617,9 @@ int launch_gemm(const uint8_t *qact, const __half *ascale, const uint8_t *wq, co
 }
 
 }  // namespace vdmq
+
+#ifdef VDMQ_DBG_TIMELINE
+extern "C" int vdmq_debug_timeline(void *host_out, long long bytes) {
+    return hipMemcpyFromSymbol(host_out, HIP_SYMBOL(vdmq::g_timeline), bytes) == hipSuccess ? 0 : -1;
+}
+#endif
