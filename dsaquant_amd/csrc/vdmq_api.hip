@@ -141,6 +141,30 @@ int vdmq_ln_f16(const void *x, int64_t M, int64_t K, int64_t ldx, float eps, int
                               as_stream(stream));
 }
 
+static int check_tail(const GemmTail &tail, int64_t N) {
+    if (tail.gate != nullptr) {
+        VDMQ_TRY(check_ptr(tail.gate, "gate"));
+        if (tail.ldg < N || tail.ldg % 8 != 0) return fail(VDMQ_ESHAPE, "ldg must be >= N and a multiple of 8 (got %lld)", (long long)tail.ldg);
+        if (tail.rows_per_gate <= 0) return fail(VDMQ_ESHAPE, "rows_per_gate must be positive");
+    }
+    if (tail.residual != nullptr) {
+        VDMQ_TRY(check_ptr(tail.residual, "residual"));
+        if (tail.ldr < N || tail.ldr % 8 != 0) return fail(VDMQ_ESHAPE, "ldr must be >= N and a multiple of 8 (got %lld)", (long long)tail.ldr);
+    }
+    return VDMQ_OK;
+}
+
+static GemmTail make_tail(const void *gate, int64_t ldg, int64_t rows_per_gate, const void *residual, int64_t ldr) {
+    if (rows_per_gate > (int64_t(1) << 30)) rows_per_gate = int64_t(1) << 30; /* "one gate vector for every row" */
+    GemmTail tail;
+    tail.gate = static_cast<const __half *>(gate);
+    tail.ldg = ldg;
+    tail.rows_per_gate = static_cast<int>(rows_per_gate);
+    tail.residual = static_cast<const __half *>(residual);
+    tail.ldr = ldr;
+    return tail;
+}
+
 static int gemm_checked(const void *qact, const void *ascale, const void *wq, const void *wscale, const void *bias, void *out,
                         int out_dtype, int32_t *acc, int64_t M, int64_t N, int64_t K, int64_t ldo, const GemmTail &tail,
                         vdmq_stream_t stream) {
@@ -159,15 +183,7 @@ static int gemm_checked(const void *qact, const void *ascale, const void *wq, co
         if (ldo < N || ldo % 8 != 0) return fail(VDMQ_ESHAPE, "ldo must be >= N and a multiple of 8 (got %lld)", (long long)ldo);
         if (tail.gate != nullptr || tail.residual != nullptr) {
             if (out_dtype != VDMQ_OUT_F16) return fail(VDMQ_EINVAL, "gate and residual need an fp16 output");
-            if (tail.gate != nullptr) {
-                VDMQ_TRY(check_ptr(tail.gate, "gate"));
-                if (tail.ldg < N || tail.ldg % 8 != 0) return fail(VDMQ_ESHAPE, "ldg must be >= N and a multiple of 8 (got %lld)", (long long)tail.ldg);
-                if (tail.rows_per_gate <= 0) return fail(VDMQ_ESHAPE, "rows_per_gate must be positive");
-            }
-            if (tail.residual != nullptr) {
-                VDMQ_TRY(check_ptr(tail.residual, "residual"));
-                if (tail.ldr < N || tail.ldr % 8 != 0) return fail(VDMQ_ESHAPE, "ldr must be >= N and a multiple of 8 (got %lld)", (long long)tail.ldr);
-            }
+            VDMQ_TRY(check_tail(tail, N));
         }
     } else {
         VDMQ_TRY(check_ptr(acc, "acc"));
@@ -185,14 +201,8 @@ int vdmq_gemm_w4a4(const void *qact, const void *ascale, const void *wq, const v
 int vdmq_gemm_w4a4_ex(const void *qact, const void *ascale, const void *wq, const void *wscale, const void *bias, const void *gate,
                       int64_t ldg, int64_t rows_per_gate, const void *residual, int64_t ldr, void *out, int out_dtype, int64_t M,
                       int64_t N, int64_t K, int64_t ldo, vdmq_stream_t stream) {
-    if (rows_per_gate > (int64_t(1) << 30)) rows_per_gate = int64_t(1) << 30; /* "one gate vector for every row" */
-    GemmTail tail;
-    tail.gate = static_cast<const __half *>(gate);
-    tail.ldg = ldg;
-    tail.rows_per_gate = static_cast<int>(rows_per_gate);
-    tail.residual = static_cast<const __half *>(residual);
-    tail.ldr = ldr;
-    return gemm_checked(qact, ascale, wq, wscale, bias, out, out_dtype, nullptr, M, N, K, ldo, tail, stream);
+    return gemm_checked(qact, ascale, wq, wscale, bias, out, out_dtype, nullptr, M, N, K, ldo, make_tail(gate, ldg, rows_per_gate, residual, ldr),
+                        stream);
 }
 
 int vdmq_gemm_w4a4_acc(const void *qact, const void *wq, int32_t *acc, int64_t M, int64_t N, int64_t K, vdmq_stream_t stream) {
@@ -245,6 +255,61 @@ int vdmq_linear_w4a4(const void *x, int64_t M, int64_t K, int64_t ldx, float cli
                      vdmq_stream_t stream) {
     return vdmq_linear_w4a4_ex(x, M, K, ldx, clip, VDMQ_ACT_NONE, wq, wscale, bias, out, out_dtype, N, ldo, workspace, workspace_bytes,
                                stream);
+}
+
+int64_t vdmq_bf6_bytes(int64_t rows, int64_t K) {
+    if (rows < 0 || K <= 0) return 0;
+    return bf6_bytes(rows, K);
+}
+
+int vdmq_native_to_bf6(const void *native, int64_t rows, int64_t K, void *blocks, vdmq_stream_t stream) {
+    VDMQ_TRY(check_k(K));
+    VDMQ_TRY(check_m(rows));
+    if (rows == 0) return VDMQ_OK;
+    VDMQ_TRY(check_ptr(native, "native"));
+    VDMQ_TRY(check_ptr(blocks, "blocks"));
+    return launch_nibbles_to_bf6(static_cast<const uint8_t *>(native), rows, K, static_cast<uint8_t *>(blocks), as_stream(stream));
+}
+
+static int gemm_bf6_checked(const void *xblocks, const void *ascale, const void *wblocks, const void *wscale, const void *bias, void *out,
+                            int32_t *acc, int64_t M, int64_t N, int64_t K, int64_t ldo, const GemmTail &tail, vdmq_stream_t stream) {
+    VDMQ_TRY(check_k(K));
+    VDMQ_TRY(check_n(N));
+    VDMQ_TRY(check_m(M));
+    if (M == 0) return VDMQ_OK;
+    VDMQ_TRY(check_ptr(xblocks, "xblocks"));
+    VDMQ_TRY(check_ptr(wblocks, "wblocks"));
+    if (acc == nullptr) {
+        VDMQ_TRY(check_ptr(ascale, "ascale", false));
+        VDMQ_TRY(check_ptr(wscale, "wscale"));
+        VDMQ_TRY(check_ptr(out, "out"));
+        if (bias != nullptr) VDMQ_TRY(check_ptr(bias, "bias"));
+        if (ldo < N || ldo % 8 != 0) return fail(VDMQ_ESHAPE, "ldo must be >= N and a multiple of 8 (got %lld)", (long long)ldo);
+        VDMQ_TRY(check_tail(tail, N));
+    } else {
+        VDMQ_TRY(check_ptr(acc, "acc"));
+    }
+    return launch_gemm_bf6(static_cast<const uint8_t *>(xblocks), static_cast<const __half *>(ascale), static_cast<const uint8_t *>(wblocks),
+                           static_cast<const __half *>(wscale), static_cast<const __half *>(bias), static_cast<__half *>(out), acc, M, N, K,
+                           ldo, tail, as_stream(stream));
+}
+
+int vdmq_gemm_w4a4_bf6(const void *xblocks, const void *ascale, const void *wblocks, const void *wscale, const void *bias, void *out,
+                       int64_t M, int64_t N, int64_t K, int64_t ldo, vdmq_stream_t stream) {
+    return gemm_bf6_checked(xblocks, ascale, wblocks, wscale, bias, out, nullptr, M, N, K, ldo, GemmTail{}, stream);
+}
+
+int vdmq_gemm_w4a4_bf6_ex(const void *xblocks, const void *ascale, const void *wblocks, const void *wscale, const void *bias,
+                          const void *gate, int64_t ldg, int64_t rows_per_gate, const void *residual, int64_t ldr, void *out, int64_t M,
+                          int64_t N, int64_t K, int64_t ldo, vdmq_stream_t stream) {
+    return gemm_bf6_checked(xblocks, ascale, wblocks, wscale, bias, out, nullptr, M, N, K, ldo,
+                            make_tail(gate, ldg, rows_per_gate, residual, ldr), stream);
+}
+
+int vdmq_gemm_w4a4_bf6_acc(const void *xblocks, const void *wblocks, int32_t *acc, int64_t M, int64_t N, int64_t K,
+                           vdmq_stream_t stream) {
+    if (acc == nullptr && M != 0) return fail(VDMQ_EINVAL, "acc is null");
+    return gemm_bf6_checked(xblocks, nullptr, wblocks, nullptr, nullptr, nullptr, acc, M, N, K, N, GemmTail{}, stream);
 }
 
 int vdmq_weight_v1_to_native(const void *qweight_v1, void *wq_native, int64_t N, int64_t K, vdmq_stream_t stream) {

@@ -1,0 +1,357 @@
+// W4A4 GEMM through the bf6 (E3M2) matrix path of gfx950 -- an alternative to
+// the int8 kernel of vdmq_gemm.hip, selected by the caller.
+//
+// v_mfma_f32_32x32x64_f8f6f4 multiplies 6-bit floats at twice the int8 rate.
+// E3M2 represents every integer of [-8, 8] exactly, products and sums of such
+// integers stay exact in the fp32 accumulator while |acc| < 2^24 (K <= 65536
+// gives |acc| <= 2^22), so float(acc) is the same integer the int8 kernel
+// accumulates and the epilogue that follows is bit-identical.
+//
+// Operand layout ("bf6 blocks"): a [rows, K] int4 matrix is stored as blocks of
+// 32 rows x 64 k, row-block major, 1536 bytes each, in the order the MFMA wants
+// its operands: lane (r % 32) + 32 * h of a block holds the 32 six-bit codes of
+// k = 64 * kb + 32 * h + e (code e in bits [6e, 6e + 6) of a 192-bit string);
+// the block is [64 lanes x 16 bytes (bits 0..127)][64 lanes x 8 bytes (bits
+// 128..191)].  A block goes from HBM to LDS with 128-bit direct-to-LDS loads as
+// it is, and from LDS straight into the MFMA operand registers (one 128-bit and
+// one 64-bit read per lane, conflict-free by construction): no widening VALU
+// work at all.  Rows are padded to 32 (zero codes), K to 128.
+#include <type_traits>
+
+#include "vdmq_internal.h"
+
+namespace vdmq {
+namespace {
+
+typedef int v8i __attribute__((ext_vector_type(8)));
+typedef int v4i __attribute__((ext_vector_type(4)));
+typedef float v16f __attribute__((ext_vector_type(16)));
+typedef unsigned int u32x4 __attribute__((ext_vector_type(4)));
+typedef unsigned int u32x2 __attribute__((ext_vector_type(2)));
+typedef _Float16 f16x4 __attribute__((ext_vector_type(4)));
+typedef _Float16 f16x8 __attribute__((ext_vector_type(8)));
+
+#define VDMQ_GLOBAL_PTR(p) ((const __attribute__((address_space(1))) void *)(p))
+#define VDMQ_LDS_PTR(p) ((__attribute__((address_space(3))) void *)(p))
+
+constexpr int waitcnt_imm(int vm, int lgkm) { return (vm & 15) | ((vm >> 4) << 14) | (7 << 4) | ((lgkm & 15) << 8); }
+
+__device__ __forceinline__ void lds_barrier() {
+    asm volatile("" ::: "memory");
+    __builtin_amdgcn_s_barrier();
+    asm volatile("" ::: "memory");
+}
+
+constexpr int kBlkBytes = 1536;                 /* 32 rows x 64 k */
+constexpr int kBlkPlaneB = 1024;                /* offset of the 8-byte plane */
+constexpr int BM = 256, BN = 256, KS = 128, S = 3;
+constexpr int kWavesM = 2, kWavesN = 4, kWaves = kWavesM * kWavesN;
+constexpr int MI = BM / 32 / kWavesM, NI = BN / 32 / kWavesN; /* 32-row blocks per wave: 4 token, 2 weight */
+constexpr int kRbStage = (KS / 64) * kBlkBytes; /* bytes of one row-block per stage */
+constexpr int kStageBytes = (BM + BN) / 32 * kRbStage;
+constexpr int kLoads = kStageBytes / 1024 / kWaves;
+constexpr int kLdsBytes = S * kStageBytes;
+constexpr int kWaveN = NI * 32;
+constexpr int kStageRowBytes = kWaveN * 2 + 16; /* epilogue staging: fp16 strip rows padded by 16 bytes */
+constexpr int kStagingBytes = 32 * kStageRowBytes;
+constexpr int kPiecesPerRow = kWaveN / 8;
+static_assert(kStagingBytes * kWaves <= kLdsBytes, "epilogue staging reuses the stage ring");
+static_assert(kStageBytes % (1024 * kWaves) == 0, "stage splits evenly over the waves");
+static_assert(kLoads * (S - 1) < 64, "vmcnt is a 6-bit counter");
+
+constexpr int kXcds = 8, kGroupM = 8, kGroupN = 4;
+struct Bf6TileMap {
+    int tiles_m, tiles_n, super_n, total_super;
+};
+
+// workgroup b runs on XCD b % 8; each XCD walks 8 x 4 super-tiles (see vdmq_gemm.hip)
+__device__ __forceinline__ bool map_tile(const Bf6TileMap &tm, int bid, int &tile_m, int &tile_n) {
+    const int xcd = bid % kXcds, slot = bid / kXcds, per = kGroupM * kGroupN;
+    const int st = (slot / per) * kXcds + xcd, j = slot % per;
+    if (st >= tm.total_super) return false;
+    tile_m = (st / tm.super_n) * kGroupM + j / kGroupN;
+    tile_n = (st % tm.super_n) * kGroupN + j % kGroupN;
+    return tile_m < tm.tiles_m && tile_n < tm.tiles_n;
+}
+
+__device__ __forceinline__ v8i ld_frag(const uint8_t *p, uint32_t la, uint32_t lb) {
+    const u32x4 a = *reinterpret_cast<const u32x4 *>(p + la);
+    const u32x2 b = *reinterpret_cast<const u32x2 *>(p + lb);
+    v8i r = {(int)a.x, (int)a.y, (int)a.z, (int)a.w, (int)b.x, (int)b.y, 0, 0}; /* the MFMA reads six registers */
+    return r;
+}
+
+template <int NDS, int NVMEM, int I = 0>
+__device__ __forceinline__ void schedule_region() {
+    if constexpr (I < NI * MI) {
+        __builtin_amdgcn_sched_group_barrier(0x008, 1, 0); /* MFMA */
+        if constexpr (2 * I < NDS) __builtin_amdgcn_sched_group_barrier(0x100, 2, 0); /* DS reads */
+        if constexpr (I < NVMEM) __builtin_amdgcn_sched_group_barrier(0x020, 1, 0); /* direct-to-LDS load */
+        schedule_region<NDS, NVMEM, I + 1>();
+    } else {
+        __builtin_amdgcn_sched_barrier(0);
+    }
+}
+
+// OUT_MODE: 0 = scaled fp16 output, 1 = the same with non-temporal stores, 2 = raw accumulators as int32,
+// 3 / 4 = 0 / 1 followed by the gated residual update out = residual + y * gate (see vdmq_gemm.hip)
+template <int OUT_MODE>
+__global__ __launch_bounds__(kWaves * 64, kWaves / 4) void gemm_bf6_kernel(const uint8_t *__restrict__ X, const uint8_t *__restrict__ W,
+                                                                         const __half *__restrict__ ascale,
+                                                                         const __half *__restrict__ wscale,
+                                                                         const __half *__restrict__ bias, __half *out,
+                                                                         int32_t *__restrict__ acc_out, int M, int N, int kblocks,
+                                                                         int64_t ldo, Bf6TileMap tmap, GemmTail tail) {
+    constexpr bool ACC_OUT = OUT_MODE == 2, STREAM_OUT = OUT_MODE == 1 || OUT_MODE == 4, TAIL = OUT_MODE >= 3;
+    extern __shared__ __attribute__((aligned(1024))) uint8_t lds[];
+    int tile_m, tile_n;
+    if (!map_tile(tmap, blockIdx.x, tile_m, tile_n)) return;
+    const int lane = threadIdx.x & 63, wave = __builtin_amdgcn_readfirstlane(threadIdx.x >> 6);
+    const int wn = wave % kWavesN, wm = wave / kWavesN;
+    const int64_t rbs = static_cast<int64_t>(kblocks) * kBlkBytes; /* bytes of one row-block over all K */
+    const int last_rb_m = (M + 31) / 32 - 1, last_rb_n = N / 32 - 1;
+    // global -> LDS: a stage is 16 row-blocks x 3 KiB; this wave's i-th instruction moves KiB (i * kWaves + wave) of it
+    const uint8_t *src[kLoads];
+#pragma unroll
+    for (int i = 0; i < kLoads; ++i) {
+        const int idx = i * kWaves + wave, q = idx / 3, part = idx % 3;
+        const uint8_t *base = q < BN / 32 ? W + static_cast<int64_t>(min(tile_n * (BN / 32) + q, last_rb_n)) * rbs
+                                           : X + static_cast<int64_t>(min(tile_m * (BM / 32) + q - BN / 32, last_rb_m)) * rbs;
+        src[i] = base + part * 1024 + lane * 16; /* rows past M or N re-read the last row-block and are never stored */
+    }
+    auto issue = [&](int kt, int slot) __attribute__((always_inline)) {
+#pragma unroll
+        for (int i = 0; i < kLoads; ++i)
+            __builtin_amdgcn_global_load_lds(VDMQ_GLOBAL_PTR(src[i] + static_cast<int64_t>(kt) * kRbStage),
+                                             VDMQ_LDS_PTR(lds + slot * kStageBytes + (i * kWaves + wave) * 1024), 16, 0, 0);
+    };
+    const uint32_t la = lane * 16, lb = kBlkPlaneB + lane * 8;
+    auto read = [&](v8i (&wf)[NI], v8i (&xf)[MI], const uint8_t *stage, int kb) __attribute__((always_inline)) {
+#pragma unroll
+        for (int ni = 0; ni < NI; ++ni) wf[ni] = ld_frag(stage + ((wn * NI + ni) * 2 + kb) * kBlkBytes, la, lb);
+#pragma unroll
+        for (int mi = 0; mi < MI; ++mi) xf[mi] = ld_frag(stage + ((BN / 32 + wm * MI + mi) * 2 + kb) * kBlkBytes, la, lb);
+    };
+    v16f acc[NI][MI];
+#pragma unroll
+    for (int ni = 0; ni < NI; ++ni)
+#pragma unroll
+        for (int mi = 0; mi < MI; ++mi)
+#pragma unroll
+            for (int r = 0; r < 16; ++r) acc[ni][mi][r] = 0.f;
+    // weight rows are the A operand, token rows the B operand: accumulator register r of a 32 x 32
+    // tile holds n = 8 * (r / 4) + 4 * (lane / 32) + r % 4, m = lane % 32
+    auto mma = [&](const v8i (&wf)[NI], const v8i (&xf)[MI]) __attribute__((always_inline)) {
+#pragma unroll
+        for (int ni = 0; ni < NI; ++ni)
+#pragma unroll
+            for (int mi = 0; mi < MI; ++mi)
+                acc[ni][mi] = __builtin_amdgcn_mfma_scale_f32_32x32x64_f8f6f4(wf[ni], xf[mi], acc[ni][mi], 3, 3, 0, 0, 0, 0); /* bf6 x bf6, no scaling */
+    };
+    const int ksteps = kblocks / (KS / 64);
+#pragma unroll
+    for (int s = 0; s < S; ++s)
+        if (s < ksteps) issue(s, s);
+    if (ksteps >= S)
+        __builtin_amdgcn_s_waitcnt(waitcnt_imm(kLoads * (S - 1), 15));
+    else
+        __builtin_amdgcn_s_waitcnt(waitcnt_imm(0, 15));
+    lds_barrier();
+    v8i wfa[NI], xfa[MI], wfb[NI], xfb[MI];
+    read(wfa, xfa, lds, 0);
+    int cur = 0;
+    // one stage = two k-blocks; the ring is published by one barrier per stage, placed before the second k-block's MFMAs
+    auto k_step = [&](int kt, auto steady_tag) __attribute__((always_inline)) {
+        constexpr bool STEADY = decltype(steady_tag)::value;
+        const uint8_t *stage = lds + cur * kStageBytes;
+        const int nxt = cur + 1 == S ? 0 : cur + 1;
+        read(wfb, xfb, stage, 1);
+        mma(wfa, xfa);
+        schedule_region<2 * (NI + MI), 0>();
+        if (STEADY)
+            __builtin_amdgcn_s_waitcnt(waitcnt_imm(kLoads * (S - 2), 0));
+        else
+            __builtin_amdgcn_s_waitcnt(waitcnt_imm(0, 0));
+        lds_barrier();
+        if (STEADY || kt + 1 < ksteps) read(wfa, xfa, lds + nxt * kStageBytes, 0);
+        if (STEADY) issue(kt + S, cur);
+        mma(wfb, xfb);
+        if (STEADY)
+            schedule_region<2 * (NI + MI), kLoads>();
+        else
+            schedule_region<2 * (NI + MI), 0>();
+        cur = nxt;
+    };
+    int kt = 0;
+    for (; kt + S < ksteps; ++kt) k_step(kt, std::true_type{});
+    for (; kt < ksteps; ++kt) k_step(kt, std::false_type{});
+
+    const int l32 = lane & 31, lh = lane >> 5;
+    const int m0 = tile_m * BM, n0 = tile_n * BN, wm0 = wm * MI * 32, wn0 = wn * NI * 32;
+    if (ACC_OUT) {
+#pragma unroll
+        for (int mi = 0; mi < MI; ++mi) {
+            const int m = m0 + wm0 + mi * 32 + l32;
+            if (m >= M) continue;
+#pragma unroll
+            for (int ni = 0; ni < NI; ++ni)
+#pragma unroll
+                for (int rg = 0; rg < 4; ++rg) {
+                    const int n = n0 + wn0 + ni * 32 + rg * 8 + lh * 4;
+                    if (n >= N) continue;
+                    v4i o;
+#pragma unroll
+                    for (int e = 0; e < 4; ++e) o[e] = static_cast<int>(acc[ni][mi][rg * 4 + e]);
+                    *reinterpret_cast<v4i *>(acc_out + static_cast<int64_t>(m) * N + n) = o;
+                }
+        }
+        return;
+    }
+    // fp16 epilogue, as in the int8 kernel: out = fp16(float(acc) * (float(as) * float(ws))) (+ bias in fp16);
+    // one 32-row strip at a time is transposed through LDS so that rows leave as whole 128-byte lines
+    constexpr int PR = kPiecesPerRow, RS = kStageRowBytes;
+    uint8_t *stg = lds + wave * kStagingBytes;
+    const _Float16 *as_p = reinterpret_cast<const _Float16 *>(ascale);
+    float wsf[NI][4][4];
+#pragma unroll
+    for (int ni = 0; ni < NI; ++ni)
+#pragma unroll
+        for (int rg = 0; rg < 4; ++rg) {
+            const int n = n0 + wn0 + ni * 32 + rg * 8 + lh * 4;
+            const f16x4 w4 = *reinterpret_cast<const f16x4 *>(wscale + min(n, N - 4));
+#pragma unroll
+            for (int e = 0; e < 4; ++e) wsf[ni][rg][e] = static_cast<float>(w4[e]);
+        }
+    const int ncol = n0 + wn0 + (lane % PR) * 8;
+    f16x8 bv = {0, 0, 0, 0, 0, 0, 0, 0};
+    if (bias != nullptr && ncol < N) bv = *reinterpret_cast<const f16x8 *>(bias + ncol);
+#pragma unroll
+    for (int mi = 0; mi < MI; ++mi) {
+        const float as = static_cast<float>(as_p[min(m0 + wm0 + mi * 32 + l32, M - 1)]);
+        // gate and residual pieces of this strip, requested before the strip is converted and staged
+        f16x8 gv[PR / 2], rv[PR / 2];
+#pragma unroll
+        for (int it = 0; TAIL && it < PR / 2; ++it) {
+            const int mrow = m0 + wm0 + mi * 32 + it * (64 / PR) + lane / PR;
+            const bool live = mrow < M && ncol < N;
+            if (tail.gate != nullptr && live)
+                gv[it] = *reinterpret_cast<const f16x8 *>(tail.gate + static_cast<int64_t>(mrow / tail.rows_per_gate) * tail.ldg + ncol);
+            if (tail.residual != nullptr && live)
+                rv[it] = *reinterpret_cast<const f16x8 *>(tail.residual + static_cast<int64_t>(mrow) * tail.ldr + ncol);
+        }
+#pragma unroll
+        for (int ni = 0; ni < NI; ++ni)
+#pragma unroll
+            for (int rg = 0; rg < 4; ++rg) {
+                f16x4 h;
+#pragma unroll
+                for (int e = 0; e < 4; ++e) h[e] = static_cast<_Float16>(acc[ni][mi][rg * 4 + e] * (as * wsf[ni][rg][e]));
+                *reinterpret_cast<f16x4 *>(stg + l32 * RS + (ni * 32 + rg * 8 + lh * 4) * 2) = h;
+            }
+#pragma unroll
+        for (int it = 0; it < PR / 2; ++it) {
+            const int row = it * (64 / PR) + lane / PR;
+            f16x8 hv = *reinterpret_cast<const f16x8 *>(stg + row * RS + (lane % PR) * 16);
+            if (bias != nullptr) hv += bv;
+            const int mrow = m0 + wm0 + mi * 32 + row;
+            if (TAIL && tail.gate != nullptr && mrow < M && ncol < N) hv *= gv[it];
+            if (TAIL && tail.residual != nullptr && mrow < M && ncol < N) hv = rv[it] + hv;
+            if (mrow < M && ncol < N) {
+                f16x8 *dst = reinterpret_cast<f16x8 *>(out + static_cast<int64_t>(mrow) * ldo + ncol);
+                if (STREAM_OUT)
+                    __builtin_nontemporal_store(hv, dst);
+                else
+                    *dst = hv;
+            }
+        }
+    }
+}
+
+// E3M2 code of an int4 value given as a two's complement nibble: sign << 5 | exponent/mantissa of |q|
+__device__ __forceinline__ uint32_t bf6_code(uint32_t nib) {
+    const int q = static_cast<int>(nib << 28) >> 28;
+    const uint32_t a = static_cast<uint32_t>(q < 0 ? -q : q);
+    // |q| = 0..8 -> 0, 1.0, 2.0, 3.0, 4.0, 5.0, 6.0, 7.0, 8.0 as (e << 2 | m): 0, 12, 16, 18, 20, 21, 22, 23, 24
+    const uint64_t table = 0x1716151412100C00ull;
+    const uint32_t mag = a == 8 ? 24u : static_cast<uint32_t>(table >> (8 * a)) & 0xFFu;
+    return (q < 0 ? 32u : 0u) | mag;
+}
+
+// native int4 rows (row-major, low nibble = even k) -> bf6 blocks; one thread per (row-block, k-block, lane)
+__global__ __launch_bounds__(256) void nibbles_to_bf6_kernel(const uint8_t *__restrict__ src, int64_t rows, int64_t src_row_bytes,
+                                                             int kblocks, int src_kblocks, uint8_t *__restrict__ dst, int64_t total) {
+    const int64_t idx = static_cast<int64_t>(blockIdx.x) * blockDim.x + threadIdx.x;
+    if (idx >= total) return;
+    const int l = static_cast<int>(idx & 63);
+    const int64_t blk = idx >> 6;
+    const int kb = static_cast<int>(blk % kblocks);
+    const int64_t rb = blk / kblocks;
+    const int64_t r = rb * 32 + (l & 31);
+    const int h = l >> 5;
+    uint32_t regs[6] = {0, 0, 0, 0, 0, 0};
+    if (r < rows && kb < src_kblocks) {
+        const u32x4 v = *reinterpret_cast<const u32x4 *>(src + r * src_row_bytes + kb * 32 + h * 16); /* 32 nibbles */
+        const uint32_t w[4] = {v.x, v.y, v.z, v.w};
+#pragma unroll
+        for (int e = 0; e < 32; ++e) {
+            const uint64_t code = bf6_code((w[e / 8] >> (4 * (e % 8))) & 0xFu);
+            const int bit = 6 * e, word = bit / 32, sh = bit % 32;
+            regs[word] |= static_cast<uint32_t>(code << sh);
+            if (sh > 26) regs[word + 1] |= static_cast<uint32_t>(code >> (32 - sh));
+        }
+    }
+    uint8_t *b = dst + blk * kBlkBytes;
+    *reinterpret_cast<u32x4 *>(b + l * 16) = u32x4{regs[0], regs[1], regs[2], regs[3]};
+    *reinterpret_cast<u32x2 *>(b + kBlkPlaneB + l * 8) = u32x2{regs[4], regs[5]};
+}
+
+}  // namespace
+
+int64_t bf6_kblocks(int64_t K) { return (K + 127) / 128 * 2; }
+int64_t bf6_bytes(int64_t rows, int64_t K) { return (rows + 31) / 32 * bf6_kblocks(K) * kBlkBytes; }
+
+int launch_nibbles_to_bf6(const uint8_t *native, int64_t rows, int64_t K, uint8_t *blocks, hipStream_t s) {
+    if (rows == 0) return VDMQ_OK;
+    const int64_t kblocks = bf6_kblocks(K);
+    const int64_t total = (rows + 31) / 32 * kblocks * 64;
+    hipLaunchKernelGGL(nibbles_to_bf6_kernel, dim3(static_cast<unsigned>(ceil_div(total, 256))), dim3(256), 0, s, native, rows,
+                       k_padded(K) / 2, static_cast<int>(kblocks), static_cast<int>(k_padded(K) / 64), blocks, total);
+    return check_launch("nibbles_to_bf6_kernel");
+}
+
+int launch_gemm_bf6(const uint8_t *xblocks, const __half *ascale, const uint8_t *wblocks, const __half *wscale, const __half *bias,
+                    __half *out, int32_t *acc_out, int64_t M, int64_t N, int64_t K, int64_t ldo, const GemmTail &tail, hipStream_t s) {
+    if (M == 0 || N == 0) return VDMQ_OK;
+    Bf6TileMap tm;
+    tm.tiles_m = static_cast<int>(ceil_div(M, BM));
+    tm.tiles_n = static_cast<int>(ceil_div(N, BN));
+    const int super_m = static_cast<int>(ceil_div(tm.tiles_m, kGroupM));
+    tm.super_n = static_cast<int>(ceil_div(tm.tiles_n, kGroupN));
+    const int64_t total_super = static_cast<int64_t>(super_m) * tm.super_n;
+    if (total_super * kGroupM * kGroupN + kXcds * kGroupM * kGroupN > (int64_t(1) << 30))
+        return fail(VDMQ_ESHAPE, "M x N = %lld x %lld needs more workgroups than one launch can hold", (long long)M, (long long)N);
+    tm.total_super = static_cast<int>(total_super);
+    const int rounds = static_cast<int>(ceil_div(total_super, kXcds));
+    const dim3 grid(static_cast<unsigned>(rounds) * kXcds * kGroupM * kGroupN), block(kWaves * 64);
+    const bool stream_out = M * N * 2 > (int64_t(224) << 20);
+    const bool has_tail = tail.gate != nullptr || tail.residual != nullptr;
+    const int which = acc_out != nullptr ? 2 : (stream_out ? 1 : 0) + (has_tail ? 3 : 0);
+    using Kernel = void (*)(const uint8_t *, const uint8_t *, const __half *, const __half *, const __half *, __half *, int32_t *, int, int,
+                            int, int64_t, Bf6TileMap, GemmTail);
+    const Kernel kernels[5] = {gemm_bf6_kernel<0>, gemm_bf6_kernel<1>, gemm_bf6_kernel<2>, gemm_bf6_kernel<3>, gemm_bf6_kernel<4>};
+    constexpr int kMaxDevices = 64;
+    static bool attr_done[kMaxDevices][5] = {};
+    int dev = 0;
+    if (hipGetDevice(&dev) != hipSuccess || dev < 0 || dev >= kMaxDevices) return fail(VDMQ_ELAUNCH, "no current HIP device");
+    if (!attr_done[dev][which]) {
+        hipError_t e = hipFuncSetAttribute(reinterpret_cast<const void *>(kernels[which]), hipFuncAttributeMaxDynamicSharedMemorySize,
+                                           kLdsBytes);
+        if (e != hipSuccess) return fail(VDMQ_ELAUNCH, "hipFuncSetAttribute(%d bytes of LDS): %s", kLdsBytes, hipGetErrorString(e));
+        attr_done[dev][which] = true;
+    }
+    hipLaunchKernelGGL(kernels[which], grid, block, kLdsBytes, s, xblocks, wblocks, ascale, wscale, bias, out, acc_out,
+                       static_cast<int>(M), static_cast<int>(N), static_cast<int>(bf6_kblocks(K)), ldo, tm, tail);
+    return check_launch("gemm_bf6_kernel");
+}
+
+}  // namespace vdmq

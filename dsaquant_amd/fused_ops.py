@@ -191,11 +191,7 @@ def linear_fused(
             else:
                 _lib.check(lib.vdmq_quantize_act_ex(x_2d.data_ptr(), M, K, x_2d.stride(0), float(clip_ratio), act_code, qact.data_ptr(),
                                                     scales.data_ptr(), s))
-            _lib.check(lib.vdmq_gemm_w4a4_ex(
-                qact.data_ptr(), scales.data_ptr(), native_w.data_ptr(), wscale.data_ptr(), None if b is None else b.data_ptr(),
-                None if g2 is None else g2.data_ptr(), 0 if g2 is None else g2.stride(0), rows_per_gate,
-                None if r2 is None else r2.data_ptr(), 0 if r2 is None else r2.stride(0), out.data_ptr(), _lib.VDMQ_OUT_F16, M, N, K,
-                out.stride(0), s))
+            _k._gemm_dispatch(qact, scales, native_w, wscale, b, out, K, gate=g2, rows_per_gate=rows_per_gate, residual=r2)
     return out.view(*lead, N)
 
 

@@ -19,6 +19,7 @@ kernel function raises.
 """
 from __future__ import annotations
 
+import os
 import weakref
 from typing import Dict, Optional, Tuple
 
@@ -136,6 +137,80 @@ def _native_weights(qweight: torch.Tensor, wscales: torch.Tensor) -> Tuple[torch
 
 def clear_native_cache() -> None:
     _NATIVE_CACHE.clear()
+    _BF6_CACHE.clear()
+
+
+# ------------------------------------------------- which matrix instructions run the GEMM
+# "int8": v_mfma_i32_32x32x32_i8 on nibbles widened in registers.  "bf6": v_mfma_f32_32x32x64_f8f6f4 on 6-bit
+# floats (twice the rate, no widening work; every int4 value is exact in E3M2, so is the fp32 accumulation).
+# Both give bit-identical results.  "auto" takes bf6 where it is faster: problems with at least
+# _BF6_MIN_TILES 256 x 256 output tiles (its kernel has that one tile shape).
+_MATRIX_PATH = os.environ.get("VDMQ_MATRIX_PATH", "auto")
+_BF6_MIN_TILES = 512
+
+
+def set_matrix_path(name: str) -> None:
+    global _MATRIX_PATH
+    if name not in ("auto", "int8", "bf6"):
+        raise ValueError("matrix path must be 'auto', 'int8' or 'bf6'")
+    _MATRIX_PATH = name
+
+
+def matrix_path() -> str:
+    return _MATRIX_PATH
+
+
+def _use_bf6(M: int, N: int, K: int, out_dtype: torch.dtype = torch.float16) -> bool:
+    if out_dtype != torch.float16 or _MATRIX_PATH == "int8" or M == 0:
+        return False
+    if _MATRIX_PATH == "bf6":
+        return True
+    return ((M + 255) // 256) * ((N + 255) // 256) >= _BF6_MIN_TILES
+
+
+_BF6_CACHE: Dict[tuple, torch.Tensor] = {}
+
+
+def _to_bf6(native: torch.Tensor, rows: int, K: int) -> torch.Tensor:
+    lib = _load_ext()
+    blocks = torch.empty((int(lib.vdmq_bf6_bytes(rows, K)),), dtype=torch.uint8, device=native.device)
+    if rows:
+        _lib.check(lib.vdmq_native_to_bf6(native.data_ptr(), rows, K, blocks.data_ptr(), _stream(native.device)))
+    return blocks
+
+
+def _bf6_weights(native_w: torch.Tensor, K: int) -> torch.Tensor:
+    """bf6 blocks of a native weight tensor, converted once and kept as long as the native tensor lives."""
+    key = (native_w.data_ptr(), tuple(native_w.shape), native_w.device.index, K)
+    hit = _BF6_CACHE.get(key)
+    if hit is None:
+        with torch.cuda.device(native_w.device):
+            hit = _to_bf6(native_w, native_w.shape[0], K)
+        _BF6_CACHE[key] = hit
+        weakref.finalize(native_w, _BF6_CACHE.pop, key, None)
+    return hit
+
+
+def _gemm_dispatch(qact: torch.Tensor, scales: torch.Tensor, native_w: torch.Tensor, wscale: torch.Tensor, bias: Optional[torch.Tensor],
+                   out: torch.Tensor, K: int, gate: Optional[torch.Tensor] = None, rows_per_gate: int = 1,
+                   residual: Optional[torch.Tensor] = None) -> None:
+    """GEMM + epilogue on a quantized activation (native layout) into ``out`` on the chosen matrix path.
+    Must run under ``torch.cuda.device(out.device)``."""
+    lib = _load_ext()
+    M, N = out.shape
+    s = _stream(out.device)
+    bias_p = None if bias is None else bias.data_ptr()
+    gate_p, ldg = (None, 0) if gate is None else (gate.data_ptr(), gate.stride(0))
+    res_p, ldr = (None, 0) if residual is None else (residual.data_ptr(), residual.stride(0))
+    if _use_bf6(M, N, K, out.dtype):
+        wblocks = _bf6_weights(native_w, K)
+        xblocks = _to_bf6(qact, M, K)
+        _lib.check(lib.vdmq_gemm_w4a4_bf6_ex(xblocks.data_ptr(), scales.data_ptr(), wblocks.data_ptr(), wscale.data_ptr(), bias_p, gate_p, ldg,
+                                             rows_per_gate, res_p, ldr, out.data_ptr(), M, N, K, out.stride(0), s))
+        return
+    code = _lib.VDMQ_OUT_F16 if out.dtype == torch.float16 else _lib.VDMQ_OUT_BF16
+    _lib.check(lib.vdmq_gemm_w4a4_ex(qact.data_ptr(), scales.data_ptr(), native_w.data_ptr(), wscale.data_ptr(), bias_p, gate_p, ldg,
+                                     rows_per_gate, res_p, ldr, out.data_ptr(), code, M, N, K, out.stride(0), s))
 
 
 # -------------------------------------------------------------- public API
@@ -212,13 +287,11 @@ def _linear_2d(x_2d: torch.Tensor, native_w: torch.Tensor, wscale: torch.Tensor,
         out = torch.empty((M, N), dtype=out_dtype, device=dev)
         if M == 0:
             return out
-        ws_bytes = int(lib.vdmq_workspace_bytes(M, K))
-        workspace = torch.empty((ws_bytes,), dtype=torch.uint8, device=dev)
-        _lib.check(lib.vdmq_linear_w4a4_ex(
-            x_2d.data_ptr(), M, K, x_2d.stride(0), float(clip_ratio), _act_code(act), native_w.data_ptr(), wscale.data_ptr(),
-            None if bias is None else bias.data_ptr(), out.data_ptr(),
-            _lib.VDMQ_OUT_F16 if out_dtype == torch.float16 else _lib.VDMQ_OUT_BF16, N, out.stride(0), workspace.data_ptr(),
-            ws_bytes, _stream(dev)))
+        qact = torch.empty((M, k_padded(K) // 2), dtype=torch.uint8, device=dev)
+        scales = torch.empty((M,), dtype=torch.float16, device=dev)
+        _lib.check(lib.vdmq_quantize_act_ex(x_2d.data_ptr(), M, K, x_2d.stride(0), float(clip_ratio), _act_code(act), qact.data_ptr(),
+                                            scales.data_ptr(), _stream(dev)))
+        _gemm_dispatch(qact, scales, native_w, wscale, bias, out, K)
     return out
 
 
@@ -313,21 +386,31 @@ def linear_prequantized(qact: torch.Tensor, ascales: torch.Tensor, qweight: torc
         native = torch.empty((M, k_padded(K) // 2), dtype=torch.uint8, device=dev)
         scales = torch.empty((M,), dtype=torch.float16, device=dev)
         _lib.check(lib.vdmq_act_v1_to_native(qact.data_ptr(), ascales.data_ptr(), M, K, native.data_ptr(), scales.data_ptr(), s))
-        _lib.check(lib.vdmq_gemm_w4a4(native.data_ptr(), scales.data_ptr(), native_w.data_ptr(), wscale.data_ptr(), None,
-                                      out.data_ptr(), _lib.VDMQ_OUT_F16, M, N, K, out.stride(0), s))
+        _gemm_dispatch(native, scales, native_w, wscale, None, out, K)
     return out
 
 
-def gemm_int32_accumulators(qact_native: torch.Tensor, wq_native: torch.Tensor, K: int) -> torch.Tensor:
-    """Checker's view: the exact int32 accumulators of the GEMM, [M, N]."""
+def gemm_int32_accumulators(qact_native: torch.Tensor, wq_native: torch.Tensor, K: int, path: Optional[str] = None) -> torch.Tensor:
+    """Checker's view: the exact int32 accumulators of the GEMM, [M, N], on the int8 or the bf6 matrix path
+    (``path`` None: the one ``matrix_path()`` selects for this shape)."""
     lib = _load_ext()
     M, N = qact_native.shape[0], wq_native.shape[0]
     dev = qact_native.device
+    bf6 = path == "bf6" or (path is None and _use_bf6(M, N, K))
     with torch.cuda.device(dev):
         acc = torch.empty((M, N), dtype=torch.int32, device=dev)
-        if M:
+        if M and bf6:
+            xb, wb = _to_bf6(qact_native, M, K), _to_bf6(wq_native, N, K)
+            _lib.check(lib.vdmq_gemm_w4a4_bf6_acc(xb.data_ptr(), wb.data_ptr(), acc.data_ptr(), M, N, K, _stream(dev)))
+        elif M:
             _lib.check(lib.vdmq_gemm_w4a4_acc(qact_native.data_ptr(), wq_native.data_ptr(), acc.data_ptr(), M, N, K, _stream(dev)))
     return acc
+
+
+def bf6_blocks(native: torch.Tensor, K: int) -> torch.Tensor:
+    """The bf6 block form (see include/vdmq.h) of a native int4 buffer, for inspection."""
+    with torch.cuda.device(native.device):
+        return _to_bf6(native.contiguous(), native.shape[0], K)
 
 
 def linear_vdm_w4a4_qkv(

@@ -167,6 +167,26 @@ int vdmq_linear_ln_w4a4(const void *x, int64_t M, int64_t K, int64_t ldx, float 
                         int64_t ldv, int64_t rows_per_vec, float clip, const void *wq, const void *wscale, const void *bias, void *out,
                         int out_dtype, int64_t N, int64_t ldo, void *workspace, int64_t workspace_bytes, vdmq_stream_t stream);
 
+/* ---- bf6 matrix path (optional; no counterpart in the reference).
+ * gfx950 multiplies 6-bit floats (E3M2) at twice its int8 rate, E3M2 holds every
+ * int4 value exactly and fp32 accumulation of their products is exact for
+ * K <= 65536, so the same GEMM can run on v_mfma_f32_32x32x64_f8f6f4 with
+ * bit-identical results.  Operands are "bf6 blocks": 32 rows x 64 k per
+ * 1536-byte block, row-block major, rows padded to 32 and K to 128 with zeros
+ * (vdmq_bf6_bytes gives the size).  vdmq_native_to_bf6 converts a native int4
+ * buffer (weights once per module; activations per call unless the quantizer
+ * writes blocks itself); vdmq_gemm_w4a4_bf6 is vdmq_gemm_w4a4 on such operands
+ * (fp16 output only), vdmq_gemm_w4a4_bf6_acc the int32 accumulator view. */
+int64_t vdmq_bf6_bytes(int64_t rows, int64_t K);
+int vdmq_native_to_bf6(const void *native, int64_t rows, int64_t K, void *blocks, vdmq_stream_t stream);
+int vdmq_gemm_w4a4_bf6(const void *xblocks, const void *ascale, const void *wblocks, const void *wscale, const void *bias, void *out,
+                       int64_t M, int64_t N, int64_t K, int64_t ldo, vdmq_stream_t stream);
+int vdmq_gemm_w4a4_bf6_ex(const void *xblocks, const void *ascale, const void *wblocks, const void *wscale, const void *bias,
+                          const void *gate, int64_t ldg, int64_t rows_per_gate, const void *residual, int64_t ldr, void *out, int64_t M,
+                          int64_t N, int64_t K, int64_t ldo, vdmq_stream_t stream); /* with vdmq_gemm_w4a4_ex's tail */
+int vdmq_gemm_w4a4_bf6_acc(const void *xblocks, const void *wblocks, int32_t *acc, int64_t M, int64_t N, int64_t K,
+                           vdmq_stream_t stream);
+
 /* One-time relayouts between the checkpoint's v1 buffers and native ones.
  * v1 weight layout: weight_quantize_per_channel_kernel + pack_wscales
  * (vdm_w4a4_kernel.cu:518-551, :286-294).  N % 128 == 0, K % 64 == 0. */

@@ -299,6 +299,36 @@ def np_gated_residual(y_h: np.ndarray, gate_h, res_h, rows_per_gate: int = 1) ->
     return out
 
 
+# E3M2 ("bf6") codes of the integers -8..8: sign << 5 | exponent << 2 | mantissa, value = 2^(e-3) * (1 + m/4)
+# for e > 0 (OCP Microscaling Formats specification, FP6 E3M2, bias 3; no infinities or NaNs).
+def np_bf6_decode(code: np.ndarray) -> np.ndarray:
+    """E3M2 code (0..63) -> value, straight from the format definition (subnormals included)."""
+    code = code.astype(np.int64)
+    sign = np.where(code & 32, -1.0, 1.0)
+    e, m = (code >> 2) & 7, code & 3
+    mag = np.where(e == 0, m / 4.0 * 2.0 ** -2, 2.0 ** (e - 3.0) * (1.0 + m / 4.0))
+    return sign * mag
+
+
+def np_unpack_bf6_blocks(blocks: np.ndarray, rows: int, K: int) -> np.ndarray:
+    """bf6 block buffer (u8) -> values float64 [rows, K].  Layout: blocks of 32 rows x 64 k, row-block major, 1536
+    bytes each = [64 lanes x 16 bytes][64 lanes x 8 bytes]; lane (r % 32) + 32 h holds, as one 192-bit little-endian
+    string, the 32 six-bit codes of k = 64 kb + 32 h + e (code e at bits 6e..6e+5).  Also checks the zero padding."""
+    kblocks = (K + 127) // 128 * 2
+    rbs = (rows + 31) // 32
+    b = blocks.reshape(rbs, kblocks, 1536)
+    lo = b[:, :, :1024].reshape(rbs, kblocks, 64, 16)
+    hi = b[:, :, 1024:].reshape(rbs, kblocks, 64, 8)
+    s = np.concatenate([lo, hi], axis=3)                      # 24 bytes per lane
+    bits = np.unpackbits(s, axis=3, bitorder="little")        # 192 bits per lane
+    codes = (bits.reshape(rbs, kblocks, 64, 32, 6) * (1 << np.arange(6))).sum(axis=4)
+    vals = np_bf6_decode(codes)                               # [rb, kb, lane, e]
+    vals = vals.reshape(rbs, kblocks, 2, 32, 32)              # lane = 32 h + r
+    full = vals.transpose(0, 3, 1, 2, 4).reshape(rbs * 32, kblocks * 64)
+    assert not full[rows:].any() and not full[:, K:].any(), "padding must be zero"
+    return full[:rows, :K]
+
+
 def np_linear(x, qw, ws_h, bias_h=None, clip: float = 1.0):
     as_h = np_row_scale(x, clip)
     qx = np_quantize_rows(x, as_h)

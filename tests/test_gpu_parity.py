@@ -516,6 +516,88 @@ def test_gated_residual_in_place_through_the_c_abi_and_errors():
         fused_ops.linear_fused(xt, t16(O.np_pack_wgt_v1(qw)), t16(O.np_pack_wscales_v1(ws, K)), gate=torch.zeros(3, N, device=DEV))
 
 
+# ------------------------------------------------------------ bf6 matrix path
+
+@pytest.fixture
+def bf6_path():
+    v = vk()
+    old = v.matrix_path()
+    v.set_matrix_path("bf6")
+    yield v
+    v.set_matrix_path(old)
+
+
+@pytest.mark.parametrize("M,K", [(257, 1536), (100, 64), (77, 192), (515, 5120), (19, 16384 + 64)])
+def test_bf6_blocks_hold_the_quantized_values(M, K):
+    """native int4 -> bf6 blocks: decoding the blocks with the format's definition gives back the oracle's integers
+    (layout, E3M2 codes and zero padding of rows to 32 and K to 128)."""
+    v = vk()
+    x = special_rows(O.synth_linear(M, K, 128, seed=M + K)[0])
+    qn, sc = v.quantize_activation_native(t16(x), 0.95)
+    blocks = v.bf6_blocks(qn, K).cpu().numpy()
+    want = O.np_quantize_rows(x, O.np_row_scale(x, 0.95))
+    assert np.array_equal(O.np_unpack_bf6_blocks(blocks, M, K), want.astype(np.float64))
+
+
+@pytest.mark.parametrize("M,N,K", [(257, 1536, 1536), (1, 128, 64), (300, 128, 8960), (700, 384, 13824), (4100, 8320, 640), (8200, 8320, 2304)])
+def test_bf6_accumulators_exact(M, N, K):
+    v = vk()
+    rng = np.random.default_rng(M * 7 + N + K)
+    qx = rng.integers(-8, 8, (M, K), dtype=np.int8)
+    qw = rng.integers(-8, 8, (N, K), dtype=np.int8)
+    Kp = v.k_padded(K)
+    print(f"bf6 acc M={M} N={N} K={K}", flush=True)
+    acc = v.gemm_int32_accumulators(t16(pack_native(qx, Kp)), t16(pack_native(qw, Kp)), K, path="bf6")
+    torch.cuda.synchronize()
+    assert np.array_equal(acc.cpu().numpy(), O.np_gemm_i32(qx, qw))
+
+
+def test_bf6_extreme_values_stay_exact():
+    """|acc| up to 64 * K = 2^20 * 0.875 with K = 14336: exact in the fp32 accumulator."""
+    v = vk()
+    K = 14336
+    qx = np.full((64, K), -8, np.int8)
+    qw = np.full((128, K), -8, np.int8)
+    qw[1] = 7
+    acc = v.gemm_int32_accumulators(t16(pack_native(qx, K)), t16(pack_native(qw, K)), K, path="bf6").cpu().numpy()
+    assert (acc[:, 0] == 64 * K).all() and (acc[:, 1] == -56 * K).all()
+
+
+@pytest.mark.parametrize("M,K,N,clip,use_bias", LINEAR_CASES)
+def test_bf6_linear_matches_oracle(bf6_path, M, K, N, clip, use_bias):
+    v = bf6_path
+    x, qw, ws, bias = O.synth_linear(M, K, N, seed=0)
+    print(f"bf6 linear M={M} K={K} N={N}", flush=True)
+    y = v.linear_vdm_w4a4(t16(x), t16(O.np_pack_wgt_v1(qw)), t16(O.np_pack_wscales_v1(ws, K)), t16(bias) if use_bias else None, clip_ratio=clip)
+    torch.cuda.synchronize()
+    want = O.np_linear(x, qw, ws, bias if use_bias else None, clip)[0]
+    assert np.array_equal(y.cpu().numpy().view(np.uint16), want.view(np.uint16))
+
+
+def test_bf6_fused_paths_equal_the_int8_ones(bf6_path):
+    """LayerNorm input, GELU input and gated residual through the bf6 GEMM: bitwise equal to the int8 path."""
+    from dsaquant_amd import fused_ops
+
+    v = bf6_path
+    B, L, K, N = 2, 300, 1536, 1536
+    rng = np.random.default_rng(3)
+    x = (rng.standard_normal((B, L, K)) * 2).astype(np.float16)
+    a, b = (0.2 * rng.standard_normal((B, 1, K))).astype(np.float16), (0.3 * rng.standard_normal((B, 1, K))).astype(np.float16)
+    _, qw, ws, bias = O.synth_linear(1, K, N, seed=5)
+    qv1, sv1, bb = t16(O.np_pack_wgt_v1(qw)), t16(O.np_pack_wscales_v1(ws, K)), t16(bias)
+    res, gate = t16(rng.standard_normal((B, L, N)).astype(np.float16)), t16(rng.standard_normal((B, 1, N)).astype(np.float16))
+
+    def run():
+        pre = fused_ops.LnInput(t16(x), t16(a), t16(b), 1e-6)
+        return (fused_ops.linear_fused(pre, qv1, sv1, bb, 0.95, residual=res, gate=gate),
+                fused_ops.linear_fused(t16(x), qv1, sv1, bb, 1.0, act="gelu_tanh", residual=res))
+
+    got = run()
+    v.set_matrix_path("int8")
+    want = run()
+    assert torch.equal(got[0], want[0]) and torch.equal(got[1], want[1])
+
+
 # --------------------------- large-tile configuration, strided C-ABI calls
 
 @pytest.mark.parametrize("M,N,K", [(4100, 8320, 640), (8200, 8320, 2304)])

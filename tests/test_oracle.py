@@ -439,3 +439,34 @@ def test_gated_residual_oracle_equals_torch_fp16_tensor_arithmetic():
     got2 = O.np_gated_residual(y, None, r)
     ok = ~np.isnan(want2)
     assert np.array_equal(got2.view(np.uint16)[ok], want2.view(np.uint16)[ok])
+
+
+def test_bf6_decoder_follows_the_format_and_holds_every_int4_value():
+    """np_bf6_decode against the E3M2 value table worked by hand (exponent bias 3, 2 mantissa bits, subnormals at
+    e = 0, maximum 28): all 32 magnitudes are listed; every integer -8..8 has exactly one code."""
+    table = [0, 0.0625, 0.125, 0.1875, 0.25, 0.3125, 0.375, 0.4375, 0.5, 0.625, 0.75, 0.875, 1, 1.25, 1.5, 1.75,
+             2, 2.5, 3, 3.5, 4, 5, 6, 7, 8, 10, 12, 14, 16, 20, 24, 28]
+    codes = np.arange(64)
+    vals = O.np_bf6_decode(codes)
+    assert np.array_equal(vals[:32], np.array(table, dtype=np.float64))
+    assert np.array_equal(vals[32:], -np.array(table, dtype=np.float64))
+    for q in range(-8, 9):
+        assert (vals == q).sum() == (2 if q == 0 else 1)  # +0 and -0
+    # unpacker: a hand-built block buffer (row r, column k holds ((r + k) % 16) - 8) decodes to itself
+    rows, K = 40, 192
+    want = (np.add.outer(np.arange(rows), np.arange(K)) % 16 - 8).astype(np.int64)
+    enc = {int(v): int(c) for c, v in zip(codes, vals) if float(v).is_integer() and -8 <= v <= 8 and not (v == 0 and c >= 32)}
+    kblocks, rbs = (K + 127) // 128 * 2, (rows + 31) // 32
+    buf = np.zeros((rbs, kblocks, 1536), np.uint8)
+    for r in range(rows):
+        for kb in range(K // 64):
+            for h in range(2):
+                bits = np.zeros(192, np.uint8)
+                for e in range(32):
+                    c = enc[int(want[r, 64 * kb + 32 * h + e])]
+                    bits[6 * e: 6 * e + 6] = [(c >> i) & 1 for i in range(6)]
+                by = np.packbits(bits, bitorder="little")
+                lane = (r % 32) + 32 * h
+                buf[r // 32, kb, lane * 16: lane * 16 + 16] = by[:16]
+                buf[r // 32, kb, 1024 + lane * 8: 1024 + lane * 8 + 8] = by[16:]
+    assert np.array_equal(O.np_unpack_bf6_blocks(buf.reshape(-1), rows, K), want.astype(np.float64))
