@@ -49,6 +49,8 @@ SIGNATURES = {
     "vdmq_row_scale": (_int, [_p, _i64, _i64, _f32, _p, _p]),
     "vdmq_quantize_weight_native": (_int, [_p, _p, _p, _i64, _i64, _p]),
     "vdmq_bf6_bytes": (_i64, [_i64, _i64]),
+    "vdmq_quantize_act_bf6": (_int, [_p, _i64, _i64, _i64, _f32, _int, _p, _p, _p]),
+    "vdmq_quantize_act_ln_bf6": (_int, [_p, _i64, _i64, _i64, _f32, _int, _p, _p, _i64, _i64, _f32, _p, _p, _p]),
     "vdmq_native_to_bf6": (_int, [_p, _i64, _i64, _p, _p]),
     "vdmq_gemm_w4a4_bf6": (_int, [_p, _p, _p, _p, _p, _p, _i64, _i64, _i64, _i64, _p]),
     "vdmq_gemm_w4a4_bf6_ex": (_int, [_p, _p, _p, _p, _p, _p, _i64, _i64, _p, _i64, _p, _i64, _i64, _i64, _i64, _p]),

@@ -76,8 +76,8 @@ const char *vdmq_arch(void) { return "gfx950"; }
 const char *vdmq_last_error(void) { return g_error; }
 int64_t vdmq_k_padded(int64_t K) { return k_padded(K); }
 
-int vdmq_quantize_act_ex(const void *x, int64_t M, int64_t K, int64_t ldx, float clip, int act, void *qact, void *scale_h,
-                         vdmq_stream_t stream) {
+static int quantize_act_checked(const void *x, int64_t M, int64_t K, int64_t ldx, float clip, int act, int fmt, void *qact,
+                                void *scale_h, vdmq_stream_t stream) {
     VDMQ_TRY(check_k(K));
     VDMQ_TRY(check_m(M));
     if (act != VDMQ_ACT_NONE && act != VDMQ_ACT_GELU_TANH) return fail(VDMQ_EINVAL, "unknown activation %d", act);
@@ -86,8 +86,18 @@ int vdmq_quantize_act_ex(const void *x, int64_t M, int64_t K, int64_t ldx, float
     VDMQ_TRY(check_ptr(qact, "qact"));
     VDMQ_TRY(check_ptr(scale_h, "scale_h", false));
     if (ldx < K || ldx % 8 != 0) return fail(VDMQ_ESHAPE, "ldx must be >= K and a multiple of 8 (got %lld)", (long long)ldx);
-    return launch_quantize_act(static_cast<const __half *>(x), M, K, ldx, clip, act, static_cast<uint8_t *>(qact),
+    return launch_quantize_act(static_cast<const __half *>(x), M, K, ldx, clip, act, fmt, static_cast<uint8_t *>(qact),
                                static_cast<__half *>(scale_h), as_stream(stream));
+}
+
+int vdmq_quantize_act_ex(const void *x, int64_t M, int64_t K, int64_t ldx, float clip, int act, void *qact, void *scale_h,
+                         vdmq_stream_t stream) {
+    return quantize_act_checked(x, M, K, ldx, clip, act, 0, qact, scale_h, stream);
+}
+
+int vdmq_quantize_act_bf6(const void *x, int64_t M, int64_t K, int64_t ldx, float clip, int act, void *xblocks, void *scale_h,
+                          vdmq_stream_t stream) {
+    return quantize_act_checked(x, M, K, ldx, clip, act, 1, xblocks, scale_h, stream);
 }
 
 int vdmq_quantize_act(const void *x, int64_t M, int64_t K, int64_t ldx, float clip, void *qact, void *scale_h, vdmq_stream_t stream) {
@@ -119,15 +129,26 @@ static int ln_checked(const void *x, int64_t M, int64_t K, int64_t ldx, int ln_m
     return VDMQ_OK;
 }
 
-int vdmq_quantize_act_ln(const void *x, int64_t M, int64_t K, int64_t ldx, float eps, int ln_mode, const void *a, const void *b,
-                         int64_t ldv, int64_t rows_per_vec, float clip, void *qact, void *scale_h, vdmq_stream_t stream) {
+static int quantize_act_ln_checked(const void *x, int64_t M, int64_t K, int64_t ldx, float eps, int ln_mode, const void *a, const void *b,
+                                   int64_t ldv, int64_t rows_per_vec, float clip, int fmt, void *qact, void *scale_h,
+                                   vdmq_stream_t stream) {
     VDMQ_TRY(ln_checked(x, M, K, ldx, ln_mode, a, b, ldv, rows_per_vec));
     if (M == 0) return VDMQ_OK;
     VDMQ_TRY(check_ptr(qact, "qact"));
     VDMQ_TRY(check_ptr(scale_h, "scale_h", false));
     return launch_ln_quantize(static_cast<const __half *>(x), M, K, ldx, eps, ln_mode, static_cast<const __half *>(a),
-                              static_cast<const __half *>(b), ldv, rows_per_vec, clip, static_cast<uint8_t *>(qact),
+                              static_cast<const __half *>(b), ldv, rows_per_vec, clip, fmt, static_cast<uint8_t *>(qact),
                               static_cast<__half *>(scale_h), nullptr, 0, as_stream(stream));
+}
+
+int vdmq_quantize_act_ln(const void *x, int64_t M, int64_t K, int64_t ldx, float eps, int ln_mode, const void *a, const void *b,
+                         int64_t ldv, int64_t rows_per_vec, float clip, void *qact, void *scale_h, vdmq_stream_t stream) {
+    return quantize_act_ln_checked(x, M, K, ldx, eps, ln_mode, a, b, ldv, rows_per_vec, clip, 0, qact, scale_h, stream);
+}
+
+int vdmq_quantize_act_ln_bf6(const void *x, int64_t M, int64_t K, int64_t ldx, float eps, int ln_mode, const void *a, const void *b,
+                             int64_t ldv, int64_t rows_per_vec, float clip, void *xblocks, void *scale_h, vdmq_stream_t stream) {
+    return quantize_act_ln_checked(x, M, K, ldx, eps, ln_mode, a, b, ldv, rows_per_vec, clip, 1, xblocks, scale_h, stream);
 }
 
 int vdmq_ln_f16(const void *x, int64_t M, int64_t K, int64_t ldx, float eps, int ln_mode, const void *a, const void *b, int64_t ldv,
@@ -137,7 +158,7 @@ int vdmq_ln_f16(const void *x, int64_t M, int64_t K, int64_t ldx, float eps, int
     VDMQ_TRY(check_ptr(h, "h"));
     if (ldh < K || ldh % 8 != 0) return fail(VDMQ_ESHAPE, "ldh must be >= K and a multiple of 8 (got %lld)", (long long)ldh);
     return launch_ln_quantize(static_cast<const __half *>(x), M, K, ldx, eps, ln_mode, static_cast<const __half *>(a),
-                              static_cast<const __half *>(b), ldv, rows_per_vec, 1.0f, nullptr, nullptr, static_cast<__half *>(h), ldh,
+                              static_cast<const __half *>(b), ldv, rows_per_vec, 1.0f, 0, nullptr, nullptr, static_cast<__half *>(h), ldh,
                               as_stream(stream));
 }
 

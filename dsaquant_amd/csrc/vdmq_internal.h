@@ -23,12 +23,13 @@ inline int64_t ceil_div(int64_t a, int64_t b) { return (a + b - 1) / b; }
 inline bool aligned16(const void *p) { return (reinterpret_cast<uintptr_t>(p) & 15u) == 0; }
 
 // kernels' host launchers (no argument checking: the extern "C" layer does it)
-int launch_quantize_act(const __half *x, int64_t M, int64_t K, int64_t ldx, float clip, int act, uint8_t *qact, __half *scale_h,
-                        hipStream_t stream);
+// fmt: 0 = native int4 rows, 1 = bf6 blocks
+int launch_quantize_act(const __half *x, int64_t M, int64_t K, int64_t ldx, float clip, int act, int fmt, uint8_t *qact,
+                        __half *scale_h, hipStream_t stream);
 int launch_gelu_tanh(const __half *x, __half *y, int64_t n, hipStream_t stream);
 // h_out == nullptr: quantize into qact/scale_h; otherwise write the normalised fp16 rows to h_out
 int launch_ln_quantize(const __half *x, int64_t M, int64_t K, int64_t ldx, float eps, int ln_mode, const __half *va, const __half *vb,
-                       int64_t ldv, int64_t rows_per_vec, float clip, uint8_t *qact, __half *scale_h, __half *h_out, int64_t ldh,
+                       int64_t ldv, int64_t rows_per_vec, float clip, int fmt, uint8_t *qact, __half *scale_h, __half *h_out, int64_t ldh,
                        hipStream_t stream);
 int launch_row_scale(const __half *x, int64_t rows, int64_t K, float clip, __half *scale_h, hipStream_t stream);
 int launch_quantize_given_scale(const __half *x, const __half *scale_h, int64_t rows, int64_t K, uint8_t *q, hipStream_t stream);

@@ -202,6 +202,123 @@ __device__ __forceinline__ void quantize_held_row(const u32x4 (&v)[NCH], int lan
     if (lane == 0) scale_h[row] = sh;
 }
 
+// The same, written as bf6 blocks (the operand form of the bf6 GEMM, see vdmq_bf6.hip): 32 rows x 64 k
+// per 1536-byte block, lane (row % 32) + 32 * h of a block holding the 32 six-bit E3M2 codes of
+// k = 64 * kb + 32 * h + e as one 192-bit string.  A lane needs 32 consecutive k for that, but holds
+// 8 per chunk: four chunks at a time go through a wave-private LDS buffer in k order (16 bytes of
+// padding per 256 keep both the 16-byte writes and the 64-byte-per-lane reads free of bank
+// conflicts) and come back as 32 consecutive fp16 per lane.  Those are scaled, rounded to integers
+// (v_rndne_f32: half to even) and clamped exactly as in quantize_word_fast / quantize_word_exact,
+// and v_cvt_scalef32_pk32_bf6_f16 packs the 32 integers -- every one of [-8, 7] is an E3M2 value,
+// so the conversion is exact -- into the string.  Rows of the last row-block beyond M stay unwritten
+// (the GEMM never stores them); K is padded to 128 with zeros.
+typedef _Float16 f16x32 __attribute__((ext_vector_type(32)));
+typedef unsigned int u32x6 __attribute__((ext_vector_type(6)));
+typedef unsigned int u32x2 __attribute__((ext_vector_type(2)));
+constexpr int kBf6Rows = 8;                      /* rows (= waves) per workgroup of the bf6 quantizers */
+constexpr int kTransposeBytes = 4 * (1024 + 64); /* four chunks plus padding, per wave */
+constexpr int kStringsPerGroup = 64;             /* 2048 k = 64 strings of 32 k per row and group */
+
+struct Bf6Scratch { /* LDS of one workgroup */
+    uint8_t transpose[kBf6Rows][kTransposeBytes];
+    // the strings of one group, 16-byte and 8-byte parts, [row][string] with one string of padding per row;
+    // two copies, used alternately, so that one barrier per group is enough
+    uint8_t part_a[2][kBf6Rows][(kStringsPerGroup + 1) * 16];
+    uint8_t part_b[2][kBf6Rows][(kStringsPerGroup + 1) * 8];
+};
+
+// `valid`: the wave's row exists (a workgroup's waves all run this function -- it synchronises them --
+// the ones past M on a copy of the last row, storing nothing).
+template <int NCH>
+__device__ __forceinline__ void quantize_held_row_bf6(const u32x4 (&v)[NCH], int lane, int wave, int64_t row0, bool valid, int M, int Kb,
+                                                      float clip, uint8_t *__restrict__ blocks, __half *__restrict__ scale_h,
+                                                      Bf6Scratch &lds) {
+    uint32_t m2 = 0;
+#pragma unroll
+    for (int c = 0; c < NCH; ++c) m2 = absmax_bits(v[c], m2);
+    uint32_t m16 = (m2 & 0xFFFFu) > (m2 >> 16) ? (m2 & 0xFFFFu) : (m2 >> 16);
+    m16 = wave_max(m16);
+    __half sh;
+    bool fast = m16 < 0x7C00u; /* every element finite */
+    if (fast) {
+        sh = scale_from_absmax(half_bits_to_float(m16), clip);
+        fast = scale_is_ordinary(sh);
+    }
+    if (!fast) {
+        float mx = 0.0f;
+#pragma unroll
+        for (int c = 0; c < NCH; ++c) mx = absmax_exact(v[c], mx);
+        mx = wave_max(mx);
+        sh = scale_from_absmax(mx, clip);
+    }
+    const float rscale = 1.0f / __half2float(sh);
+    const bool fast_u = __builtin_amdgcn_readfirstlane(fast ? 1 : 0) != 0; /* the same in every lane: a scalar branch */
+    if (lane == 0 && valid) scale_h[row0 + wave] = sh;
+
+    const int kblocks = Kb / 64;
+    uint8_t *tbuf = lds.transpose[wave];
+    // the thread's share of the cooperative store: string t / 8 of row t % 8 -- eight consecutive
+    // threads write the eight rows' parts of one string slot, 128 (and 64) contiguous bytes
+    const int t = threadIdx.x, srow = t % kBf6Rows, sidx = t / kBf6Rows;
+    const int64_t grow = row0 + srow;
+    uint8_t *rowblk = blocks + (grow / 32) * static_cast<int64_t>(kblocks) * 1536;
+    const int slot = static_cast<int>(grow % 32);
+    constexpr int NG = (NCH + 3) / 4;
+#pragma unroll
+    for (int g = 0; g < NG; ++g) {
+#pragma unroll
+        for (int cc = 0; cc < 4; ++cc) {
+            const int c = 4 * g + cc;
+            const uint32_t off = cc * 1024 + lane * 16;
+            *reinterpret_cast<u32x4 *>(tbuf + off + (off >> 8) * 16) = c < NCH ? v[c] : u32x4{0u, 0u, 0u, 0u};
+        }
+        // (the LDS queue of a wave is in order: the reads below see the writes above)
+        u32x4 tr[4];
+#pragma unroll
+        for (int u = 0; u < 4; ++u) tr[u] = *reinterpret_cast<const u32x4 *>(tbuf + lane * 64 + u * 16 + (lane >> 2) * 16);
+        f16x32 q; /* this lane's 32 consecutive k: 2048 g + 32 lane ... */
+        if (fast_u) {
+#pragma unroll
+            for (int u = 0; u < 4; ++u) {
+                const uint32_t w[4] = {tr[u].x, tr[u].y, tr[u].z, tr[u].w};
+#pragma unroll
+                for (int i = 0; i < 4; ++i) {
+                    const f16x2 h = __builtin_bit_cast(f16x2, w[i]);
+                    q[u * 8 + i * 2] = static_cast<_Float16>(__builtin_rintf(__builtin_amdgcn_fmed3f(static_cast<float>(h[0]) * rscale, -8.0f, 7.0f)));
+                    q[u * 8 + i * 2 + 1] = static_cast<_Float16>(__builtin_rintf(__builtin_amdgcn_fmed3f(static_cast<float>(h[1]) * rscale, -8.0f, 7.0f)));
+                }
+            }
+        } else {
+#pragma unroll
+            for (int u = 0; u < 4; ++u) {
+                const uint32_t w[4] = {tr[u].x, tr[u].y, tr[u].z, tr[u].w};
+#pragma unroll
+                for (int i = 0; i < 4; ++i) {
+                    const f16x2 h = __builtin_bit_cast(f16x2, w[i]);
+#pragma unroll
+                    for (int e = 0; e < 2; ++e) { /* NaN -> 0, saturate, round half to even: cvt.rni + cvt.pack.sat of the reference */
+                        const float p = static_cast<float>(h[e]) * rscale;
+                        q[u * 8 + i * 2 + e] = static_cast<_Float16>(p != p ? 0.0f : (p >= 7.0f ? 7.0f : (p <= -8.0f ? -8.0f : __builtin_rintf(p))));
+                    }
+                }
+            }
+        }
+        const u32x6 str = __builtin_amdgcn_cvt_scalef32_pk32_bf6_f16(q, 1.0f);
+        // per-lane stores would scatter 16-byte pieces over 64 cache lines per instruction (measured: 2x
+        // slower than the HBM-bound int4 quantizer): collect the workgroup's strings in LDS instead
+        *reinterpret_cast<u32x4 *>(lds.part_a[g & 1][wave] + lane * 16) = u32x4{str[0], str[1], str[2], str[3]};
+        *reinterpret_cast<u32x2 *>(lds.part_b[g & 1][wave] + lane * 8) = u32x2{str[4], str[5]};
+        __syncthreads(); /* also orders this group's writes after every thread's reads of the group before last */
+        const int k0 = 2048 * g + 32 * sidx;
+        if (k0 < Kb && grow < M) {
+            uint8_t *blk = rowblk + static_cast<int64_t>(k0 >> 6) * 1536;
+            const int l = slot + 32 * ((k0 >> 5) & 1);
+            *reinterpret_cast<u32x4 *>(blk + l * 16) = *reinterpret_cast<const u32x4 *>(lds.part_a[g & 1][srow] + sidx * 16);
+            *reinterpret_cast<u32x2 *>(blk + 1024 + l * 8) = *reinterpret_cast<const u32x2 *>(lds.part_b[g & 1][srow] + sidx * 8);
+        }
+    }
+}
+
 // NCH = number of 512-element chunks (one 128-bit load per lane each) that
 // cover the padded row.  STREAM_OUT: write the nibbles with non-temporal
 // stores -- measured faster once the output no longer fits the 256 MB
@@ -209,14 +326,20 @@ __device__ __forceinline__ void quantize_held_row(const u32x4 (&v)[NCH], int lan
 // ACT: an elementwise activation applied to the row (in fp32, rounded to fp16)
 // before it is quantized: the activation kernel between two linears, its write
 // and the quantizer's re-read of its output are saved.
-template <int NCH, bool STREAM_OUT, int ACT>
-__global__ __launch_bounds__(kRowsPerBlock * kWaveSize) void quantize_rows_kernel(const __half *__restrict__ x, int64_t ldx,
-                                                                                  int M, int K, int Kp, float clip,
-                                                                                  uint8_t *__restrict__ qact,
-                                                                                  __half *__restrict__ scale_h) {
-    const int lane = threadIdx.x & (kWaveSize - 1);
-    const int64_t row = static_cast<int64_t>(blockIdx.x) * kRowsPerBlock + (threadIdx.x >> 6);
-    if (row >= M) return;
+// FMT: 0 = native row-major int4 (Kp = K padded to the int8 GEMM's K step), 1 = bf6 blocks (Kp = K padded to 128)
+template <int NCH, bool STREAM_OUT, int ACT, int FMT>
+__global__ __launch_bounds__((FMT == 1 ? kBf6Rows : kRowsPerBlock) * kWaveSize) void quantize_rows_kernel(
+    const __half *__restrict__ x, int64_t ldx, int M, int K, int Kp, float clip, uint8_t *__restrict__ qact,
+    __half *__restrict__ scale_h) {
+    constexpr int ROWS = FMT == 1 ? kBf6Rows : kRowsPerBlock;
+    const int lane = threadIdx.x & (kWaveSize - 1), wave = threadIdx.x >> 6;
+    const int64_t row0 = static_cast<int64_t>(blockIdx.x) * ROWS;
+    int64_t row = row0 + wave;
+    const bool valid = row < M;
+    if (!valid) {
+        if (FMT == 0) return;
+        row = M - 1; /* the bf6 tail synchronises the workgroup: stay, on a copy of the last row */
+    }
     const u32x4 *src = reinterpret_cast<const u32x4 *>(x + row * ldx);
 
     u32x4 v[NCH];
@@ -225,8 +348,12 @@ __global__ __launch_bounds__(kRowsPerBlock * kWaveSize) void quantize_rows_kerne
         const int k0 = c * 512 + lane * 8;
         v[c] = k0 < K ? apply_act<ACT>(__builtin_nontemporal_load(src + c * 64 + lane)) : u32x4{0u, 0u, 0u, 0u};
     }
-
-    quantize_held_row<NCH, STREAM_OUT>(v, lane, row, Kp, clip, qact, scale_h);
+    if (FMT == 1) {
+        __shared__ __attribute__((aligned(16))) Bf6Scratch scratch;
+        quantize_held_row_bf6<NCH>(v, lane, wave, row0, valid, M, Kp, clip, qact, scale_h, scratch);
+    } else {
+        quantize_held_row<NCH, STREAM_OUT>(v, lane, row, Kp, clip, qact, scale_h);
+    }
 }
 
 __device__ __forceinline__ float wave_sum(float v) {
@@ -246,14 +373,20 @@ __device__ __forceinline__ float wave_sum(float v) {
 // Row m takes vector row m / rows_per_vec of a and b (stride ldv elements): one
 // vector per batch element, or one per token.  EMIT_H writes h itself instead of
 // quantizing it (the same arithmetic: the checker's view of h).
-template <int NCH, int LNMODE, bool EMIT_H>
-__global__ __launch_bounds__(kRowsPerBlock * kWaveSize) void ln_quantize_rows_kernel(
+template <int NCH, int LNMODE, bool EMIT_H, int FMT>
+__global__ __launch_bounds__((FMT == 1 ? kBf6Rows : kRowsPerBlock) * kWaveSize) void ln_quantize_rows_kernel(
     const __half *__restrict__ x, int64_t ldx, int M, int K, int Kp, float eps, const __half *__restrict__ va,
     const __half *__restrict__ vb, int64_t ldv, int rows_per_vec, float clip, uint8_t *__restrict__ qact,
     __half *__restrict__ scale_h, __half *__restrict__ h_out, int64_t ldh) {
-    const int lane = threadIdx.x & (kWaveSize - 1);
-    const int64_t row = static_cast<int64_t>(blockIdx.x) * kRowsPerBlock + (threadIdx.x >> 6);
-    if (row >= M) return;
+    constexpr int ROWS = FMT == 1 ? kBf6Rows : kRowsPerBlock;
+    const int lane = threadIdx.x & (kWaveSize - 1), wave = threadIdx.x >> 6;
+    const int64_t row0 = static_cast<int64_t>(blockIdx.x) * ROWS;
+    int64_t row = row0 + wave;
+    const bool valid = row < M;
+    if (!valid) {
+        if (FMT == 0) return;
+        row = M - 1; /* the bf6 tail synchronises the workgroup: stay, on a copy of the last row */
+    }
     const u32x4 *src = reinterpret_cast<const u32x4 *>(x + row * ldx);
     const int64_t vrow = (row / rows_per_vec) * ldv;
     const u32x4 *pa = reinterpret_cast<const u32x4 *>(va + vrow), *pb = reinterpret_cast<const u32x4 *>(vb + vrow);
@@ -324,7 +457,12 @@ __global__ __launch_bounds__(kRowsPerBlock * kWaveSize) void ln_quantize_rows_ke
         }
         return;
     }
-    quantize_held_row<NCH, false>(v, lane, row, Kp, clip, qact, scale_h);
+    if (FMT == 1) {
+        __shared__ __attribute__((aligned(16))) Bf6Scratch scratch;
+        quantize_held_row_bf6<NCH>(v, lane, wave, row0, valid, M, Kp, clip, qact, scale_h, scratch);
+    } else {
+        quantize_held_row<NCH, false>(v, lane, row, Kp, clip, qact, scale_h);
+    }
 }
 
 // Any K: two passes over the row (the second one is served by the caches).
@@ -380,24 +518,27 @@ __global__ __launch_bounds__(256) void quantize_given_scale_kernel(const __half 
 constexpr int64_t kStreamOutBytes = int64_t(224) << 20; /* outputs larger than this bypass the caches */
 
 template <int NCH, int ACT>
-int launch_reg(const __half *x, int64_t M, int64_t K, int64_t ldx, float clip, uint8_t *qact, __half *scale_h, hipStream_t s) {
-    const unsigned grid = static_cast<unsigned>(ceil_div(M, kRowsPerBlock));
-    if (M * (k_padded(K) / 2) > kStreamOutBytes) {
-        hipLaunchKernelGGL((quantize_rows_kernel<NCH, true, ACT>), dim3(grid), dim3(kRowsPerBlock * kWaveSize), 0, s, x, ldx,
-                           static_cast<int>(M), static_cast<int>(K), static_cast<int>(k_padded(K)), clip, qact, scale_h);
-        return check_launch("quantize_rows_kernel");
-    }
-    hipLaunchKernelGGL((quantize_rows_kernel<NCH, false, ACT>), dim3(grid), dim3(kRowsPerBlock * kWaveSize), 0, s, x, ldx,
-                       static_cast<int>(M), static_cast<int>(K), static_cast<int>(k_padded(K)), clip, qact, scale_h);
+int launch_reg(const __half *x, int64_t M, int64_t K, int64_t ldx, float clip, int fmt, uint8_t *qact, __half *scale_h, hipStream_t s) {
+    const dim3 grid(static_cast<unsigned>(ceil_div(M, kRowsPerBlock))), block(kRowsPerBlock * kWaveSize);
+    if (fmt == 1)
+        hipLaunchKernelGGL((quantize_rows_kernel<NCH, false, ACT, 1>), dim3(static_cast<unsigned>(ceil_div(M, kBf6Rows))),
+                           dim3(kBf6Rows * kWaveSize), 0, s, x, ldx, static_cast<int>(M), static_cast<int>(K),
+                           static_cast<int>(bf6_kblocks(K) * 64), clip, qact, scale_h);
+    else if (M * (k_padded(K) / 2) > kStreamOutBytes)
+        hipLaunchKernelGGL((quantize_rows_kernel<NCH, true, ACT, 0>), grid, block, 0, s, x, ldx, static_cast<int>(M), static_cast<int>(K),
+                           static_cast<int>(k_padded(K)), clip, qact, scale_h);
+    else
+        hipLaunchKernelGGL((quantize_rows_kernel<NCH, false, ACT, 0>), grid, block, 0, s, x, ldx, static_cast<int>(M), static_cast<int>(K),
+                           static_cast<int>(k_padded(K)), clip, qact, scale_h);
     return check_launch("quantize_rows_kernel");
 }
 
 template <int ACT>
-int launch_quantize_act_impl(const __half *x, int64_t M, int64_t K, int64_t ldx, float clip, uint8_t *qact, __half *scale_h,
+int launch_quantize_act_impl(const __half *x, int64_t M, int64_t K, int64_t ldx, float clip, int fmt, uint8_t *qact, __half *scale_h,
                              hipStream_t s) {
     const int64_t nch = ceil_div(k_padded(K), 512);
 #define VDMQ_CASE(n) \
-    if (nch <= n) return launch_reg<n, ACT>(x, M, K, ldx, clip, qact, scale_h, s)
+    if (nch <= n) return launch_reg<n, ACT>(x, M, K, ldx, clip, fmt, qact, scale_h, s)
     VDMQ_CASE(1);
     VDMQ_CASE(2);
     VDMQ_CASE(3);
@@ -414,6 +555,7 @@ int launch_quantize_act_impl(const __half *x, int64_t M, int64_t K, int64_t ldx,
     VDMQ_CASE(28);
     VDMQ_CASE(32);
 #undef VDMQ_CASE
+    if (fmt == 1) return fail(VDMQ_ESHAPE, "the bf6 quantizer needs K <= 16384 (got %lld)", (long long)K);
     const unsigned grid = static_cast<unsigned>(ceil_div(M, kRowsPerBlock));
     hipLaunchKernelGGL(quantize_rows_anyk_kernel<ACT>, dim3(grid), dim3(kRowsPerBlock * kWaveSize), 0, s, x, ldx, static_cast<int>(M),
                        static_cast<int>(K), static_cast<int>(k_padded(K)), clip, qact, scale_h);
@@ -422,23 +564,27 @@ int launch_quantize_act_impl(const __half *x, int64_t M, int64_t K, int64_t ldx,
 
 template <int NCH, int LNMODE>
 int launch_ln_reg(const __half *x, int64_t M, int64_t K, int64_t ldx, float eps, const __half *va, const __half *vb, int64_t ldv,
-                  int64_t rows_per_vec, float clip, uint8_t *qact, __half *scale_h, __half *h_out, int64_t ldh, hipStream_t s) {
+                  int64_t rows_per_vec, float clip, int fmt, uint8_t *qact, __half *scale_h, __half *h_out, int64_t ldh, hipStream_t s) {
     const dim3 grid(static_cast<unsigned>(ceil_div(M, kRowsPerBlock))), block(kRowsPerBlock * kWaveSize);
     if (h_out != nullptr)
-        hipLaunchKernelGGL((ln_quantize_rows_kernel<NCH, LNMODE, true>), grid, block, 0, s, x, ldx, static_cast<int>(M), static_cast<int>(K),
+        hipLaunchKernelGGL((ln_quantize_rows_kernel<NCH, LNMODE, true, 0>), grid, block, 0, s, x, ldx, static_cast<int>(M), static_cast<int>(K),
                            static_cast<int>(k_padded(K)), eps, va, vb, ldv, static_cast<int>(rows_per_vec), clip, qact, scale_h, h_out, ldh);
+    else if (fmt == 1)
+        hipLaunchKernelGGL((ln_quantize_rows_kernel<NCH, LNMODE, false, 1>), dim3(static_cast<unsigned>(ceil_div(M, kBf6Rows))),
+                           dim3(kBf6Rows * kWaveSize), 0, s, x, ldx, static_cast<int>(M), static_cast<int>(K),
+                           static_cast<int>(bf6_kblocks(K) * 64), eps, va, vb, ldv, static_cast<int>(rows_per_vec), clip, qact, scale_h, h_out, ldh);
     else
-        hipLaunchKernelGGL((ln_quantize_rows_kernel<NCH, LNMODE, false>), grid, block, 0, s, x, ldx, static_cast<int>(M), static_cast<int>(K),
+        hipLaunchKernelGGL((ln_quantize_rows_kernel<NCH, LNMODE, false, 0>), grid, block, 0, s, x, ldx, static_cast<int>(M), static_cast<int>(K),
                            static_cast<int>(k_padded(K)), eps, va, vb, ldv, static_cast<int>(rows_per_vec), clip, qact, scale_h, h_out, ldh);
     return check_launch("ln_quantize_rows_kernel");
 }
 
 template <int LNMODE>
 int launch_ln_impl(const __half *x, int64_t M, int64_t K, int64_t ldx, float eps, const __half *va, const __half *vb, int64_t ldv,
-                   int64_t rows_per_vec, float clip, uint8_t *qact, __half *scale_h, __half *h_out, int64_t ldh, hipStream_t s) {
+                   int64_t rows_per_vec, float clip, int fmt, uint8_t *qact, __half *scale_h, __half *h_out, int64_t ldh, hipStream_t s) {
     const int64_t nch = ceil_div(k_padded(K), 512);
 #define VDMQ_CASE(n) \
-    if (nch <= n) return launch_ln_reg<n, LNMODE>(x, M, K, ldx, eps, va, vb, ldv, rows_per_vec, clip, qact, scale_h, h_out, ldh, s)
+    if (nch <= n) return launch_ln_reg<n, LNMODE>(x, M, K, ldx, eps, va, vb, ldv, rows_per_vec, clip, fmt, qact, scale_h, h_out, ldh, s)
     VDMQ_CASE(1);
     VDMQ_CASE(2);
     VDMQ_CASE(3);
@@ -462,20 +608,20 @@ __global__ __launch_bounds__(256) void gelu_tanh_kernel(const uint32_t *__restri
 
 }  // namespace
 
-int launch_quantize_act(const __half *x, int64_t M, int64_t K, int64_t ldx, float clip, int act, uint8_t *qact, __half *scale_h,
-                        hipStream_t s) {
+int launch_quantize_act(const __half *x, int64_t M, int64_t K, int64_t ldx, float clip, int act, int fmt, uint8_t *qact,
+                        __half *scale_h, hipStream_t s) {
     if (M == 0) return VDMQ_OK;
-    if (act == VDMQ_ACT_GELU_TANH) return launch_quantize_act_impl<VDMQ_ACT_GELU_TANH>(x, M, K, ldx, clip, qact, scale_h, s);
-    return launch_quantize_act_impl<VDMQ_ACT_NONE>(x, M, K, ldx, clip, qact, scale_h, s);
+    if (act == VDMQ_ACT_GELU_TANH) return launch_quantize_act_impl<VDMQ_ACT_GELU_TANH>(x, M, K, ldx, clip, fmt, qact, scale_h, s);
+    return launch_quantize_act_impl<VDMQ_ACT_NONE>(x, M, K, ldx, clip, fmt, qact, scale_h, s);
 }
 
 int launch_ln_quantize(const __half *x, int64_t M, int64_t K, int64_t ldx, float eps, int ln_mode, const __half *va, const __half *vb,
-                       int64_t ldv, int64_t rows_per_vec, float clip, uint8_t *qact, __half *scale_h, __half *h_out, int64_t ldh,
+                       int64_t ldv, int64_t rows_per_vec, float clip, int fmt, uint8_t *qact, __half *scale_h, __half *h_out, int64_t ldh,
                        hipStream_t s) {
     if (M == 0) return VDMQ_OK;
     if (ln_mode == VDMQ_LN_MODULATE)
-        return launch_ln_impl<VDMQ_LN_MODULATE>(x, M, K, ldx, eps, va, vb, ldv, rows_per_vec, clip, qact, scale_h, h_out, ldh, s);
-    return launch_ln_impl<VDMQ_LN_AFFINE>(x, M, K, ldx, eps, va, vb, ldv, rows_per_vec, clip, qact, scale_h, h_out, ldh, s);
+        return launch_ln_impl<VDMQ_LN_MODULATE>(x, M, K, ldx, eps, va, vb, ldv, rows_per_vec, clip, fmt, qact, scale_h, h_out, ldh, s);
+    return launch_ln_impl<VDMQ_LN_AFFINE>(x, M, K, ldx, eps, va, vb, ldv, rows_per_vec, clip, fmt, qact, scale_h, h_out, ldh, s);
 }
 
 int launch_gelu_tanh(const __half *x, __half *y, int64_t n, hipStream_t s) {

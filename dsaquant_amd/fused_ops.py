@@ -98,12 +98,16 @@ class LnInput:
                 _lib.check(lib.vdmq_ln_f16(*self._args(), h.data_ptr(), h.stride(0), _k._stream(h.device)))
         return h.view(self.shape)
 
-    def quantize(self, clip_ratio: float = 1.0):
-        """``(qact native, scales)`` of the produced input, as ``quantize_activation_native`` returns them."""
+    def quantize(self, clip_ratio: float = 1.0, bf6: bool = False):
+        """``(qact native, scales)`` of the produced input, as ``quantize_activation_native`` returns them
+        (``bf6=True``: as ``quantize_activation_bf6`` does)."""
         lib = _k._load_ext()
         _k._check_device_tensor(self.x, "input", torch.float16)
         M, K = self.x.shape
         dev = self.x.device
+        if bf6:
+            with torch.cuda.device(dev):
+                return _k._quantize_for_gemm(self.x, clip_ratio, 0, True, self._args())
         with torch.cuda.device(dev):
             native = torch.empty((M, _k.k_padded(K) // 2), dtype=torch.uint8, device=dev)
             scales = torch.empty((M,), dtype=torch.float16, device=dev)
@@ -183,15 +187,9 @@ def linear_fused(
     with torch.cuda.device(dev):
         out = torch.empty((M, N), dtype=torch.float16, device=dev)
         if M:
-            s = _k._stream(dev)
-            qact = torch.empty((M, _k.k_padded(K) // 2), dtype=torch.uint8, device=dev)
-            scales = torch.empty((M,), dtype=torch.float16, device=dev)
-            if pre is not None:
-                _lib.check(lib.vdmq_quantize_act_ln(*pre._args(), float(clip_ratio), qact.data_ptr(), scales.data_ptr(), s))
-            else:
-                _lib.check(lib.vdmq_quantize_act_ex(x_2d.data_ptr(), M, K, x_2d.stride(0), float(clip_ratio), act_code, qact.data_ptr(),
-                                                    scales.data_ptr(), s))
-            _k._gemm_dispatch(qact, scales, native_w, wscale, b, out, K, gate=g2, rows_per_gate=rows_per_gate, residual=r2)
+            bf6 = _k._use_bf6(M, N, K)
+            operand, scales = _k._quantize_for_gemm(x_2d, clip_ratio, act_code, bf6, None if pre is None else pre._args())
+            _k._gemm_dispatch(operand, scales, bf6, native_w, wscale, b, out, K, gate=g2, rows_per_gate=rows_per_gate, residual=r2)
     return out.view(*lead, N)
 
 

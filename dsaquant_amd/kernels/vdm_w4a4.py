@@ -191,10 +191,35 @@ def _bf6_weights(native_w: torch.Tensor, K: int) -> torch.Tensor:
     return hit
 
 
-def _gemm_dispatch(qact: torch.Tensor, scales: torch.Tensor, native_w: torch.Tensor, wscale: torch.Tensor, bias: Optional[torch.Tensor],
-                   out: torch.Tensor, K: int, gate: Optional[torch.Tensor] = None, rows_per_gate: int = 1,
+def _quantize_for_gemm(x_2d: torch.Tensor, clip_ratio: float, act_code: int, bf6: bool, ln_args: Optional[tuple] = None):
+    """Quantize the rows of ``x_2d`` (optionally through a fused activation, or the fused LayerNorm described by
+    ``ln_args`` = the leading arguments of vdmq_quantize_act_ln) into the operand form of the chosen matrix path:
+    bf6 blocks or native int4 rows.  Returns ``(operand, scales)``.  Must run under ``torch.cuda.device(...)``."""
+    lib = _load_ext()
+    M, K = x_2d.shape
+    dev = x_2d.device
+    s = _stream(dev)
+    scales = torch.empty((M,), dtype=torch.float16, device=dev)
+    direct = bf6 and K <= 16384  # the quantizer writes bf6 blocks itself
+    if direct:
+        op = torch.empty((int(lib.vdmq_bf6_bytes(M, K)),), dtype=torch.uint8, device=dev)
+    else:
+        op = torch.empty((M, k_padded(K) // 2), dtype=torch.uint8, device=dev)
+    if ln_args is not None:
+        fn = lib.vdmq_quantize_act_ln_bf6 if direct else lib.vdmq_quantize_act_ln
+        _lib.check(fn(*ln_args, float(clip_ratio), op.data_ptr(), scales.data_ptr(), s))
+    else:
+        fn = lib.vdmq_quantize_act_bf6 if direct else lib.vdmq_quantize_act_ex
+        _lib.check(fn(x_2d.data_ptr(), M, K, x_2d.stride(0), float(clip_ratio), act_code, op.data_ptr(), scales.data_ptr(), s))
+    if bf6 and not direct:
+        op = _to_bf6(op, M, K)
+    return op, scales
+
+
+def _gemm_dispatch(operand: torch.Tensor, scales: torch.Tensor, bf6: bool, native_w: torch.Tensor, wscale: torch.Tensor,
+                   bias: Optional[torch.Tensor], out: torch.Tensor, K: int, gate: Optional[torch.Tensor] = None, rows_per_gate: int = 1,
                    residual: Optional[torch.Tensor] = None) -> None:
-    """GEMM + epilogue on a quantized activation (native layout) into ``out`` on the chosen matrix path.
+    """GEMM + epilogue on a quantized activation (bf6 blocks if ``bf6`` else native rows) into ``out``.
     Must run under ``torch.cuda.device(out.device)``."""
     lib = _load_ext()
     M, N = out.shape
@@ -202,14 +227,13 @@ def _gemm_dispatch(qact: torch.Tensor, scales: torch.Tensor, native_w: torch.Ten
     bias_p = None if bias is None else bias.data_ptr()
     gate_p, ldg = (None, 0) if gate is None else (gate.data_ptr(), gate.stride(0))
     res_p, ldr = (None, 0) if residual is None else (residual.data_ptr(), residual.stride(0))
-    if _use_bf6(M, N, K, out.dtype):
+    if bf6:
         wblocks = _bf6_weights(native_w, K)
-        xblocks = _to_bf6(qact, M, K)
-        _lib.check(lib.vdmq_gemm_w4a4_bf6_ex(xblocks.data_ptr(), scales.data_ptr(), wblocks.data_ptr(), wscale.data_ptr(), bias_p, gate_p, ldg,
+        _lib.check(lib.vdmq_gemm_w4a4_bf6_ex(operand.data_ptr(), scales.data_ptr(), wblocks.data_ptr(), wscale.data_ptr(), bias_p, gate_p, ldg,
                                              rows_per_gate, res_p, ldr, out.data_ptr(), M, N, K, out.stride(0), s))
         return
     code = _lib.VDMQ_OUT_F16 if out.dtype == torch.float16 else _lib.VDMQ_OUT_BF16
-    _lib.check(lib.vdmq_gemm_w4a4_ex(qact.data_ptr(), scales.data_ptr(), native_w.data_ptr(), wscale.data_ptr(), bias_p, gate_p, ldg,
+    _lib.check(lib.vdmq_gemm_w4a4_ex(operand.data_ptr(), scales.data_ptr(), native_w.data_ptr(), wscale.data_ptr(), bias_p, gate_p, ldg,
                                      rows_per_gate, res_p, ldr, out.data_ptr(), code, M, N, K, out.stride(0), s))
 
 
@@ -287,11 +311,9 @@ def _linear_2d(x_2d: torch.Tensor, native_w: torch.Tensor, wscale: torch.Tensor,
         out = torch.empty((M, N), dtype=out_dtype, device=dev)
         if M == 0:
             return out
-        qact = torch.empty((M, k_padded(K) // 2), dtype=torch.uint8, device=dev)
-        scales = torch.empty((M,), dtype=torch.float16, device=dev)
-        _lib.check(lib.vdmq_quantize_act_ex(x_2d.data_ptr(), M, K, x_2d.stride(0), float(clip_ratio), _act_code(act), qact.data_ptr(),
-                                            scales.data_ptr(), _stream(dev)))
-        _gemm_dispatch(qact, scales, native_w, wscale, bias, out, K)
+        bf6 = _use_bf6(M, N, K, out_dtype)
+        operand, scales = _quantize_for_gemm(x_2d, clip_ratio, _act_code(act), bf6)
+        _gemm_dispatch(operand, scales, bf6, native_w, wscale, bias, out, K)
     return out
 
 
@@ -358,6 +380,17 @@ def quantize_activation_native(x: torch.Tensor, clip_ratio: float = 1.0, act: Op
     return native, act_scales
 
 
+def quantize_activation_bf6(x: torch.Tensor, clip_ratio: float = 1.0, act: Optional[str] = None):
+    """The quantizer writing the bf6 GEMM's operand form directly: ``(blocks u8 [vdmq_bf6_bytes(M, K)], scales fp16 [M])``
+    -- the same integers and scales as ``quantize_activation_native``; rows of the last 32-row block beyond M are unspecified."""
+    _load_ext()
+    x_2d, _ = _as_2d_half_contiguous(x)
+    _check_device_tensor(x_2d, "input", torch.float16)
+    _require(x_2d.shape[1] % WARP_K == 0, f"K must be a multiple of {WARP_K}")
+    with torch.cuda.device(x_2d.device):
+        return _quantize_for_gemm(x_2d, clip_ratio, _act_code(act), True)
+
+
 def linear_prequantized(qact: torch.Tensor, ascales: torch.Tensor, qweight: torch.Tensor, wscales: torch.Tensor) -> torch.Tensor:
     """GEMM only, on v1-layout activations already padded to BLOCK_M rows; no
     bias (vdm_w4a4.py:253-256 / vdm_w4a4_kernel.cu:876-918)."""
@@ -386,7 +419,8 @@ def linear_prequantized(qact: torch.Tensor, ascales: torch.Tensor, qweight: torc
         native = torch.empty((M, k_padded(K) // 2), dtype=torch.uint8, device=dev)
         scales = torch.empty((M,), dtype=torch.float16, device=dev)
         _lib.check(lib.vdmq_act_v1_to_native(qact.data_ptr(), ascales.data_ptr(), M, K, native.data_ptr(), scales.data_ptr(), s))
-        _gemm_dispatch(native, scales, native_w, wscale, None, out, K)
+        bf6 = _use_bf6(M, N, K)
+        _gemm_dispatch(_to_bf6(native, M, K) if bf6 else native, scales, bf6, native_w, wscale, None, out, K)
     return out
 
 

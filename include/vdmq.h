@@ -176,8 +176,15 @@ int vdmq_linear_ln_w4a4(const void *x, int64_t M, int64_t K, int64_t ldx, float 
  * (vdmq_bf6_bytes gives the size).  vdmq_native_to_bf6 converts a native int4
  * buffer (weights once per module; activations per call unless the quantizer
  * writes blocks itself); vdmq_gemm_w4a4_bf6 is vdmq_gemm_w4a4 on such operands
- * (fp16 output only), vdmq_gemm_w4a4_bf6_acc the int32 accumulator view. */
+ * (fp16 output only), vdmq_gemm_w4a4_bf6_acc the int32 accumulator view.
+ * vdmq_quantize_act_bf6 / vdmq_quantize_act_ln_bf6 are vdmq_quantize_act_ex /
+ * vdmq_quantize_act_ln writing bf6 blocks (xblocks, vdmq_bf6_bytes(M, K) bytes)
+ * instead of native rows: same scales, same integers; K <= 16384. */
 int64_t vdmq_bf6_bytes(int64_t rows, int64_t K);
+int vdmq_quantize_act_bf6(const void *x, int64_t M, int64_t K, int64_t ldx, float clip, int act, void *xblocks, void *scale_h,
+                          vdmq_stream_t stream);
+int vdmq_quantize_act_ln_bf6(const void *x, int64_t M, int64_t K, int64_t ldx, float eps, int ln_mode, const void *a, const void *b,
+                             int64_t ldv, int64_t rows_per_vec, float clip, void *xblocks, void *scale_h, vdmq_stream_t stream);
 int vdmq_native_to_bf6(const void *native, int64_t rows, int64_t K, void *blocks, vdmq_stream_t stream);
 int vdmq_gemm_w4a4_bf6(const void *xblocks, const void *ascale, const void *wblocks, const void *wscale, const void *bias, void *out,
                        int64_t M, int64_t N, int64_t K, int64_t ldo, vdmq_stream_t stream);

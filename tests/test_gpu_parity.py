@@ -539,6 +539,45 @@ def test_bf6_blocks_hold_the_quantized_values(M, K):
     assert np.array_equal(O.np_unpack_bf6_blocks(blocks, M, K), want.astype(np.float64))
 
 
+def rows_of_blocks(blocks: torch.Tensor, M: int, K: int) -> np.ndarray:
+    """Decode a bf6 block buffer whose rows beyond M (in the last 32-row block) are unspecified."""
+    b = blocks.cpu().numpy().reshape((M + 31) // 32, -1, 1536).copy()
+    if M % 32:
+        lanes = np.arange(64) % 32 >= M % 32  # slots of rows beyond M
+        b[-1, :, :1024].reshape(-1, 64, 16)[:, lanes] = 0
+        b[-1, :, 1024:].reshape(-1, 64, 8)[:, lanes] = 0
+    return O.np_unpack_bf6_blocks(b.reshape(-1), M, K)
+
+
+@pytest.mark.parametrize("M,K", [(257, 1536), (100, 64), (77, 192), (515, 5120), (130, 13824), (19, 16384), (4096, 8960), (33, 3072)])
+def test_bf6_quantizers_write_the_oracle_integers(M, K):
+    """The quantizers that emit bf6 blocks directly (plain, GELU, LayerNorm): decoded with the format's definition,
+    the blocks hold the oracle's integers (plain) / the integers of the int4 quantizer (fused producers), scales equal."""
+    from dsaquant_amd import fused_ops
+
+    v = vk()
+    x = special_rows((2.0 * O.synth_linear(M, K, 128, seed=M + K)[0].astype(np.float32)).astype(np.float16))
+    print(f"bf6 quantizers M={M} K={K}", flush=True)
+    for clip in (1.0, 0.95):
+        blocks, sc = v.quantize_activation_bf6(t16(x), clip)
+        want_s = O.np_row_scale(x, clip)
+        assert np.array_equal(sc.cpu().numpy().view(np.uint16), want_s.view(np.uint16))
+        assert np.array_equal(rows_of_blocks(blocks, M, K), O.np_quantize_rows(x, want_s).astype(np.float64))
+    blocks, sc = v.quantize_activation_bf6(t16(x), 1.0, act="gelu_tanh")
+    qn, sc4 = v.quantize_activation_native(t16(x), 1.0, act="gelu_tanh")
+    assert torch.equal(sc.view(torch.int16), sc4.view(torch.int16))
+    assert np.array_equal(rows_of_blocks(blocks, M, K), unpack_native(qn.cpu().numpy(), K).astype(np.float64))
+    rng = np.random.default_rng(M)
+    a, b = (0.2 * rng.standard_normal((1, K))).astype(np.float16), (0.3 * rng.standard_normal((1, K))).astype(np.float16)
+    xf = np.where(np.isfinite(x), x, np.float16(1.0))
+    for mode in ("modulate", "affine"):
+        pre = fused_ops.LnInput(t16(xf), t16(a), t16(b), 1e-6, mode)
+        blocks, sc = pre.quantize(0.95, bf6=True)
+        qn, sc4 = pre.quantize(0.95)
+        assert torch.equal(sc.view(torch.int16), sc4.view(torch.int16))
+        assert np.array_equal(rows_of_blocks(blocks, M, K), unpack_native(qn.cpu().numpy(), K).astype(np.float64))
+
+
 @pytest.mark.parametrize("M,N,K", [(257, 1536, 1536), (1, 128, 64), (300, 128, 8960), (700, 384, 13824), (4100, 8320, 640), (8200, 8320, 2304)])
 def test_bf6_accumulators_exact(M, N, K):
     v = vk()
