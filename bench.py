@@ -12,9 +12,14 @@ timed region.  Prints ONE JSON line.
              (quantizer time included)
   roofline   the GEMM kernel alone (HIP events around its launches):
              algorithmic ops 2*M*N*K per launch / average launch duration,
-             against the dense INT8 MFMA peak of 5.0 POP/s
-  quantizer  the A4 quantizer alone: algorithmic bytes 2*M*K + M*K/2 + 2*M per
-             launch / average launch duration, against the 8 TB/s HBM3E peak
+             against the peak of the matrix instructions it runs on: the bf6
+             path (v_mfma_f32_32x32x64_f8f6f4, what the library picks for
+             shapes this large) 10.1 PFLOP/s dense FP6, --matrix-path int8
+             (v_mfma_i32_32x32x32_i8) 5.0 POP/s dense INT8; the fraction of the
+             INT8 peak is reported next to it in either case
+  quantizer  the A4 quantizer alone: algorithmic bytes per launch (fp16 in,
+             int4 rows or 6-bit blocks + one fp16 scale per row out) / average
+             launch duration, against the 8 TB/s HBM3E peak
   cpu_baseline  the torch QuantLinear floating-point path (oracle/quantlinear_torch.py,
              a restatement of the reference's CPU-runnable path) on config 0
 """
@@ -32,13 +37,14 @@ ROOT = Path(__file__).resolve().parent
 sys.path.insert(0, str(ROOT))
 
 INT8_PEAK_TOPS = 5000.0  # MI355X dense INT8 MFMA, published
+FP6_PEAK_TOPS = 10100.0  # MI355X dense FP6 MFMA, published
 # HBM bytes per launch of the dominant kernels on the default workload, from rocprofv3 --pmc FETCH_SIZE and
 # WRITE_SIZE runs of this program (mean over the four launches of a step; the summary with the scaling by
 # the copy kernel's readings is profiles/gemm_w4a4_kernel+quantize_rows_kernel.wan14b_720p_block.md)
 # gemm: (FETCH_SIZE 1373495 KiB x 2.0 + WRITE_SIZE 1455416 KiB x 1.0) x 1024; the reads are requests leaving L2
 # (Infinity Cache or HBM), 9x the operand bytes because every XCD fetches most of its super-tile's slabs once.
 # quant: (FETCH_SIZE 538736 KiB x 2.0 + WRITE_SIZE 269920 KiB x 1.0) x 1024 = 1.0005 x the algorithmic bytes.
-MEASURED_TRAFFIC = {"wan14b_720p_block": {"gemm": 4303263744, "quant": 1379729408}}
+MEASURED_TRAFFIC = {("wan14b_720p_block", "int8"): {"gemm": 4303263744, "quant": 1379729408}}
 HBM_PEAK_GBS = 8000.0    # MI355X HBM3E, published
 
 # (name, K, N) at M tokens
@@ -48,7 +54,9 @@ WAN5B = dict(M=27280, linears=[("qkv", 3072, 9216), ("o", 3072, 3072), ("ffn_up"
 WORKLOADS = {"wan14b_720p_block": WAN14B_720P, "wan1.3b_480p_block": WAN13B_480P, "wan5b_704x1280_block": WAN5B}
 
 
-def quant_bytes(M, K):
+def quant_bytes(M, K, bf6=False):
+    if bf6:  # 6-bit codes, K padded to 128
+        return 2 * M * K + M * (-(-K // 128) * 128) * 3 // 4 + 2 * M
     return 2 * M * K + M * K // 2 + 2 * M
 
 
@@ -108,6 +116,8 @@ def main():
     ap.add_argument("--steps", type=int, default=20)
     ap.add_argument("--warmup", type=int, default=5)
     ap.add_argument("--workload", default="wan14b_720p_block", choices=sorted(WORKLOADS))
+    ap.add_argument("--matrix-path", default="auto", choices=["auto", "int8", "bf6"],
+                    help="matrix instructions of the GEMM: auto = what the library picks for the shape")
     ap.add_argument("--no-cpu-baseline", action="store_true")
     ap.add_argument("--calibrate-copy", action="store_true",
                     help="also run the library's plain 1 GiB copy kernel three times first, so that a rocprofv3 --pmc FETCH_SIZE / WRITE_SIZE "
@@ -138,27 +148,43 @@ def main():
         torch.cuda.synchronize()
         del src, dst
 
+    v.set_matrix_path(args.matrix_path)
+    stream = torch.cuda.current_stream(dev)
+    s = stream.cuda_stream
     layers = []
     for i, (name, K, N) in enumerate(wl["linears"]):
         x, wq, ws, bias = synth_inputs(torch, M, K, N, seed=i, dev=dev)
         Kp = v.k_padded(K)
         assert Kp == K
-        layers.append(dict(name=name, K=K, N=N, x=x, wq=wq, ws=ws, bias=bias,
-                           qact=torch.empty((M, Kp // 2), dtype=torch.uint8, device=dev),
+        bf6 = v._use_bf6(M, N, K)
+        if bf6:  # operands of the bf6 path: 6-bit blocks (weights converted once, like a module's cache does)
+            wblocks = torch.empty(int(lib.vdmq_bf6_bytes(N, K)), dtype=torch.uint8, device=dev)
+            _lib.check(lib.vdmq_native_to_bf6(wq.data_ptr(), N, K, wblocks.data_ptr(), s))
+            wq = wblocks
+            qact = torch.empty(int(lib.vdmq_bf6_bytes(M, K)), dtype=torch.uint8, device=dev)
+        else:
+            qact = torch.empty((M, Kp // 2), dtype=torch.uint8, device=dev)
+        layers.append(dict(name=name, K=K, N=N, x=x, wq=wq, ws=ws, bias=bias, bf6=bf6, qact=qact,
                            scale=torch.empty((M,), dtype=torch.float16, device=dev),
                            out=torch.empty((M, N), dtype=torch.float16, device=dev)))
-    stream = torch.cuda.current_stream(dev)
-    s = stream.cuda_stream
+    torch.cuda.synchronize()
 
     def run_step(events=None):
         for li, L in enumerate(layers):
             if events is not None:
                 events[li][0].record(stream)
-            _lib.check(lib.vdmq_quantize_act(L["x"].data_ptr(), M, L["K"], L["K"], 1.0, L["qact"].data_ptr(), L["scale"].data_ptr(), s))
+            if L["bf6"]:
+                _lib.check(lib.vdmq_quantize_act_bf6(L["x"].data_ptr(), M, L["K"], L["K"], 1.0, 0, L["qact"].data_ptr(), L["scale"].data_ptr(), s))
+            else:
+                _lib.check(lib.vdmq_quantize_act(L["x"].data_ptr(), M, L["K"], L["K"], 1.0, L["qact"].data_ptr(), L["scale"].data_ptr(), s))
             if events is not None:
                 events[li][1].record(stream)
-            _lib.check(lib.vdmq_gemm_w4a4(L["qact"].data_ptr(), L["scale"].data_ptr(), L["wq"].data_ptr(), L["ws"].data_ptr(),
-                                          L["bias"].data_ptr(), L["out"].data_ptr(), _lib.VDMQ_OUT_F16, M, L["N"], L["K"], L["N"], s))
+            if L["bf6"]:
+                _lib.check(lib.vdmq_gemm_w4a4_bf6(L["qact"].data_ptr(), L["scale"].data_ptr(), L["wq"].data_ptr(), L["ws"].data_ptr(),
+                                                  L["bias"].data_ptr(), L["out"].data_ptr(), M, L["N"], L["K"], L["N"], s))
+            else:
+                _lib.check(lib.vdmq_gemm_w4a4(L["qact"].data_ptr(), L["scale"].data_ptr(), L["wq"].data_ptr(), L["ws"].data_ptr(),
+                                              L["bias"].data_ptr(), L["out"].data_ptr(), _lib.VDMQ_OUT_F16, M, L["N"], L["K"], L["N"], s))
             if events is not None:
                 events[li][2].record(stream)
 
@@ -185,28 +211,38 @@ def main():
         quant_ms_sum += q_ms
         per_layer[L["name"]] = {
             "K": L["K"], "N": L["N"], "gemm_ms": round(g_ms, 4), "gemm_tops": round(2.0 * M * L["N"] * L["K"] / g_ms / 1e9, 1),
-            "quant_ms": round(q_ms, 4), "quant_gbs": round(quant_bytes(M, L["K"]) / q_ms / 1e6, 1),
+            "quant_ms": round(q_ms, 4), "quant_gbs": round(quant_bytes(M, L["K"], L["bf6"]) / q_ms / 1e6, 1),
+            "matrix_path": "bf6" if L["bf6"] else "int8",
         }
     gemm_tops = total_ops / gemm_ms_sum / 1e9
-    quant_gbs = sum(quant_bytes(M, L["K"]) for L in layers) / quant_ms_sum / 1e6
+    quant_gbs = sum(quant_bytes(M, L["K"], L["bf6"]) for L in layers) / quant_ms_sum / 1e6
+    paths = sorted({"bf6" if L["bf6"] else "int8" for L in layers})
+    path = paths[0] if len(paths) == 1 else "mixed"
+    # a step that mixes both kinds of launches is priced against the higher peak
+    peak = INT8_PEAK_TOPS if path == "int8" else FP6_PEAK_TOPS
+    gemm_kernel = {"int8": "gemm_w4a4_kernel", "bf6": "gemm_bf6_kernel"}.get(path, "gemm_w4a4_kernel + gemm_bf6_kernel")
+    traffic = MEASURED_TRAFFIC.get((args.workload, path), {})
     value = total_ops / (ms_per_step * 1e-3) / 1e12
 
     result = {
         "metric": "W4A4 GEMM TOPS (% INT8-MFMA peak) at Wan-14B 720p shapes; A4-quant GB/s",
         "value": round(value, 1), "unit": "TOPS", "n_gpus": 1, "steps": args.steps, "warmup": args.warmup,
         "ms_per_step": round(ms_per_step, 4), "higher_is_better": True, "scaling": "weak", "vs_baseline": None,
-        "dtype": "int4 x int4 -> int32 (int8 MFMA), fp16 in/out", "data": "synthetic",
+        "dtype": ("int4 x int4 -> int32 (int8 MFMA), fp16 in/out" if path == "int8" else
+                  "int4 x int4 as exact E3M2 floats -> fp32 accumulator holding the exact integer (FP6 MFMA), fp16 in/out"),
+        "data": "synthetic", "matrix_path": path,
         "config": {"workload": f"{args.workload}: M={M} tokens, linears " + ", ".join(f"{n} {k}->{o}" for n, k, o in wl["linears"])
                                + "; each = A4 quantizer + W4A4 GEMM + scale/bias epilogue, clip 1.0"},
-        "roofline": {"bound": "mfma", "achieved": round(gemm_tops, 1), "peak": INT8_PEAK_TOPS, "unit": "TOP/s",
-                     "frac": round(gemm_tops / INT8_PEAK_TOPS, 4), "traffic": MEASURED_TRAFFIC.get(args.workload, {}).get("gemm"),
-                     "traffic_unit": "HBM bytes per launch (mean of the step's four launches)", "kernel": "gemm_w4a4_kernel",
+        "roofline": {"bound": "mfma", "achieved": round(gemm_tops, 1), "peak": peak, "unit": "TOP/s",
+                     "frac": round(gemm_tops / peak, 4), "frac_of_int8_peak": round(gemm_tops / INT8_PEAK_TOPS, 4),
+                     "traffic": traffic.get("gemm"),
+                     "traffic_unit": "HBM bytes per launch (mean of the step's four launches)", "kernel": gemm_kernel,
                      "algorithmic_ops_per_launch": total_ops / len(layers),
                      "avg_launch_ms": round(gemm_ms_sum / len(layers), 4)},
         "quantizer": {"bound": "hbm", "achieved": round(quant_gbs, 1), "peak": HBM_PEAK_GBS, "unit": "GB/s",
-                      "frac": round(quant_gbs / HBM_PEAK_GBS, 4), "traffic": MEASURED_TRAFFIC.get(args.workload, {}).get("quant"),
+                      "frac": round(quant_gbs / HBM_PEAK_GBS, 4), "traffic": traffic.get("quant"),
                       "traffic_unit": "HBM bytes per launch (mean of the step's four launches)", "kernel": "quantize_rows_kernel",
-                      "algorithmic_bytes_per_launch": sum(quant_bytes(M, L["K"]) for L in layers) / len(layers),
+                      "algorithmic_bytes_per_launch": sum(quant_bytes(M, L["K"], L["bf6"]) for L in layers) / len(layers),
                       "avg_launch_ms": round(quant_ms_sum / len(layers), 4)},
         "per_linear": per_layer,
     }

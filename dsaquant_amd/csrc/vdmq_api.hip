@@ -333,6 +333,28 @@ int vdmq_gemm_w4a4_bf6_acc(const void *xblocks, const void *wblocks, int32_t *ac
     return gemm_bf6_checked(xblocks, nullptr, wblocks, nullptr, nullptr, nullptr, acc, M, N, K, N, GemmTail{}, stream);
 }
 
+int64_t vdmq_workspace_bytes_bf6(int64_t M, int64_t K) {
+    if (M < 0 || K <= 0) return 0;
+    return (bf6_bytes(M, K) + 255) / 256 * 256 + (M * 2 + 255) / 256 * 256;
+}
+
+int vdmq_linear_w4a4_bf6(const void *x, int64_t M, int64_t K, int64_t ldx, float clip, int act, const void *wblocks, const void *wscale,
+                         const void *bias, void *out, int64_t N, int64_t ldo, void *workspace, int64_t workspace_bytes,
+                         vdmq_stream_t stream) {
+    VDMQ_TRY(check_k(K));
+    VDMQ_TRY(check_n(N));
+    VDMQ_TRY(check_m(M));
+    if (M == 0) return VDMQ_OK;
+    VDMQ_TRY(check_ptr(workspace, "workspace"));
+    if (workspace_bytes < vdmq_workspace_bytes_bf6(M, K))
+        return fail(VDMQ_ENOSPACE, "workspace has %lld bytes, %lld needed", (long long)workspace_bytes,
+                    (long long)vdmq_workspace_bytes_bf6(M, K));
+    uint8_t *xblocks = static_cast<uint8_t *>(workspace);
+    void *scale = xblocks + (bf6_bytes(M, K) + 255) / 256 * 256;
+    VDMQ_TRY(vdmq_quantize_act_bf6(x, M, K, ldx, clip, act, xblocks, scale, stream));
+    return vdmq_gemm_w4a4_bf6(xblocks, scale, wblocks, wscale, bias, out, M, N, K, ldo, stream);
+}
+
 int vdmq_weight_v1_to_native(const void *qweight_v1, void *wq_native, int64_t N, int64_t K, vdmq_stream_t stream) {
     VDMQ_TRY(check_k(K));
     VDMQ_TRY(check_n(N));

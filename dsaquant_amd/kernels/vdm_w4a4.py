@@ -144,9 +144,11 @@ def clear_native_cache() -> None:
 # "int8": v_mfma_i32_32x32x32_i8 on nibbles widened in registers.  "bf6": v_mfma_f32_32x32x64_f8f6f4 on 6-bit
 # floats (twice the rate, no widening work; every int4 value is exact in E3M2, so is the fp32 accumulation).
 # Both give bit-identical results.  "auto" takes bf6 where it is faster: problems with at least
-# _BF6_MIN_TILES 256 x 256 output tiles (its kernel has that one tile shape).
+# _BF6_MIN_TILES 256 x 256 output tiles (its kernel has that one tile shape; measured on the Wan shapes:
+# +17 % per 14B block, +14 % per 5B block, and at 768 tiles -- Wan-1.3B o-proj -- the int8 kernel's 256 x 128
+# configuration still wins).
 _MATRIX_PATH = os.environ.get("VDMQ_MATRIX_PATH", "auto")
-_BF6_MIN_TILES = 512
+_BF6_MIN_TILES = 1024
 
 
 def set_matrix_path(name: str) -> None:

@@ -185,6 +185,12 @@ int vdmq_quantize_act_bf6(const void *x, int64_t M, int64_t K, int64_t ldx, floa
                           vdmq_stream_t stream);
 int vdmq_quantize_act_ln_bf6(const void *x, int64_t M, int64_t K, int64_t ldx, float eps, int ln_mode, const void *a, const void *b,
                              int64_t ldv, int64_t rows_per_vec, float clip, void *xblocks, void *scale_h, vdmq_stream_t stream);
+/* vdmq_linear_w4a4_ex on the bf6 path: quantizer writing blocks + bf6 GEMM; wblocks = vdmq_native_to_bf6 of the
+ * native weights; workspace of vdmq_workspace_bytes_bf6(M, K) bytes. */
+int64_t vdmq_workspace_bytes_bf6(int64_t M, int64_t K);
+int vdmq_linear_w4a4_bf6(const void *x, int64_t M, int64_t K, int64_t ldx, float clip, int act, const void *wblocks, const void *wscale,
+                         const void *bias, void *out, int64_t N, int64_t ldo, void *workspace, int64_t workspace_bytes,
+                         vdmq_stream_t stream);
 int vdmq_native_to_bf6(const void *native, int64_t rows, int64_t K, void *blocks, vdmq_stream_t stream);
 int vdmq_gemm_w4a4_bf6(const void *xblocks, const void *ascale, const void *wblocks, const void *wscale, const void *bias, void *out,
                        int64_t M, int64_t N, int64_t K, int64_t ldo, vdmq_stream_t stream);

@@ -613,6 +613,32 @@ def test_bf6_linear_matches_oracle(bf6_path, M, K, N, clip, use_bias):
     assert np.array_equal(y.cpu().numpy().view(np.uint16), want.view(np.uint16))
 
 
+def test_bf6_linear_through_the_c_abi():
+    """vdmq_linear_w4a4_bf6 with an input row stride, GELU fused, against the oracle chain; short workspace refused."""
+    from dsaquant_amd import _lib
+
+    v = vk()
+    lib = _lib.load()
+    M, K, N, ldx = 300, 320, 256, 384
+    x, qw, ws, bias = O.synth_linear(M, K, N, seed=31)
+    xs = torch.full((M, ldx), 1000.0, dtype=torch.float16, device=DEV)
+    xs[:, :K] = t16(x)
+    wb = v.bf6_blocks(t16(pack_native(qw, v.k_padded(K))), K)
+    wsd, bd = t16(ws), t16(bias)
+    out = torch.empty((M, N), dtype=torch.float16, device=DEV)
+    need = int(lib.vdmq_workspace_bytes_bf6(M, K))
+    wsp = torch.empty(need, dtype=torch.uint8, device=DEV)
+    s = torch.cuda.current_stream().cuda_stream
+    _lib.check(lib.vdmq_linear_w4a4_bf6(xs.data_ptr(), M, K, ldx, 1.0, _lib.VDMQ_ACT_GELU_TANH, wb.data_ptr(), wsd.data_ptr(), bd.data_ptr(),
+                                        out.data_ptr(), N, N, wsp.data_ptr(), need, s))
+    torch.cuda.synchronize()
+    _, table = gpu_gelu_table()
+    want = O.np_linear(table[x.view(np.uint16)], qw, ws, bias, 1.0)[0]
+    assert np.array_equal(out.cpu().numpy().view(np.uint16), want.view(np.uint16))
+    assert lib.vdmq_linear_w4a4_bf6(xs.data_ptr(), M, K, ldx, 1.0, 0, wb.data_ptr(), wsd.data_ptr(), bd.data_ptr(), out.data_ptr(), N, N,
+                                    wsp.data_ptr(), need - 1, s) == -4
+
+
 def test_bf6_fused_paths_equal_the_int8_ones(bf6_path):
     """LayerNorm input, GELU input and gated residual through the bf6 GEMM: bitwise equal to the int8 path."""
     from dsaquant_amd import fused_ops
