@@ -46,6 +46,7 @@ constexpr int kBlkBytes = 1536;                 /* 32 rows x 64 k */
 constexpr int kBlkPlaneB = 1024;                /* offset of the 8-byte plane */
 constexpr int BM = 256, BN = 256, KS = 128, S = 3;
 constexpr int kWavesM = 2, kWavesN = 4, kWaves = kWavesM * kWavesN;
+constexpr int kValuPerMfma = 3; /* address arithmetic and operand assembly spread between the MFMAs */
 constexpr int MI = BM / 32 / kWavesM, NI = BN / 32 / kWavesN; /* 32-row blocks per wave: 4 token, 2 weight */
 constexpr int kRbStage = (KS / 64) * kBlkBytes; /* bytes of one row-block per stage */
 constexpr int kStageBytes = (BM + BN) / 32 * kRbStage;
@@ -87,6 +88,7 @@ __device__ __forceinline__ void schedule_region() {
         __builtin_amdgcn_sched_group_barrier(0x008, 1, 0); /* MFMA */
         if constexpr (2 * I < NDS) __builtin_amdgcn_sched_group_barrier(0x100, 2, 0); /* DS reads */
         if constexpr (I < NVMEM) __builtin_amdgcn_sched_group_barrier(0x020, 1, 0); /* direct-to-LDS load */
+        __builtin_amdgcn_sched_group_barrier(0x002, kValuPerMfma, 0); /* VALU */
         schedule_region<NDS, NVMEM, I + 1>();
     } else {
         __builtin_amdgcn_sched_barrier(0);
@@ -96,7 +98,7 @@ __device__ __forceinline__ void schedule_region() {
 // OUT_MODE: 0 = scaled fp16 output, 1 = the same with non-temporal stores, 2 = raw accumulators as int32,
 // 3 / 4 = 0 / 1 followed by the gated residual update out = residual + y * gate (see vdmq_gemm.hip)
 template <int OUT_MODE>
-__global__ __launch_bounds__(kWaves * 64, kWaves / 4) void gemm_bf6_kernel(const uint8_t *__restrict__ X, const uint8_t *__restrict__ W,
+__global__ __launch_bounds__(kWaves * 64, (kWaves + 3) / 4) void gemm_bf6_kernel(const uint8_t *__restrict__ X, const uint8_t *__restrict__ W,
                                                                          const __half *__restrict__ ascale,
                                                                          const __half *__restrict__ wscale,
                                                                          const __half *__restrict__ bias, __half *out,

@@ -228,11 +228,21 @@ struct Bf6Scratch { /* LDS of one workgroup */
 };
 
 // `valid`: the wave's row exists (a workgroup's waves all run this function -- it synchronises them --
-// the ones past M on a copy of the last row, storing nothing).
-template <int NCH>
-__device__ __forceinline__ void quantize_held_row_bf6(const u32x4 (&v)[NCH], int lane, int wave, int64_t row0, bool valid, int M, int Kb,
+// the ones past M on a copy of the last row, storing nothing).  `refill(c)` runs once chunk c of the
+// row has gone to the transpose buffer and its registers are free: a workgroup that walks several
+// row groups loads the next row's chunk there, so those loads overlap the rest of this row's
+// conversion.  `phase` counts the groups this workgroup has staged (it picks the staging copy).
+#ifndef VDMQ_BF6_WALK_MIN_CHUNKS
+#define VDMQ_BF6_WALK_MIN_CHUNKS 17
+#endif
+constexpr bool bf6_walks(int nch) { return nch >= VDMQ_BF6_WALK_MIN_CHUNKS; }
+struct NoRefill {
+    __device__ __forceinline__ void operator()(int) const {}
+};
+template <int NCH, class Refill>
+__device__ __forceinline__ void quantize_held_row_bf6(u32x4 (&v)[NCH], int lane, int wave, int64_t row0, bool valid, int M, int Kb,
                                                       float clip, uint8_t *__restrict__ blocks, __half *__restrict__ scale_h,
-                                                      Bf6Scratch &lds) {
+                                                      Bf6Scratch &lds, int &phase, Refill &&refill) {
     uint32_t m2 = 0;
 #pragma unroll
     for (int c = 0; c < NCH; ++c) m2 = absmax_bits(v[c], m2);
@@ -259,7 +269,7 @@ __device__ __forceinline__ void quantize_held_row_bf6(const u32x4 (&v)[NCH], int
     uint8_t *tbuf = lds.transpose[wave];
     // the thread's share of the cooperative store: string t / 8 of row t % 8 -- eight consecutive
     // threads write the eight rows' parts of one string slot, 128 (and 64) contiguous bytes
-    const int t = threadIdx.x, srow = t % kBf6Rows, sidx = t / kBf6Rows;
+    const int t = wave * kWaveSize + lane, srow = t % kBf6Rows, sidx = t / kBf6Rows;
     const int64_t grow = row0 + srow;
     uint8_t *rowblk = blocks + (grow / 32) * static_cast<int64_t>(kblocks) * 1536;
     const int slot = static_cast<int>(grow % 32);
@@ -272,6 +282,9 @@ __device__ __forceinline__ void quantize_held_row_bf6(const u32x4 (&v)[NCH], int
             const uint32_t off = cc * 1024 + lane * 16;
             *reinterpret_cast<u32x4 *>(tbuf + off + (off >> 8) * 16) = c < NCH ? v[c] : u32x4{0u, 0u, 0u, 0u};
         }
+#pragma unroll
+        for (int cc = 0; cc < 4; ++cc)
+            if (4 * g + cc < NCH) refill(4 * g + cc);
         // (the LDS queue of a wave is in order: the reads below see the writes above)
         u32x4 tr[4];
 #pragma unroll
@@ -306,15 +319,17 @@ __device__ __forceinline__ void quantize_held_row_bf6(const u32x4 (&v)[NCH], int
         const u32x6 str = __builtin_amdgcn_cvt_scalef32_pk32_bf6_f16(q, 1.0f);
         // per-lane stores would scatter 16-byte pieces over 64 cache lines per instruction (measured: 2x
         // slower than the HBM-bound int4 quantizer): collect the workgroup's strings in LDS instead
-        *reinterpret_cast<u32x4 *>(lds.part_a[g & 1][wave] + lane * 16) = u32x4{str[0], str[1], str[2], str[3]};
-        *reinterpret_cast<u32x2 *>(lds.part_b[g & 1][wave] + lane * 8) = u32x2{str[4], str[5]};
+        const int copy = phase & 1;
+        ++phase;
+        *reinterpret_cast<u32x4 *>(lds.part_a[copy][wave] + lane * 16) = u32x4{str[0], str[1], str[2], str[3]};
+        *reinterpret_cast<u32x2 *>(lds.part_b[copy][wave] + lane * 8) = u32x2{str[4], str[5]};
         __syncthreads(); /* also orders this group's writes after every thread's reads of the group before last */
         const int k0 = 2048 * g + 32 * sidx;
         if (k0 < Kb && grow < M) {
             uint8_t *blk = rowblk + static_cast<int64_t>(k0 >> 6) * 1536;
             const int l = slot + 32 * ((k0 >> 5) & 1);
-            *reinterpret_cast<u32x4 *>(blk + l * 16) = *reinterpret_cast<const u32x4 *>(lds.part_a[g & 1][srow] + sidx * 16);
-            *reinterpret_cast<u32x2 *>(blk + 1024 + l * 8) = *reinterpret_cast<const u32x2 *>(lds.part_b[g & 1][srow] + sidx * 8);
+            *reinterpret_cast<u32x4 *>(blk + l * 16) = *reinterpret_cast<const u32x4 *>(lds.part_a[copy][srow] + sidx * 16);
+            *reinterpret_cast<u32x2 *>(blk + 1024 + l * 8) = *reinterpret_cast<const u32x2 *>(lds.part_b[copy][srow] + sidx * 8);
         }
     }
 }
@@ -333,25 +348,55 @@ __global__ __launch_bounds__((FMT == 1 ? kBf6Rows : kRowsPerBlock) * kWaveSize) 
     __half *__restrict__ scale_h) {
     constexpr int ROWS = FMT == 1 ? kBf6Rows : kRowsPerBlock;
     const int lane = threadIdx.x & (kWaveSize - 1), wave = threadIdx.x >> 6;
-    const int64_t row0 = static_cast<int64_t>(blockIdx.x) * ROWS;
-    int64_t row = row0 + wave;
-    const bool valid = row < M;
-    if (!valid) {
-        if (FMT == 0) return;
-        row = M - 1; /* the bf6 tail synchronises the workgroup: stay, on a copy of the last row */
-    }
-    const u32x4 *src = reinterpret_cast<const u32x4 *>(x + row * ldx);
-
-    u32x4 v[NCH];
-#pragma unroll
-    for (int c = 0; c < NCH; ++c) {
-        const int k0 = c * 512 + lane * 8;
-        v[c] = k0 < K ? apply_act<ACT>(__builtin_nontemporal_load(src + c * 64 + lane)) : u32x4{0u, 0u, 0u, 0u};
-    }
-    if (FMT == 1) {
+    if constexpr (FMT == 1) {
+        // The workgroup walks row groups blockIdx.x, blockIdx.x + gridDim.x, ...: with the launcher's grid
+        // (what the chip holds at once) the loads of the next group's rows are in flight while this
+        // group's rows are converted -- a long row leaves room for one workgroup per CU only, whose load and
+        // convert phases would otherwise alternate.
         __shared__ __attribute__((aligned(16))) Bf6Scratch scratch;
-        quantize_held_row_bf6<NCH>(v, lane, wave, row0, valid, M, Kp, clip, qact, scale_h, scratch);
+        const int groups = (M + ROWS - 1) / ROWS;
+        auto row_ptr = [&](int group) {
+            const int64_t r = static_cast<int64_t>(group) * ROWS + wave;
+            return reinterpret_cast<const u32x4 *>(x + (r < M ? r : M - 1) * ldx); /* waves past M stay, on a copy of the last row */
+        };
+        auto load = [&](const u32x4 *src, int c) {
+            return c * 512 + lane * 8 < K ? __builtin_nontemporal_load(src + c * 64 + lane) : u32x4{0u, 0u, 0u, 0u};
+        };
+        int group = blockIdx.x, phase = 0;
+        u32x4 v[NCH];
+        const u32x4 *src = row_ptr(group);
+#pragma unroll
+        for (int c = 0; c < NCH; ++c) v[c] = load(src, c);
+        auto convert = [&](bool more) __attribute__((always_inline)) {
+            if (ACT != VDMQ_ACT_NONE) {
+#pragma unroll
+                for (int c = 0; c < NCH; ++c)
+                    if (c * 512 + lane * 8 < K) v[c] = apply_act<ACT>(v[c]);
+            }
+            const int64_t row0 = static_cast<int64_t>(group) * ROWS;
+            const u32x4 *next = row_ptr(more ? group + gridDim.x : group);
+            quantize_held_row_bf6<NCH>(v, lane, wave, row0, row0 + wave < M, M, Kp, clip, qact, scale_h, scratch, phase,
+                                       [&](int c) {
+                                           if constexpr (bf6_walks(NCH))
+                                               if (more) v[c] = load(next, c);
+                                       });
+        };
+        if constexpr (bf6_walks(NCH)) {
+            for (; group < groups; group += gridDim.x) convert(group + static_cast<int>(gridDim.x) < groups);
+        } else {
+            // short rows: one row group per workgroup -- several workgroups share a CU and overlap anyway
+            convert(false);
+        }
     } else {
+        const int64_t row = static_cast<int64_t>(blockIdx.x) * ROWS + wave;
+        if (row >= M) return;
+        const u32x4 *src = reinterpret_cast<const u32x4 *>(x + row * ldx);
+        u32x4 v[NCH];
+#pragma unroll
+        for (int c = 0; c < NCH; ++c) {
+            const int k0 = c * 512 + lane * 8;
+            v[c] = k0 < K ? apply_act<ACT>(__builtin_nontemporal_load(src + c * 64 + lane)) : u32x4{0u, 0u, 0u, 0u};
+        }
         quantize_held_row<NCH, STREAM_OUT>(v, lane, row, Kp, clip, qact, scale_h);
     }
 }
@@ -459,7 +504,8 @@ __global__ __launch_bounds__((FMT == 1 ? kBf6Rows : kRowsPerBlock) * kWaveSize) 
     }
     if (FMT == 1) {
         __shared__ __attribute__((aligned(16))) Bf6Scratch scratch;
-        quantize_held_row_bf6<NCH>(v, lane, wave, row0, valid, M, Kp, clip, qact, scale_h, scratch);
+        int phase = 0;
+        quantize_held_row_bf6<NCH>(v, lane, wave, row0, valid, M, Kp, clip, qact, scale_h, scratch, phase, NoRefill{});
     } else {
         quantize_held_row<NCH, false>(v, lane, row, Kp, clip, qact, scale_h);
     }
@@ -517,13 +563,38 @@ __global__ __launch_bounds__(256) void quantize_given_scale_kernel(const __half 
 
 constexpr int64_t kStreamOutBytes = int64_t(224) << 20; /* outputs larger than this bypass the caches */
 
+// Workgroups of `kernel` the current device runs at once (CUs x workgroups per CU), or -1.  The answer is
+// kept per device in `cache` (one array per kernel, zero-initialised): the occupancy query costs tens of
+// microseconds, which a launch on an idle stream would show.
+constexpr int kMaxDevices = 64;
+int64_t resident_workgroups(const void *kernel, int threads, int (&cache)[kMaxDevices]) {
+    int dev = 0;
+    if (hipGetDevice(&dev) != hipSuccess || dev < 0 || dev >= kMaxDevices) return -1;
+    if (cache[dev] > 0) return cache[dev];
+    int cus = 0, per_cu = 0;
+    if (hipDeviceGetAttribute(&cus, hipDeviceAttributeMultiprocessorCount, dev) != hipSuccess ||
+        hipOccupancyMaxActiveBlocksPerMultiprocessor(&per_cu, kernel, threads, 0) != hipSuccess || cus <= 0 || per_cu <= 0) {
+        (void)hipGetLastError();
+        return -1;
+    }
+    cache[dev] = cus * per_cu; /* racing first calls store the same value */
+    return cache[dev];
+}
+
 template <int NCH, int ACT>
 int launch_reg(const __half *x, int64_t M, int64_t K, int64_t ldx, float clip, int fmt, uint8_t *qact, __half *scale_h, hipStream_t s) {
     const dim3 grid(static_cast<unsigned>(ceil_div(M, kRowsPerBlock))), block(kRowsPerBlock * kWaveSize);
-    if (fmt == 1)
-        hipLaunchKernelGGL((quantize_rows_kernel<NCH, false, ACT, 1>), dim3(static_cast<unsigned>(ceil_div(M, kBf6Rows))),
+    if (fmt == 1) {
+        const int64_t groups = ceil_div(M, kBf6Rows);
+        static int cache[kMaxDevices];
+        const int64_t resident = !bf6_walks(NCH) ? groups
+                                 : resident_workgroups(reinterpret_cast<const void *>(&quantize_rows_kernel<NCH, false, ACT, 1>),
+                                                       kBf6Rows * kWaveSize, cache);
+        if (resident <= 0) return VDMQ_ELAUNCH;
+        hipLaunchKernelGGL((quantize_rows_kernel<NCH, false, ACT, 1>), dim3(static_cast<unsigned>(!bf6_walks(NCH) || groups < resident ? groups : resident)),
                            dim3(kBf6Rows * kWaveSize), 0, s, x, ldx, static_cast<int>(M), static_cast<int>(K),
                            static_cast<int>(bf6_kblocks(K) * 64), clip, qact, scale_h);
+    }
     else if (M * (k_padded(K) / 2) > kStreamOutBytes)
         hipLaunchKernelGGL((quantize_rows_kernel<NCH, true, ACT, 0>), grid, block, 0, s, x, ldx, static_cast<int>(M), static_cast<int>(K),
                            static_cast<int>(k_padded(K)), clip, qact, scale_h);

@@ -549,10 +549,12 @@ def rows_of_blocks(blocks: torch.Tensor, M: int, K: int) -> np.ndarray:
     return O.np_unpack_bf6_blocks(b.reshape(-1), M, K)
 
 
-@pytest.mark.parametrize("M,K", [(257, 1536), (100, 64), (77, 192), (515, 5120), (130, 13824), (19, 16384), (4096, 8960), (33, 3072)])
+@pytest.mark.parametrize("M,K", [(257, 1536), (100, 64), (77, 192), (515, 5120), (130, 13824), (19, 16384), (4096, 8960), (33, 3072), (2100, 13824)])
 def test_bf6_quantizers_write_the_oracle_integers(M, K):
     """The quantizers that emit bf6 blocks directly (plain, GELU, LayerNorm): decoded with the format's definition,
-    the blocks hold the oracle's integers (plain) / the integers of the int4 quantizer (fused producers), scales equal."""
+    the blocks hold the oracle's integers (plain) / the integers of the int4 quantizer (fused producers), scales equal.
+    Rows longer than 8192 make a workgroup walk several row groups once there are more groups than the chip
+    holds (256 CUs x 1): (4096, 8960) gives every workgroup two, (2100, 13824) a few of them a second, ragged one."""
     from dsaquant_amd import fused_ops
 
     v = vk()
