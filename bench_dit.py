@@ -33,6 +33,8 @@ def main():
     ap.add_argument("--fuse-ln", action="store_true", help="run the blocks' LayerNorm + modulation inside the following activation quantizers")
     ap.add_argument("--fuse-residual", action="store_true", help="run the blocks' gated residual updates in the preceding GEMM epilogues")
     ap.add_argument("--fuse-gelu", action="store_true", help="evaluate the FFN's GELU inside the second linear's activation quantizer")
+    ap.add_argument("--reuse-context", action="store_true",
+                    help="embed each context once, keep the cross-attention K/V per prompt, quantize a context once per forward")
     args = ap.parse_args()
 
     import torch
@@ -52,6 +54,7 @@ def main():
     W.FeedForward.fuse_gelu = bool(args.fuse_gelu)
     W.Block.fuse_ln = bool(args.fuse_ln)
     W.Block.fuse_residual = bool(args.fuse_residual)
+    W.WanDiT.reuse_context = W.Attention.cache_cross_kv = bool(args.reuse_context)
     n_quant = sum(isinstance(m, QuantLinear) for m in model.modules())
     n_fused = sum(isinstance(m, W.Attention) and m.use_fused_qkv_kernel for m in model.modules())
 
@@ -83,7 +86,7 @@ def main():
         "w4a4_ms_per_forward": round(tot.get("w4a4", 0.0) / forwards, 2), "attention_ms_per_forward": round(tot.get("attention", 0.0) / forwards, 2),
         "w4a4_calls_per_forward": cnt.get("w4a4", 0) // forwards, "attention_calls_per_forward": cnt.get("attention", 0) // forwards,
         "tokens_per_forward": tokens, "timesteps": ts, "quant_linears": n_quant, "fused_attention_modules": n_fused,
-        "layers": args.layers, "fuse_gelu": bool(args.fuse_gelu), "fuse_ln": bool(args.fuse_ln), "fuse_residual": bool(args.fuse_residual), "build_s": round(build_s, 1), "data": "synthetic", "n_gpus": 1,
+        "layers": args.layers, "fuse_gelu": bool(args.fuse_gelu), "fuse_ln": bool(args.fuse_ln), "fuse_residual": bool(args.fuse_residual), "reuse_context": bool(args.reuse_context), "build_s": round(build_s, 1), "data": "synthetic", "n_gpus": 1,
     }))
 
 

@@ -129,6 +129,26 @@ def linear_ln_vdm_w4a4(
     return linear_fused(pre, qweight, wscales, bias, clip_ratio, bias_half)
 
 
+class QuantizedInput:
+    """A linear's input that is already quantized per token (native int4 rows and fp16
+    scales): one quantizer launch serves every linear that reads the same tensor with the
+    same clip ratio.  The cross-attention context is such a tensor -- every block's
+    ``attn2`` K/V projection reads ``encoder_hidden_states`` (dit_block.py:109 of the
+    reference), which the reference quantizes again in each of them."""
+
+    def __init__(self, x: torch.Tensor, clip_ratio: float = 1.0):
+        self.shape = tuple(x.shape)
+        self.clip_ratio = float(clip_ratio)
+        x_2d, _ = _k._as_2d_half_contiguous(x)
+        _k._require(x_2d.is_cuda, "input must be a CUDA tensor")
+        self.M, self.K = x_2d.shape
+        self.device = x_2d.device
+        if self.M:
+            self.qact, self.scales = _k._quantize_for_gemm(x_2d, self.clip_ratio, _lib.VDMQ_ACT_NONE, False, None)
+        else:
+            self.qact = self.scales = None
+
+
 def linear_fused(
     x,
     qweight: torch.Tensor,
@@ -144,7 +164,8 @@ def linear_fused(
     """``residual + linear_vdm_w4a4(act(x), ...) * gate`` in two kernels.
 
     ``x`` is a tensor (optionally with ``act="gelu_tanh"`` applied to it inside the
-    quantizer) or an ``LnInput``.  ``gate`` (fp16, one ``[N]`` vector per batch element
+    quantizer), an ``LnInput`` or a ``QuantizedInput`` (whose clip ratio must be the
+    layer's; the int8 matrix path then runs whatever the problem size).  ``gate`` (fp16, one ``[N]`` vector per batch element
     or per token) and ``residual`` (fp16, shaped like the output) are folded into the
     GEMM epilogue as the two fp16 tensor operations of the reference's
     ``hidden_states + attn_output * gate`` (dit_block.py:102, :107, :112); either may
@@ -154,16 +175,26 @@ def linear_fused(
         if act is not None:
             raise ValueError("an activation cannot be combined with a LayerNorm input")
         pre, x_2d, lead = x, x.x, x.shape[:-1]
+    elif isinstance(x, QuantizedInput):
+        if act is not None:
+            raise ValueError("an activation cannot be applied to an input that is already quantized")
+        if x.clip_ratio != float(clip_ratio):
+            raise ValueError(f"input quantized with clip ratio {x.clip_ratio}, the layer wants {float(clip_ratio)}")
+        pre, x_2d, lead = x, None, x.shape[:-1]
     else:
         pre = None
         x_2d, lead = _k._as_2d_half_contiguous(x)
-    _k._check_linear_shapes(x_2d, qweight, wscales)
-    _k._require(x_2d.is_cuda, "input must be a CUDA tensor")
+    if x_2d is not None:
+        _k._check_linear_shapes(x_2d, qweight, wscales)
+        _k._require(x_2d.is_cuda, "input must be a CUDA tensor")
+        M, K = x_2d.shape
+        dev = x_2d.device
+    else:
+        M, K, dev = pre.M, pre.K, pre.device
+        _k._check_packed_weight(qweight, wscales, K)
     act_code = _k._act_code(act)
     native_w, wscale = _k._native_weights(qweight.contiguous(), wscales.contiguous())
-    M, K = x_2d.shape
     N = native_w.shape[0]
-    dev = x_2d.device
     b = bias_half if bias_half is not None else bias
     if b is not None:
         b = b.half().contiguous().view(-1)
@@ -186,7 +217,9 @@ def linear_fused(
         _k._check_device_tensor(r2, "residual", torch.float16)
     with torch.cuda.device(dev):
         out = torch.empty((M, N), dtype=torch.float16, device=dev)
-        if M:
+        if M and isinstance(pre, QuantizedInput):
+            _k._gemm_dispatch(pre.qact, pre.scales, False, native_w, wscale, b, out, K, gate=g2, rows_per_gate=rows_per_gate, residual=r2)
+        elif M:
             bf6 = _k._use_bf6(M, N, K)
             operand, scales = _k._quantize_for_gemm(x_2d, clip_ratio, act_code, bf6, None if pre is None else pre._args())
             _k._gemm_dispatch(operand, scales, bf6, native_w, wscale, b, out, K, gate=g2, rows_per_gate=rows_per_gate, residual=r2)
@@ -205,10 +238,11 @@ def qkv_projections_ln(attn, pre: LnInput):
     return out.split(n, dim=-1)
 
 
-def kv_projections(attn, encoder_hidden_states: torch.Tensor):
-    """Cross-attention K, V through the cached concatenation Wk|Wv (attention.py:70-107 of the reference)."""
+def kv_projections(attn, encoder_hidden_states):
+    """Cross-attention K, V through the cached concatenation Wk|Wv (attention.py:70-107 of the reference);
+    ``encoder_hidden_states`` is the tensor or a ``QuantizedInput`` of it shared between blocks."""
     from .fused_qkv import _cat_cached
 
     w, s, b = _cat_cached(attn, ["to_k", "to_v"], "kv")
-    kv = _k.linear_vdm_w4a4(encoder_hidden_states, w, s, bias=None, clip_ratio=attn.to_k.kernel_clip_ratio, bias_half=b)
+    kv = linear_fused(encoder_hidden_states, w, s, None, attn.to_k.kernel_clip_ratio, bias_half=b)
     return kv.split(attn.to_k.vdm_weight_packed.shape[0], dim=-1)

@@ -95,16 +95,20 @@ def _as_2d_half_contiguous(x: torch.Tensor) -> Tuple[torch.Tensor, Tuple[int, ..
     return x.reshape(-1, x.shape[-1]).half().contiguous(), orig_shape
 
 
-def _check_linear_shapes(x_2d: torch.Tensor, qweight: torch.Tensor, wscales: torch.Tensor) -> None:
+def _check_packed_weight(qweight: torch.Tensor, wscales: torch.Tensor, K: int) -> None:
     # same conditions, order and exception type as vdm_w4a4.py:198-206
-    if x_2d.shape[1] % WARP_K != 0:
-        raise ValueError(f"K={x_2d.shape[1]} must be a multiple of {WARP_K}")
+    if K % WARP_K != 0:
+        raise ValueError(f"K={K} must be a multiple of {WARP_K}")
     if qweight.shape[0] % BLOCK_N != 0:
         raise ValueError(f"N={qweight.shape[0]} must be a multiple of {BLOCK_N}")
-    if qweight.shape[1] != x_2d.shape[1] // 2:
+    if qweight.shape[1] != K // 2:
         raise ValueError("qweight shape must be [N, K/2]")
-    if wscales.shape != (qweight.shape[0], x_2d.shape[1] // WARP_K):
+    if wscales.shape != (qweight.shape[0], K // WARP_K):
         raise ValueError("wscales shape must be [N, K/64]")
+
+
+def _check_linear_shapes(x_2d: torch.Tensor, qweight: torch.Tensor, wscales: torch.Tensor) -> None:
+    _check_packed_weight(qweight, wscales, x_2d.shape[1])
 
 
 def k_padded(K: int) -> int:

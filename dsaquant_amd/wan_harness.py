@@ -99,6 +99,37 @@ def apply_rope(x: torch.Tensor, freqs: torch.Tensor) -> torch.Tensor:
     return torch.view_as_real(xc * freqs).flatten(3).to(x.dtype)
 
 
+class SharedContext:
+    """The cross-attention context of one forward together with its per-token quantization, made once per clip
+    ratio and read by every block's K/V projection (the reference quantizes it in each block, dit_block.py:109)."""
+
+    def __init__(self, tensor: torch.Tensor):
+        self.tensor = tensor
+        self._quantized = {}
+
+    def quantized(self, clip_ratio: float):
+        from . import fused_ops
+
+        q = self._quantized.get(float(clip_ratio))
+        if q is None:
+            q = self._quantized[float(clip_ratio)] = fused_ops.QuantizedInput(self.tensor, clip_ratio)
+        return q
+
+
+def _weak_lookup(cache: dict, tensor: torch.Tensor):
+    hit = cache.get(id(tensor))
+    if hit is not None and hit[0]() is tensor and hit[1] == tensor._version:
+        return hit[2]
+    return None
+
+
+def _weak_store(cache: dict, tensor: torch.Tensor, value) -> None:
+    import weakref
+
+    key = id(tensor)
+    cache[key] = (weakref.ref(tensor, lambda _, d=cache, k=key: d.pop(k, None)), tensor._version, value)
+
+
 class Attention(nn.Module):
     def __init__(self, dim: int, heads: int, eps: float, cross: bool):
         super().__init__()
@@ -110,23 +141,59 @@ class Attention(nn.Module):
         self.fused_projections = False
         self.use_fused_qkv_kernel = False
         self.qkv_kernel_backend = None
+        self._cross_kv = {}
+
+    # Cross-attention K (after norm_k) and V depend on the context only, which is the same tensor in every denoise
+    # step of a prompt: keep them per context tensor (held weakly: a new tensor at a recycled address is a miss).
+    cache_cross_kv = False
+
+    def _context_kv(self, context):
+        """K (normalised) and V of the cross-attention context, a tensor or a SharedContext."""
+        from . import fused_ops
+
+        tensor = context.tensor if isinstance(context, SharedContext) else context
+        if self.cache_cross_kv:
+            hit = _weak_lookup(self._cross_kv, tensor)
+            if hit is not None:
+                return hit
+        kernel = getattr(self.to_k, "use_vdm_kernel", False)
+        if kernel and isinstance(context, SharedContext):
+            k, v = fused_ops.kv_projections(self, context.quantized(self.to_k.kernel_clip_ratio))
+        elif kernel and self.use_fused_qkv_kernel:
+            k, v = fused_ops.kv_projections(self, tensor)
+        else:
+            k, v = self.to_k(tensor), self.to_v(tensor)
+        k = self.norm_k(k)
+        if self.cache_cross_kv:
+            _weak_store(self._cross_kv, tensor, (k, v))
+        return k, v
 
     def forward(self, x, context: Optional[torch.Tensor], freqs: Optional[torch.Tensor], timers=None, residual=None, gate=None) -> torch.Tensor:
         """Returns the attention output, or ``residual + output * gate`` when ``residual`` is given (the update
         then runs in the output projection's GEMM epilogue if that projection is in kernel mode)."""
         from . import fused_ops
 
-        if isinstance(x, fused_ops.LnInput):  # the LayerNorm in front of this module runs inside the quantizer
-            if context is None:
-                q, k, v = fused_ops.qkv_projections_ln(self, x)
-            else:
-                tq = self.to_q
+        if context is not None and (self.cache_cross_kv or isinstance(context, SharedContext)):
+            tq = self.to_q
+            if isinstance(x, fused_ops.LnInput):
                 q = fused_ops.linear_ln_vdm_w4a4(x, tq.vdm_weight_packed, tq.vdm_weight_scale_packed, tq.bias, tq.kernel_clip_ratio,
                                                  bias_half=tq._bias_half)
-                k, v = fused_ops.kv_projections(self, context)
+            else:
+                q = tq(x)
+            q = self.norm_q(q)
+            k, v = self._context_kv(context)
         else:
-            q, k, v = get_qkv_projections(self, x, context)
-        q, k = self.norm_q(q), self.norm_k(k)
+            if isinstance(x, fused_ops.LnInput):  # the LayerNorm in front of this module runs inside the quantizer
+                if context is None:
+                    q, k, v = fused_ops.qkv_projections_ln(self, x)
+                else:
+                    tq = self.to_q
+                    q = fused_ops.linear_ln_vdm_w4a4(x, tq.vdm_weight_packed, tq.vdm_weight_scale_packed, tq.bias, tq.kernel_clip_ratio,
+                                                     bias_half=tq._bias_half)
+                    k, v = fused_ops.kv_projections(self, context)
+            else:
+                q, k, v = get_qkv_projections(self, x, context)
+            q, k = self.norm_q(q), self.norm_k(k)
         q, k, v = (t.unflatten(2, (self.heads, -1)) for t in (q, k, v))
         if freqs is not None:
             q, k = apply_rope(q, freqs), apply_rope(k, freqs)
@@ -244,6 +311,21 @@ class WanDiT(nn.Module):
         x = tokens.reshape(1, f // p1, h // p2, w // p3, c, p1, p2, p3)
         return x.permute(0, 4, 1, 5, 2, 6, 3, 7).reshape(1, c, f, h, w)
 
+    # reuse_context: embed each context tensor once (the prompt's cond / uncond embeddings are the same tensors in
+    # every denoise step), keep the blocks' cross-attention K/V per embedded context, and quantize a context that
+    # does have to be projected once per forward for all blocks.  Outputs are bit-identical either way.
+    reuse_context = False
+
+    def _embedded_context(self, context: torch.Tensor):
+        if not self.reuse_context:
+            return self.text_embedder(context)
+        cache = self.__dict__.setdefault("_context_cache", {})
+        ctx = _weak_lookup(cache, context)
+        if ctx is None:
+            ctx = SharedContext(self.text_embedder(context))
+            _weak_store(cache, context, ctx)
+        return ctx
+
     def forward(self, latent: torch.Tensor, timestep: torch.Tensor, context: torch.Tensor, timers=None) -> torch.Tensor:
         """latent [1, C, F, H, W] fp16, timestep [1], context [1, 512, text_dim] -> noise prediction like latent."""
         a = self.args
@@ -254,7 +336,7 @@ class WanDiT(nn.Module):
         ang = torch.outer(timestep.double(), torch.pow(10000.0, -torch.arange(half, dtype=torch.float64, device=latent.device) / half))
         temb = self.time_embedder(torch.cat([torch.cos(ang), torch.sin(ang)], dim=1).to(x.dtype))
         tproj = self.time_proj(F.silu(temb)).unflatten(1, (6, -1))
-        ctx = self.text_embedder(context)
+        ctx = self._embedded_context(context)
         for blk in self.blocks:
             x = blk(x, ctx, tproj, freqs, timers)
         shift, scale = (self.scale_shift_table.to(temb.dtype) + temb[:, None, :]).unbind(dim=1)

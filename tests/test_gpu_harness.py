@@ -97,6 +97,51 @@ def test_small_dit_structure_and_numerics():
     assert (n1, n2) == (4, 3)
 
 
+def test_context_reuse_changes_nothing_but_the_work():
+    """One quantization of the cross-attention context per forward (QuantizedInput shared by the blocks), the embedded
+    context and the blocks' K/V kept per context tensor: bit-identical outputs, fewer W4A4 calls from the second
+    forward on, and a different context tensor is a miss."""
+    from dsaquant_amd import fused_ops
+    from dsaquant_amd import wan_harness as W
+    from dsaquant_amd.kernels import vdm_w4a4 as v
+
+    dev = "cuda:0"
+    args = replace(W.WAN21_1P3B, num_layers=2, num_heads=2, ffn_dim=512, text_dim=128)
+    model = W.build_quantized(args, dev, seed=3)
+    g = torch.Generator(device=dev).manual_seed(5)
+    latent = torch.randn((1, 16, 3, 8, 12), generator=g, device=dev).half()
+    ctx_a = torch.randn((1, 512, args.text_dim), generator=g, device=dev).half()
+    ctx_b = torch.randn((1, 512, args.text_dim), generator=g, device=dev).half()
+    t = torch.tensor([700.0], device=dev)
+
+    # a linear fed by a QuantizedInput equals the linear that quantizes for itself
+    lay = model.blocks[0].attn2.to_k
+    e = model.text_embedder(ctx_a)
+    want = v.linear_vdm_w4a4(e, lay.vdm_weight_packed, lay.vdm_weight_scale_packed, lay.bias, lay.kernel_clip_ratio, bias_half=lay._bias_half)
+    shared = fused_ops.QuantizedInput(e, lay.kernel_clip_ratio)
+    got = fused_ops.linear_fused(shared, lay.vdm_weight_packed, lay.vdm_weight_scale_packed, lay.bias, lay.kernel_clip_ratio, bias_half=lay._bias_half)
+    assert torch.equal(got, want)
+    with pytest.raises(ValueError):
+        fused_ops.linear_fused(shared, lay.vdm_weight_packed, lay.vdm_weight_scale_packed, lay.bias, lay.kernel_clip_ratio * 0.5)
+
+    with torch.no_grad():
+        plain = [model(latent, t, c) for c in (ctx_a, ctx_b, ctx_a)]
+    W.WanDiT.reuse_context = W.Attention.cache_cross_kv = True
+    try:
+        counts, outs = [], []
+        for c in (ctx_a, ctx_b, ctx_a, ctx_a.clone()):
+            timers = W.KernelTimers()
+            with torch.no_grad(), W.time_w4a4_calls(timers):
+                outs.append(model(latent, t, c, timers))
+            timers.collect()
+            counts.append(timers.counts()["w4a4"])
+    finally:
+        W.WanDiT.reuse_context = W.Attention.cache_cross_kv = False
+    assert all(torch.equal(o, p) for o, p in zip(outs, plain)) and torch.equal(outs[3], plain[0])
+    L = args.num_layers
+    assert counts == [7 * L, 7 * L, 6 * L, 7 * L]  # third forward: no K/V projection; a cloned context is a new tensor
+
+
 def test_patchify_roundtrip():
     from dsaquant_amd import wan_harness as W
 
