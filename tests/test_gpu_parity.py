@@ -727,8 +727,17 @@ def test_c_abi_with_row_strides():
 
 # ---------------------------------------------------- full-size properties
 
-def test_config3_sized_rows_sampled_against_oracle_and_ragged_tail():
-    """Wan-14B 720p fused QKV shape with the ragged M = 75600 + 37: a sample of
+@pytest.fixture(params=["int8", "bf6"])
+def each_matrix_path(request):
+    v = vk()
+    old = v.matrix_path()
+    v.set_matrix_path(request.param)
+    yield request.param
+    v.set_matrix_path(old)
+
+
+def test_config3_sized_rows_sampled_against_oracle_and_ragged_tail(each_matrix_path):
+    """Wan-14B 720p fused QKV shape with the ragged M = 75600 + 37, on either matrix path: a sample of
     rows (including the last tile's tail) against the oracle, every row's token
     scale, and the un-ragged prefix against a second run with M = 75600."""
     v = vk()
@@ -755,6 +764,33 @@ def test_config3_sized_rows_sampled_against_oracle_and_ragged_tail():
     assert torch.equal(yp, y[:4096][perm.to(DEV)])
     _, sc = v.quantize_activation_native(xd, 1.0)
     assert np.array_equal(sc.cpu().numpy().view(np.uint16), O.np_row_scale(x.numpy(), 1.0).view(np.uint16))
+
+
+def test_config3_sized_ffn_down_long_rows(each_matrix_path):
+    """Wan-14B 720p FFN-down shape (K = 13824: the quantizers' long-row forms, on the bf6 path workgroups that walk
+    37 row groups each) with the ragged M = 75600 + 37: sampled rows against the oracle, every token scale against
+    the scale formula evaluated by torch in fp32, prefix equality."""
+    v = vk()
+    M, K, N = 75637, 13824, 5120
+    g = torch.Generator(device=DEV).manual_seed(11)
+    xd = torch.randn((M, K), generator=g, device=DEV, dtype=torch.float16)
+    xd[:, :: 97] *= 12
+    _, qw, ws, bias = O.synth_linear(1, K, N, seed=2)
+    qv1, sv1, b = t16(O.np_pack_wgt_v1(qw)), t16(O.np_pack_wscales_v1(ws, K)), t16(bias)
+    print(f"config-3 ffn-down {each_matrix_path}", flush=True)
+    y = v.linear_vdm_w4a4(xd, qv1, sv1, b, clip_ratio=0.95)
+    y0 = v.linear_vdm_w4a4(xd[:75600], qv1, sv1, b, clip_ratio=0.95)
+    assert torch.equal(y[:75600], y0)
+    rows = torch.from_numpy(np.concatenate([np.arange(0, 40), np.arange(2040, 2060), np.arange(40000, 40024), np.arange(75590, M)])).to(DEV)
+    want, _, _, _ = O.np_linear(xd[rows].cpu().numpy(), qw, ws, bias, 0.95)
+    assert np.array_equal(y[rows].cpu().numpy().view(np.uint16), want.view(np.uint16))
+    if each_matrix_path == "bf6":
+        _, sc = v.quantize_activation_bf6(xd, 0.95)
+    else:
+        _, sc = v.quantize_activation_native(xd, 0.95)
+    amax = xd.abs().amax(dim=1).float()
+    seven = torch.full_like(amax, 7.0)  # a tensor divisor: torch turns division by a Python scalar into a multiplication
+    assert torch.equal(sc.view(-1), ((amax / seven) * 0.95).half())
 
 
 # ------------------------------------------------------- committed fixture
