@@ -793,6 +793,46 @@ def test_config3_sized_ffn_down_long_rows(each_matrix_path):
     assert torch.equal(sc.view(-1), ((amax / seven) * 0.95).half())
 
 
+# ------------------------------------------------------------- HIP graphs
+
+def test_linear_replays_from_a_hip_graph(each_matrix_path):
+    """Nothing on the path allocates through HIP, synchronises or clears memory with a memset node: the whole fused
+    linear (LayerNorm quantizer, GEMM with the gated residual tail) and the plain one are captured into one graph and
+    replayed with new inputs, eager work and synchronisations between the replays; every replay equals the eager result."""
+    from dsaquant_amd import fused_ops
+
+    v = vk()
+    B, L, K, N = 2, 1500, 1536, 1536
+    rng = np.random.default_rng(9)
+    _, qw, ws, bias = O.synth_linear(1, K, N, seed=4)
+    qv1, sv1, b = t16(O.np_pack_wgt_v1(qw)), t16(O.np_pack_wscales_v1(ws, K)), t16(bias)
+
+    def fresh(shape, scale=1.0):
+        return t16((scale * rng.standard_normal(shape)).astype(np.float16))
+
+    def step(x, a, sh, res, gate):
+        h = fused_ops.linear_fused(fused_ops.LnInput(x, a, sh, 1e-6), qv1, sv1, b, 0.95, residual=res, gate=gate)
+        return v.linear_vdm_w4a4(h, qv1, sv1, b, clip_ratio=1.0)
+
+    statics = [fresh((B, L, K)), fresh((B, 1, K), 0.2), fresh((B, 1, K), 0.3), fresh((B, L, N)), fresh((B, 1, N))]
+    step(*statics)  # first call: weight relayouts and per-device kernel attributes, outside the capture
+    torch.cuda.synchronize()
+    graph = torch.cuda.CUDAGraph()
+    print(f"graph capture {each_matrix_path}", flush=True)
+    with torch.cuda.graph(graph):
+        out = step(*statics)
+    for it in range(3):
+        new = [fresh((B, L, K), 1.0 + it), fresh((B, 1, K), 0.2), fresh((B, 1, K), 0.3), fresh((B, L, N)), fresh((B, 1, N))]
+        for dst, src in zip(statics, new):
+            dst.copy_(src)
+        graph.replay()
+        torch.cuda.synchronize()
+        got = out.clone()
+        want = step(*new)
+        torch.cuda.synchronize()
+        assert torch.equal(got, want), it
+
+
 # ------------------------------------------------------- committed fixture
 
 def test_hip_path_reproduces_the_committed_emulation_fixture():
