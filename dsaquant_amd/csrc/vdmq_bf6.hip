@@ -44,34 +44,49 @@ __device__ __forceinline__ void lds_barrier() {
 
 constexpr int kBlkBytes = 1536;                 /* 32 rows x 64 k */
 constexpr int kBlkPlaneB = 1024;                /* offset of the 8-byte plane */
-constexpr int BM = 256, BN = 256, KS = 128, S = 3;
-constexpr int kWavesM = 2, kWavesN = 4, kWaves = kWavesM * kWavesN;
-constexpr int kValuPerMfma = 3; /* address arithmetic and operand assembly spread between the MFMAs */
-constexpr int MI = BM / 32 / kWavesM, NI = BN / 32 / kWavesN; /* 32-row blocks per wave: 4 token, 2 weight */
+constexpr int KS = 128;                         /* K step: two k-blocks per stage */
 constexpr int kRbStage = (KS / 64) * kBlkBytes; /* bytes of one row-block per stage */
-constexpr int kStageBytes = (BM + BN) / 32 * kRbStage;
-constexpr int kLoads = kStageBytes / 1024 / kWaves;
-constexpr int kLdsBytes = S * kStageBytes;
-constexpr int kWaveN = NI * 32;
-constexpr int kStageRowBytes = kWaveN * 2 + 16; /* epilogue staging: fp16 strip rows padded by 16 bytes */
-constexpr int kStagingBytes = 32 * kStageRowBytes;
-constexpr int kPiecesPerRow = kWaveN / 8;
-static_assert(kStagingBytes * kWaves <= kLdsBytes, "epilogue staging reuses the stage ring");
-static_assert(kStageBytes % (1024 * kWaves) == 0, "stage splits evenly over the waves");
-static_assert(kLoads * (S - 1) < 64, "vmcnt is a 6-bit counter");
+constexpr int kXcds = 8;
 
-constexpr int kXcds = 8, kGroupM = 8, kGroupN = 4;
+// Tile configuration.  BM token rows x BN weight rows per workgroup, WAVES_M x WAVES_N waves (a wave owns
+// 128 x 64: 4 x 2 MFMA tiles), STAGES ring slots of (BM + BN) / 32 row-blocks, OCC workgroups per CU.  One
+// configuration is instantiated: one workgroup of eight waves owns the CU, the fewest operand bytes per MAC.
+// (128 x 256 tiles with two workgroups of four waves per CU, so that one's prologue and epilogue run under the
+// other's K loop, measured 2...10 % slower on every shape down to K = 1536, with and without a start offset
+// between the two.)
+template <int BM_, int BN_, int WAVES_M_, int WAVES_N_, int STAGES_, int OCC_>
+struct Bf6Cfg {
+    static constexpr int BM = BM_, BN = BN_, kWavesM = WAVES_M_, kWavesN = WAVES_N_, kWaves = WAVES_M_ * WAVES_N_, S = STAGES_, kOcc = OCC_;
+    static constexpr int MI = BM / 32 / kWavesM, NI = BN / 32 / kWavesN; /* 32-row blocks per wave: token, weight */
+    static constexpr int kStageBytes = (BM + BN) / 32 * kRbStage;
+    static constexpr int kLoads = kStageBytes / 1024 / kWaves;
+    static constexpr int kLdsBytes = S * kStageBytes;
+    static constexpr int kWaveN = NI * 32;
+    static constexpr int kStageRowBytes = kWaveN * 2 + 16; /* epilogue staging: fp16 strip rows padded by 16 bytes */
+    static constexpr int kStagingBytes = 32 * kStageRowBytes;
+    static constexpr int kPiecesPerRow = kWaveN / 8;
+    static constexpr int kPerLog2 = BM == 256 ? 5 : 6; /* tiles per super-tile: what an XCD's 32 CUs hold at once */
+    static_assert(MI == 4 && NI == 2, "the schedule below is written for 128 x 64 wave tiles");
+    static_assert(kStagingBytes * kWaves <= kLdsBytes, "epilogue staging reuses the stage ring");
+    static_assert(kStageBytes % (1024 * kWaves) == 0, "stage splits evenly over the waves");
+    static_assert(kLoads * (S - 1) < 64, "vmcnt is a 6-bit counter");
+    static_assert(kLdsBytes * kOcc <= 160 * 1024, "the CU's LDS holds OCC workgroups");
+};
+using Bf6Big = Bf6Cfg<256, 256, 2, 4, 3, 1>;
+constexpr int kValuPerMfma = 3; /* address arithmetic and operand assembly spread between the MFMAs */
+
 struct Bf6TileMap {
     int tiles_m, tiles_n, super_n, total_super;
+    int group_n_log2, per_log2; /* a super-tile is (per / group_n) x group_n tiles */
 };
 
-// workgroup b runs on XCD b % 8; each XCD walks 8 x 4 super-tiles (see vdmq_gemm.hip)
+// workgroup b runs on XCD b % 8; each XCD walks super-tiles (see vdmq_gemm.hip)
 __device__ __forceinline__ bool map_tile(const Bf6TileMap &tm, int bid, int &tile_m, int &tile_n) {
-    const int xcd = bid % kXcds, slot = bid / kXcds, per = kGroupM * kGroupN;
-    const int st = (slot / per) * kXcds + xcd, j = slot % per;
+    const int xcd = bid % kXcds, slot = bid / kXcds;
+    const int st = (slot >> tm.per_log2) * kXcds + xcd, j = slot & ((1 << tm.per_log2) - 1);
     if (st >= tm.total_super) return false;
-    tile_m = (st / tm.super_n) * kGroupM + j / kGroupN;
-    tile_n = (st % tm.super_n) * kGroupN + j % kGroupN;
+    tile_m = ((st / tm.super_n) << (tm.per_log2 - tm.group_n_log2)) + (j >> tm.group_n_log2);
+    tile_n = ((st % tm.super_n) << tm.group_n_log2) + (j & ((1 << tm.group_n_log2) - 1));
     return tile_m < tm.tiles_m && tile_n < tm.tiles_n;
 }
 
@@ -84,7 +99,7 @@ __device__ __forceinline__ v8i ld_frag(const uint8_t *p, uint32_t la, uint32_t l
 
 template <int NDS, int NVMEM, int I = 0>
 __device__ __forceinline__ void schedule_region() {
-    if constexpr (I < NI * MI) {
+    if constexpr (I < 8) { /* the 4 x 2 MFMAs of a k-block */
         __builtin_amdgcn_sched_group_barrier(0x008, 1, 0); /* MFMA */
         if constexpr (2 * I < NDS) __builtin_amdgcn_sched_group_barrier(0x100, 2, 0); /* DS reads */
         if constexpr (I < NVMEM) __builtin_amdgcn_sched_group_barrier(0x020, 1, 0); /* direct-to-LDS load */
@@ -97,14 +112,17 @@ __device__ __forceinline__ void schedule_region() {
 
 // OUT_MODE: 0 = scaled fp16 output, 1 = the same with non-temporal stores, 2 = raw accumulators as int32,
 // 3 / 4 = 0 / 1 followed by the gated residual update out = residual + y * gate (see vdmq_gemm.hip)
-template <int OUT_MODE>
-__global__ __launch_bounds__(kWaves * 64, (kWaves + 3) / 4) void gemm_bf6_kernel(const uint8_t *__restrict__ X, const uint8_t *__restrict__ W,
+template <class Cfg, int OUT_MODE>
+__global__ __launch_bounds__(Cfg::kWaves * 64, (Cfg::kWaves * Cfg::kOcc + 3) / 4) void gemm_bf6_kernel(const uint8_t *__restrict__ X, const uint8_t *__restrict__ W,
                                                                          const __half *__restrict__ ascale,
                                                                          const __half *__restrict__ wscale,
                                                                          const __half *__restrict__ bias, __half *out,
                                                                          int32_t *__restrict__ acc_out, int M, int N, int kblocks,
                                                                          int64_t ldo, Bf6TileMap tmap, GemmTail tail) {
     constexpr bool ACC_OUT = OUT_MODE == 2, STREAM_OUT = OUT_MODE == 1 || OUT_MODE == 4, TAIL = OUT_MODE >= 3;
+    constexpr int BM = Cfg::BM, BN = Cfg::BN, S = Cfg::S, MI = Cfg::MI, NI = Cfg::NI, kWaves = Cfg::kWaves, kWavesN = Cfg::kWavesN;
+    constexpr int kLoads = Cfg::kLoads, kStageBytes = Cfg::kStageBytes;
+    constexpr int kPiecesPerRow = Cfg::kPiecesPerRow, kStageRowBytes = Cfg::kStageRowBytes, kStagingBytes = Cfg::kStagingBytes;
     extern __shared__ __attribute__((aligned(1024))) uint8_t lds[];
     int tile_m, tile_n;
     if (!map_tile(tmap, blockIdx.x, tile_m, tile_n)) return;
@@ -112,7 +130,7 @@ __global__ __launch_bounds__(kWaves * 64, (kWaves + 3) / 4) void gemm_bf6_kernel
     const int wn = wave % kWavesN, wm = wave / kWavesN;
     const int64_t rbs = static_cast<int64_t>(kblocks) * kBlkBytes; /* bytes of one row-block over all K */
     const int last_rb_m = (M + 31) / 32 - 1, last_rb_n = N / 32 - 1;
-    // global -> LDS: a stage is 16 row-blocks x 3 KiB; this wave's i-th instruction moves KiB (i * kWaves + wave) of it
+    // global -> LDS: a stage is (BN + BM) / 32 row-blocks x 3 KiB, weights first; this wave's i-th instruction moves KiB (i * kWaves + wave) of it
     const uint8_t *src[kLoads];
 #pragma unroll
     for (int i = 0; i < kLoads; ++i) {
@@ -321,39 +339,72 @@ int launch_nibbles_to_bf6(const uint8_t *native, int64_t rows, int64_t K, uint8_
     return check_launch("nibbles_to_bf6_kernel");
 }
 
-int launch_gemm_bf6(const uint8_t *xblocks, const __half *ascale, const uint8_t *wblocks, const __half *wscale, const __half *bias,
-                    __half *out, int32_t *acc_out, int64_t M, int64_t N, int64_t K, int64_t ldo, const GemmTail &tail, hipStream_t s) {
-    if (M == 0 || N == 0) return VDMQ_OK;
+namespace {
+
+template <class Cfg>
+int launch_bf6_cfg(const uint8_t *xblocks, const __half *ascale, const uint8_t *wblocks, const __half *wscale, const __half *bias,
+                   __half *out, int32_t *acc_out, int64_t M, int64_t N, int64_t K, int64_t ldo, const GemmTail &tail, hipStream_t s) {
+    constexpr int per = 1 << Cfg::kPerLog2;
     Bf6TileMap tm;
-    tm.tiles_m = static_cast<int>(ceil_div(M, BM));
-    tm.tiles_n = static_cast<int>(ceil_div(N, BN));
-    const int super_m = static_cast<int>(ceil_div(tm.tiles_m, kGroupM));
-    tm.super_n = static_cast<int>(ceil_div(tm.tiles_n, kGroupN));
-    const int64_t total_super = static_cast<int64_t>(super_m) * tm.super_n;
-    if (total_super * kGroupM * kGroupN + kXcds * kGroupM * kGroupN > (int64_t(1) << 30))
+    tm.tiles_m = static_cast<int>(ceil_div(M, Cfg::BM));
+    tm.tiles_n = static_cast<int>(ceil_div(N, Cfg::BN));
+    tm.per_log2 = Cfg::kPerLog2;
+    // Super-tile shape: per / gn x gn tiles.  Super-tiles go round the XCDs in turn and a ragged edge leaves some
+    // of them partly empty -- six tile columns in groups of four give every other XCD half the work -- so groups of
+    // two columns replace the groups of four (2048 token rows x 1024 weight rows, the fewest operand bytes per tile
+    // and measured best wherever the work is even) when that takes at least a tenth off the busiest XCD's tile
+    // count (N = 1536 at M = 32760: +16 % at K = 1536, +23 % at K = 8960).
+    int64_t best_load = -1, total_super = 0;
+    for (int gn_log2 : {2, 1}) {
+        const int gn = 1 << gn_log2, gm = per >> gn_log2;
+        const int64_t sm = ceil_div(tm.tiles_m, gm), sn = ceil_div(tm.tiles_n, gn);
+        const int64_t last_m = tm.tiles_m - (sm - 1) * gm, last_n = tm.tiles_n - (sn - 1) * gn;
+        int64_t load[kXcds] = {};
+        if (sm * sn <= 4096) /* beyond that the edges no longer matter: the first shape is taken */
+            for (int64_t st = 0; st < sm * sn; ++st)
+                load[st % kXcds] += (st / sn == sm - 1 ? last_m : gm) * (st % sn == sn - 1 ? last_n : gn);
+        int64_t worst = 0;
+        for (int x = 0; x < kXcds; ++x) worst = load[x] > worst ? load[x] : worst;
+        if (best_load < 0 || worst * 10 <= best_load * 9) {
+            best_load = worst;
+            tm.group_n_log2 = gn_log2;
+            tm.super_n = static_cast<int>(sn);
+            total_super = sm * sn;
+        }
+    }
+    if (best_load < 0 || total_super * per + kXcds * per > (int64_t(1) << 30))
         return fail(VDMQ_ESHAPE, "M x N = %lld x %lld needs more workgroups than one launch can hold", (long long)M, (long long)N);
     tm.total_super = static_cast<int>(total_super);
     const int rounds = static_cast<int>(ceil_div(total_super, kXcds));
-    const dim3 grid(static_cast<unsigned>(rounds) * kXcds * kGroupM * kGroupN), block(kWaves * 64);
+    const dim3 grid(static_cast<unsigned>(rounds) * kXcds * per), block(Cfg::kWaves * 64);
     const bool stream_out = M * N * 2 > (int64_t(224) << 20);
     const bool has_tail = tail.gate != nullptr || tail.residual != nullptr;
     const int which = acc_out != nullptr ? 2 : (stream_out ? 1 : 0) + (has_tail ? 3 : 0);
     using Kernel = void (*)(const uint8_t *, const uint8_t *, const __half *, const __half *, const __half *, __half *, int32_t *, int, int,
                             int, int64_t, Bf6TileMap, GemmTail);
-    const Kernel kernels[5] = {gemm_bf6_kernel<0>, gemm_bf6_kernel<1>, gemm_bf6_kernel<2>, gemm_bf6_kernel<3>, gemm_bf6_kernel<4>};
+    const Kernel kernels[5] = {gemm_bf6_kernel<Cfg, 0>, gemm_bf6_kernel<Cfg, 1>, gemm_bf6_kernel<Cfg, 2>, gemm_bf6_kernel<Cfg, 3>,
+                               gemm_bf6_kernel<Cfg, 4>};
     constexpr int kMaxDevices = 64;
     static bool attr_done[kMaxDevices][5] = {};
     int dev = 0;
     if (hipGetDevice(&dev) != hipSuccess || dev < 0 || dev >= kMaxDevices) return fail(VDMQ_ELAUNCH, "no current HIP device");
     if (!attr_done[dev][which]) {
         hipError_t e = hipFuncSetAttribute(reinterpret_cast<const void *>(kernels[which]), hipFuncAttributeMaxDynamicSharedMemorySize,
-                                           kLdsBytes);
-        if (e != hipSuccess) return fail(VDMQ_ELAUNCH, "hipFuncSetAttribute(%d bytes of LDS): %s", kLdsBytes, hipGetErrorString(e));
+                                           Cfg::kLdsBytes);
+        if (e != hipSuccess) return fail(VDMQ_ELAUNCH, "hipFuncSetAttribute(%d bytes of LDS): %s", Cfg::kLdsBytes, hipGetErrorString(e));
         attr_done[dev][which] = true;
     }
-    hipLaunchKernelGGL(kernels[which], grid, block, kLdsBytes, s, xblocks, wblocks, ascale, wscale, bias, out, acc_out,
+    hipLaunchKernelGGL(kernels[which], grid, block, Cfg::kLdsBytes, s, xblocks, wblocks, ascale, wscale, bias, out, acc_out,
                        static_cast<int>(M), static_cast<int>(N), static_cast<int>(bf6_kblocks(K)), ldo, tm, tail);
     return check_launch("gemm_bf6_kernel");
+}
+
+}  // namespace
+
+int launch_gemm_bf6(const uint8_t *xblocks, const __half *ascale, const uint8_t *wblocks, const __half *wscale, const __half *bias,
+                    __half *out, int32_t *acc_out, int64_t M, int64_t N, int64_t K, int64_t ldo, const GemmTail &tail, hipStream_t s) {
+    if (M == 0 || N == 0) return VDMQ_OK;
+    return launch_bf6_cfg<Bf6Big>(xblocks, ascale, wblocks, wscale, bias, out, acc_out, M, N, K, ldo, tail, s);
 }
 
 }  // namespace vdmq
