@@ -47,6 +47,9 @@ constexpr int kBlkPlaneB = 1024;                /* offset of the 8-byte plane */
 constexpr int KS = 128;                         /* K step: two k-blocks per stage */
 constexpr int kRbStage = (KS / 64) * kBlkBytes; /* bytes of one row-block per stage */
 constexpr int kXcds = 8;
+// per wave, beside the stage ring: the fp16 token scales of its 128 rows, the channel scales and the bias of its 64
+// columns, fetched when the tile starts so that the epilogue does not wait for them
+constexpr int kSideAs = 0, kSideWs = 256, kSideBias = 384, kSideBytes = 512;
 
 // Tile configuration.  BM token rows x BN weight rows per workgroup, WAVES_M x WAVES_N waves (a wave owns
 // 128 x 64: 4 x 2 MFMA tiles), STAGES ring slots of (BM + BN) / 32 row-blocks, OCC workgroups per CU.  One
@@ -60,14 +63,15 @@ struct Bf6Cfg {
     static constexpr int MI = BM / 32 / kWavesM, NI = BN / 32 / kWavesN; /* 32-row blocks per wave: token, weight */
     static constexpr int kStageBytes = (BM + BN) / 32 * kRbStage;
     static constexpr int kLoads = kStageBytes / 1024 / kWaves;
-    static constexpr int kLdsBytes = S * kStageBytes;
+    static constexpr int kRingBytes = S * kStageBytes;
+    static constexpr int kLdsBytes = kRingBytes + kWaves * kSideBytes; /* stage ring + the waves' scale and bias vectors */
     static constexpr int kWaveN = NI * 32;
     static constexpr int kStageRowBytes = kWaveN * 2 + 16; /* epilogue staging: fp16 strip rows padded by 16 bytes */
     static constexpr int kStagingBytes = 32 * kStageRowBytes;
     static constexpr int kPiecesPerRow = kWaveN / 8;
     static constexpr int kPerLog2 = BM == 256 ? 5 : 6; /* tiles per super-tile: what an XCD's 32 CUs hold at once */
     static_assert(MI == 4 && NI == 2, "the schedule below is written for 128 x 64 wave tiles");
-    static_assert(kStagingBytes * kWaves <= kLdsBytes, "epilogue staging reuses the stage ring");
+    static_assert(kStagingBytes * kWaves <= kRingBytes, "epilogue staging reuses the stage ring");
     static_assert(kStageBytes % (1024 * kWaves) == 0, "stage splits evenly over the waves");
     static_assert(kLoads * (S - 1) < 64, "vmcnt is a 6-bit counter");
     static_assert(kLdsBytes * kOcc <= 160 * 1024, "the CU's LDS holds OCC workgroups");
@@ -169,6 +173,16 @@ __global__ __launch_bounds__(Cfg::kWaves * 64, (Cfg::kWaves * Cfg::kOcc + 3) / 4
                 acc[ni][mi] = __builtin_amdgcn_mfma_scale_f32_32x32x64_f8f6f4(wf[ni], xf[mi], acc[ni][mi], 3, 3, 0, 0, 0, 0); /* bf6 x bf6, no scaling */
     };
     const int ksteps = kblocks / (KS / 64);
+    const int m0 = tile_m * BM, n0 = tile_n * BN, wm0 = wm * MI * 32, wn0 = wn * NI * 32;
+    uint8_t *side = lds + Cfg::kRingBytes + wave * kSideBytes;
+    _Float16 side_as[2] = {0, 0}, side_ws = 0, side_bias = 0;
+    if (!ACC_OUT) { /* older than the stage loads below: complete before the first of those is waited for */
+        const _Float16 *as_p = reinterpret_cast<const _Float16 *>(ascale);
+        side_as[0] = as_p[min(m0 + wm0 + lane, M - 1)];
+        side_as[1] = as_p[min(m0 + wm0 + 64 + lane, M - 1)];
+        side_ws = reinterpret_cast<const _Float16 *>(wscale)[min(n0 + wn0 + lane, N - 1)];
+        if (bias != nullptr) side_bias = reinterpret_cast<const _Float16 *>(bias)[min(n0 + wn0 + lane, N - 1)];
+    }
 #pragma unroll
     for (int s = 0; s < S; ++s)
         if (s < ksteps) issue(s, s);
@@ -177,6 +191,12 @@ __global__ __launch_bounds__(Cfg::kWaves * 64, (Cfg::kWaves * Cfg::kOcc + 3) / 4
     else
         __builtin_amdgcn_s_waitcnt(waitcnt_imm(0, 15));
     lds_barrier();
+    if (!ACC_OUT) { /* wave-private: the epilogue's reads follow these writes in the wave's own LDS queue */
+        *reinterpret_cast<_Float16 *>(side + kSideAs + lane * 2) = side_as[0];
+        *reinterpret_cast<_Float16 *>(side + kSideAs + 128 + lane * 2) = side_as[1];
+        *reinterpret_cast<_Float16 *>(side + kSideWs + lane * 2) = side_ws;
+        *reinterpret_cast<_Float16 *>(side + kSideBias + lane * 2) = side_bias;
+    }
     v8i wfa[NI], xfa[MI], wfb[NI], xfb[MI];
     read(wfa, xfa, lds, 0);
     int cur = 0;
@@ -207,7 +227,6 @@ __global__ __launch_bounds__(Cfg::kWaves * 64, (Cfg::kWaves * Cfg::kOcc + 3) / 4
     for (; kt < ksteps; ++kt) k_step(kt, std::false_type{});
 
     const int l32 = lane & 31, lh = lane >> 5;
-    const int m0 = tile_m * BM, n0 = tile_n * BN, wm0 = wm * MI * 32, wn0 = wn * NI * 32;
     if (ACC_OUT) {
 #pragma unroll
         for (int mi = 0; mi < MI; ++mi) {
@@ -231,23 +250,21 @@ __global__ __launch_bounds__(Cfg::kWaves * 64, (Cfg::kWaves * Cfg::kOcc + 3) / 4
     // one 32-row strip at a time is transposed through LDS so that rows leave as whole 128-byte lines
     constexpr int PR = kPiecesPerRow, RS = kStageRowBytes;
     uint8_t *stg = lds + wave * kStagingBytes;
-    const _Float16 *as_p = reinterpret_cast<const _Float16 *>(ascale);
     float wsf[NI][4][4];
 #pragma unroll
     for (int ni = 0; ni < NI; ++ni)
 #pragma unroll
         for (int rg = 0; rg < 4; ++rg) {
-            const int n = n0 + wn0 + ni * 32 + rg * 8 + lh * 4;
-            const f16x4 w4 = *reinterpret_cast<const f16x4 *>(wscale + min(n, N - 4));
+            const f16x4 w4 = *reinterpret_cast<const f16x4 *>(side + kSideWs + (ni * 32 + rg * 8 + lh * 4) * 2);
 #pragma unroll
             for (int e = 0; e < 4; ++e) wsf[ni][rg][e] = static_cast<float>(w4[e]);
         }
     const int ncol = n0 + wn0 + (lane % PR) * 8;
     f16x8 bv = {0, 0, 0, 0, 0, 0, 0, 0};
-    if (bias != nullptr && ncol < N) bv = *reinterpret_cast<const f16x8 *>(bias + ncol);
+    if (bias != nullptr) bv = *reinterpret_cast<const f16x8 *>(side + kSideBias + (lane % PR) * 16);
 #pragma unroll
     for (int mi = 0; mi < MI; ++mi) {
-        const float as = static_cast<float>(as_p[min(m0 + wm0 + mi * 32 + l32, M - 1)]);
+        const float as = static_cast<float>(*reinterpret_cast<const _Float16 *>(side + kSideAs + (mi * 32 + l32) * 2));
         // gate and residual pieces of this strip, requested before the strip is converted and staged
         f16x8 gv[PR / 2], rv[PR / 2];
 #pragma unroll
