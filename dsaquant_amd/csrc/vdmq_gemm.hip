@@ -86,7 +86,11 @@ struct GemmCfg {
     static constexpr int kNI = kWaveN / 32;
     static constexpr int kRows = BM + BN;
     static constexpr int kStageBytes = kRows * kRowBytes;
-    static constexpr int kLdsBytes = kStageBytes * STAGES;
+    static constexpr int kRingBytes = kStageBytes * STAGES;
+    // beside the ring, per wave: the fp16 token scales of its rows, the channel scales and the bias of its columns,
+    // fetched when the tile starts so that the fp16 epilogue does not wait for them
+    static constexpr int kSideAs = 0, kSideWs = 2 * kWaveM, kSideBias = 2 * kWaveM + 2 * kWaveN, kSideBytes = 2 * kWaveM + 4 * kWaveN;
+    static constexpr int kLdsBytes = kRingBytes + kWaves * kSideBytes;
     // one direct-to-LDS instruction of one wave fills kDmaRows rows (1 KiB)
     static constexpr int kRowBlocks = kRows / kDmaRows;
     static constexpr int kLoads = kRowBlocks / kWaves; /* per wave (= per lane) and stage */
@@ -95,6 +99,7 @@ struct GemmCfg {
     static constexpr int kStagingBytes = 32 * kStageRowBytes;
     static constexpr int kPiecesPerRow = kWaveN / 8; /* 16-byte pieces of one strip row */
     static_assert(kStagingBytes * kWaves <= kStageBytes * STAGES_, "epilogue staging reuses the stage ring");
+    static_assert(kWaveN <= 64, "one lane per column fetches the channel scale and the bias");
     static_assert(kRowBlocks % kWaves == 0, "row blocks must divide evenly over the waves");
     static_assert(BN % kDmaRows == 0 && kWaveM % 32 == 0 && kWaveN % 32 == 0, "tile shape");
     static_assert(kLoads * (STAGES - 1) < 64, "vmcnt is a 6-bit counter");
@@ -301,6 +306,16 @@ __global__ __launch_bounds__(Cfg::kThreads, Cfg::kOccupancy * Cfg::kWaves / 4) v
     const bool k_reverse = tmap.contig && ((blockIdx.x / (kXcds * kGroupM * kGroupN)) & 1) != 0;
     auto kpos = [&](int kt) { return k_reverse ? ksteps - 1 - kt : kt; };
 
+    uint8_t *side = lds + Cfg::kRingBytes + wave * Cfg::kSideBytes;
+    const bool f16_out = !ACC_OUT && out_dtype == VDMQ_OUT_F16;
+    _Float16 side_as[(Cfg::kWaveM + 63) / 64] = {}, side_ws = 0, side_bias = 0;
+    if (f16_out) { /* older than the stage loads below: complete before the first of those is waited for */
+#pragma unroll
+        for (int i = 0; i < (Cfg::kWaveM + 63) / 64; ++i)
+            side_as[i] = reinterpret_cast<const _Float16 *>(ascale)[min(m0 + wm0 + i * 64 + lane, M - 1)];
+        side_ws = reinterpret_cast<const _Float16 *>(wscale)[min(n0 + wn0 + (lane & (Cfg::kWaveN - 1)), N - 1)];
+        if (bias != nullptr) side_bias = reinterpret_cast<const _Float16 *>(bias)[min(n0 + wn0 + (lane & (Cfg::kWaveN - 1)), N - 1)];
+    }
     // prologue: fill the ring (as far as K reaches), wait for stage 0
 #pragma unroll
     for (int s = 0; s < S; ++s)
@@ -311,6 +326,15 @@ __global__ __launch_bounds__(Cfg::kThreads, Cfg::kOccupancy * Cfg::kWaves / 4) v
         __builtin_amdgcn_s_waitcnt(waitcnt_imm(0, 15));
     lds_barrier();
     VDMQ_STAMP(1);
+    if (f16_out) { /* wave-private: the epilogue's reads follow these writes in the wave's own LDS queue */
+#pragma unroll
+        for (int i = 0; i < (Cfg::kWaveM + 63) / 64; ++i)
+            if (i * 64 + lane < Cfg::kWaveM) *reinterpret_cast<_Float16 *>(side + Cfg::kSideAs + (i * 64 + lane) * 2) = side_as[i];
+        if (lane < Cfg::kWaveN) {
+            *reinterpret_cast<_Float16 *>(side + Cfg::kSideWs + lane * 2) = side_ws;
+            *reinterpret_cast<_Float16 *>(side + Cfg::kSideBias + lane * 2) = side_bias;
+        }
+    }
 
     // Software pipeline.  fa/fb hold the raw LDS fragments of the 128-bit read
     // being consumed and of the next one; `lo` holds the widened first half of
@@ -397,29 +421,26 @@ __global__ __launch_bounds__(Cfg::kThreads, Cfg::kOccupancy * Cfg::kWaves / 4) v
         // kWaveN outputs leave as whole 128-byte lines.
         constexpr int PR = Cfg::kPiecesPerRow, RS = Cfg::kStageRowBytes;
         uint8_t *stg = lds + wave * Cfg::kStagingBytes;
-        const _Float16 *as_p = reinterpret_cast<const _Float16 *>(ascale);
         // channel scales of this wave's columns as fp32, once per tile
         float wsf[Cfg::kNI][4][4];
 #pragma unroll
         for (int ni = 0; ni < Cfg::kNI; ++ni)
 #pragma unroll
             for (int rg = 0; rg < 4; ++rg) {
-                const int n = n0 + wn0 + ni * 32 + rg * 8 + lh * 4;
-                const f16x4 w4 = *reinterpret_cast<const f16x4 *>(wscale + min(n, N - 4));
+                const f16x4 w4 = *reinterpret_cast<const f16x4 *>(side + Cfg::kSideWs + (ni * 32 + rg * 8 + lh * 4) * 2);
 #pragma unroll
                 for (int e = 0; e < 4; ++e) wsf[ni][rg][e] = static_cast<float>(w4[e]);
             }
         const int ncol = n0 + wn0 + (lane % PR) * 8;
         f16x8 bv = {0, 0, 0, 0, 0, 0, 0, 0};
-        if (bias != nullptr && ncol < N) bv = *reinterpret_cast<const f16x8 *>(bias + ncol);
+        if (bias != nullptr) bv = *reinterpret_cast<const f16x8 *>(side + Cfg::kSideBias + (lane % PR) * 16);
 #pragma unroll
         for (int mi = 0; mi < Cfg::kMI; ++mi) {
-            const int m = m0 + wm0 + mi * 32 + l32;
             // The accumulator holds 256*acc.  float(256*acc) = 256*float(acc) exactly (|acc| < 2^24),
             // and scaling the token scale by 2^-8 is exact too, so
             //   float(256*acc) * fl((as/256) * ws) == fl(float(acc) * fl(as * ws))   bit for bit
             // (no under- or overflow: as*ws/256 >= 2^-56, |256*acc| < 2^31).
-            const float as = static_cast<float>(as_p[min(m, M - 1)]) * 0.00390625f;
+            const float as = static_cast<float>(*reinterpret_cast<const _Float16 *>(side + Cfg::kSideAs + (mi * 32 + l32) * 2)) * 0.00390625f;
             // gate and residual pieces of this strip, requested before the strip is converted and
             // staged so that their latency runs under that work
             f16x8 gv[PR / 2], rv[PR / 2];
