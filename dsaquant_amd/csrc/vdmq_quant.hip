@@ -401,6 +401,17 @@ __global__ __launch_bounds__((FMT == 1 ? kBf6Rows : kRowsPerBlock) * kWaveSize) 
     }
 }
 
+// Chunk counts the fused LayerNorm kernel is instantiated for (launch_ln_impl picks the first that covers the row):
+// with NCH chunks the row is longer than the next smaller count, so the chunks below that one are complete in every
+// lane and need no bounds test.
+constexpr int ln_full_chunks(int nch) {
+    constexpr int counts[] = {1, 2, 3, 4, 6, 8, 10, 12, 16, 20, 24, 32};
+    int prev = 0;
+    for (int n : counts)
+        if (n < nch) prev = n;
+    return prev;
+}
+
 __device__ __forceinline__ float wave_sum(float v) {
 #pragma unroll
     for (int off = 32; off > 0; off >>= 1) v += __shfl_xor(v, off, 64);
@@ -438,38 +449,50 @@ __global__ __launch_bounds__((FMT == 1 ? kBf6Rows : kRowsPerBlock) * kWaveSize) 
 
     u32x4 v[NCH];
     float sum = 0.0f;
+    float one = 1.0f; /* a multiplier the compiler cannot see through: fma(x, one, y) stays a fused multiply-add */
+    asm volatile("" : "+s"(one));
 #pragma unroll
     for (int c = 0; c < NCH; ++c) {
         const int k0 = c * 512 + lane * 8;
-        v[c] = k0 < K ? __builtin_nontemporal_load(src + c * 64 + lane) : u32x4{0u, 0u, 0u, 0u};
+        v[c] = c < ln_full_chunks(NCH) || k0 < K ? __builtin_nontemporal_load(src + c * 64 + lane) : u32x4{0u, 0u, 0u, 0u};
         const uint32_t w[4] = {v[c].x, v[c].y, v[c].z, v[c].w};
 #pragma unroll
         for (int i = 0; i < 4; ++i) {
             const f16x2 h = __builtin_bit_cast(f16x2, w[i]);
-            sum += static_cast<float>(h[0]) + static_cast<float>(h[1]); /* padding adds zeros */
+            // fma(x, 1, s) = fl(x + s) as one v_fma_mix_f32, which reads the fp16 value directly (padding adds zeros)
+            sum = __builtin_fmaf(static_cast<float>(h[0]), one, sum);
+            sum = __builtin_fmaf(static_cast<float>(h[1]), one, sum);
         }
     }
     const float mean = wave_sum(sum) / static_cast<float>(K);
+    // Each pass converts the fp16 row again: the compiler would otherwise keep the 8 * NCH converted floats of one
+    // pass for the next (80 registers for a 5120-wide row, a workgroup per CU less); the empty asm makes the row
+    // a new value for it.
+#pragma unroll
+    for (int c = 0; c < NCH; ++c) asm volatile("" : "+v"(v[c]));
     float sq = 0.0f;
 #pragma unroll
     for (int c = 0; c < NCH; ++c) {
         const int k0 = c * 512 + lane * 8;
-        if (k0 < K) {
+        if (c < ln_full_chunks(NCH) || k0 < K) {
             const uint32_t w[4] = {v[c].x, v[c].y, v[c].z, v[c].w};
 #pragma unroll
             for (int i = 0; i < 4; ++i) {
                 const f16x2 h = __builtin_bit_cast(f16x2, w[i]);
-                const float d0 = static_cast<float>(h[0]) - mean, d1 = static_cast<float>(h[1]) - mean;
-                sq += d0 * d0 + d1 * d1;
+                const float d0 = __builtin_fmaf(static_cast<float>(h[0]), one, -mean), d1 = __builtin_fmaf(static_cast<float>(h[1]), one, -mean);
+                sq = __builtin_fmaf(d0, d0, sq);
+                sq = __builtin_fmaf(d1, d1, sq);
             }
         }
     }
     const float rstd = 1.0f / __builtin_sqrtf(wave_sum(sq) / static_cast<float>(K) + eps);
+#pragma unroll
+    for (int c = 0; c < NCH; ++c) asm volatile("" : "+v"(v[c]));
 
 #pragma unroll
     for (int c = 0; c < NCH; ++c) {
         const int k0 = c * 512 + lane * 8;
-        if (k0 < K) {
+        if (c < ln_full_chunks(NCH) || k0 < K) {
             const u32x4 a4 = pa[c * 64 + lane], b4 = pb[c * 64 + lane];
             const uint32_t w[4] = {v[c].x, v[c].y, v[c].z, v[c].w};
             const uint32_t aw[4] = {a4.x, a4.y, a4.z, a4.w}, bw[4] = {b4.x, b4.y, b4.z, b4.w};
@@ -478,7 +501,8 @@ __global__ __launch_bounds__((FMT == 1 ? kBf6Rows : kRowsPerBlock) * kWaveSize) 
             for (int i = 0; i < 4; ++i) {
                 const f16x2 h = __builtin_bit_cast(f16x2, w[i]);
                 const f16x2 a = __builtin_bit_cast(f16x2, aw[i]), b = __builtin_bit_cast(f16x2, bw[i]);
-                const float n0 = (static_cast<float>(h[0]) - mean) * rstd, n1 = (static_cast<float>(h[1]) - mean) * rstd;
+                const float n0 = __builtin_fmaf(static_cast<float>(h[0]), one, -mean) * rstd;
+                const float n1 = __builtin_fmaf(static_cast<float>(h[1]), one, -mean) * rstd;
                 f16x2 r;
                 if (LNMODE == VDMQ_LN_MODULATE) {
                     const f16x2 ln = {static_cast<_Float16>(n0), static_cast<_Float16>(n1)};
