@@ -77,8 +77,10 @@ __device__ __forceinline__ uint32_t quantize_word_fast(u32x4 v, float rscale) {
 #pragma unroll
     for (int i = 0; i < 4; ++i) {
         const f16x2 h = __builtin_bit_cast(f16x2, w[i]);
-        float t0 = __builtin_amdgcn_fmed3f(static_cast<float>(h[0]) * rscale, -8.0f, 7.0f);
-        float t1 = __builtin_amdgcn_fmed3f(static_cast<float>(h[1]) * rscale, -8.0f, 7.0f);
+        // fma(x, r, +0) = fl(x * r) (a product of -0 becomes +0, which rounds to the same integer): one
+        // v_fma_mix_f32 reading the fp16 value, instead of a conversion and a multiplication
+        float t0 = __builtin_amdgcn_fmed3f(__builtin_fmaf(static_cast<float>(h[0]), rscale, 0.0f), -8.0f, 7.0f);
+        float t1 = __builtin_amdgcn_fmed3f(__builtin_fmaf(static_cast<float>(h[1]), rscale, 0.0f), -8.0f, 7.0f);
         acc += __float_as_uint(t0 + kMagic) << (8 * i);
         acc += __float_as_uint(t1 + kMagic) << (8 * i + 4);
     }
@@ -297,8 +299,8 @@ __device__ __forceinline__ void quantize_held_row_bf6(u32x4 (&v)[NCH], int lane,
 #pragma unroll
                 for (int i = 0; i < 4; ++i) {
                     const f16x2 h = __builtin_bit_cast(f16x2, w[i]);
-                    q[u * 8 + i * 2] = static_cast<_Float16>(__builtin_rintf(__builtin_amdgcn_fmed3f(static_cast<float>(h[0]) * rscale, -8.0f, 7.0f)));
-                    q[u * 8 + i * 2 + 1] = static_cast<_Float16>(__builtin_rintf(__builtin_amdgcn_fmed3f(static_cast<float>(h[1]) * rscale, -8.0f, 7.0f)));
+                    q[u * 8 + i * 2] = static_cast<_Float16>(__builtin_rintf(__builtin_amdgcn_fmed3f(__builtin_fmaf(static_cast<float>(h[0]), rscale, 0.0f), -8.0f, 7.0f)));
+                    q[u * 8 + i * 2 + 1] = static_cast<_Float16>(__builtin_rintf(__builtin_amdgcn_fmed3f(__builtin_fmaf(static_cast<float>(h[1]), rscale, 0.0f), -8.0f, 7.0f)));
                 }
             }
         } else {
