@@ -47,6 +47,16 @@ int launch_gemm(const uint8_t *qact, const __half *ascale, const uint8_t *wq, co
                 hipStream_t stream);
 
 // bf6 matrix path (vdmq_bf6.hip)
+constexpr int kBf6PanelKb = 384; /* one 64-deep k-block of an 8-row panel of a bf6 operand, bytes */
+// Byte offset, in an operand of `kblocks` k-blocks, of the 16-byte (part_b = false) or 8-byte (true) part of the
+// 192-bit string that holds row `row`, k = 64 * kb + 32 * h ... + 31.  Rows are stored in panels of eight, a panel
+// k-block after k-block, a k-block as [h = 0: 8 rows x 16 B][h = 1: 8 x 16 B][h = 0: 8 x 8 B][h = 1: 8 x 8 B]: what the
+// quantizer's eight-row workgroup writes is one contiguous stream, and the GEMM still fetches whole 128-byte lines.
+__host__ __device__ __forceinline__ int64_t bf6_piece(int64_t row, int kb, int h, bool part_b, int kblocks) {
+    return (row >> 3) * kblocks * kBf6PanelKb + static_cast<int64_t>(kb) * kBf6PanelKb +
+           (part_b ? 256 + h * 64 + (row & 7) * 8 : h * 128 + (row & 7) * 16);
+}
+
 int64_t bf6_kblocks(int64_t K);
 int64_t bf6_bytes(int64_t rows, int64_t K);
 int launch_nibbles_to_bf6(const uint8_t *native, int64_t rows, int64_t K, uint8_t *blocks, hipStream_t stream);

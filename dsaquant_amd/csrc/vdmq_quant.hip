@@ -204,9 +204,9 @@ __device__ __forceinline__ void quantize_held_row(const u32x4 (&v)[NCH], int lan
     if (lane == 0) scale_h[row] = sh;
 }
 
-// The same, written as bf6 blocks (the operand form of the bf6 GEMM, see vdmq_bf6.hip): 32 rows x 64 k
-// per 1536-byte block, lane (row % 32) + 32 * h of a block holding the 32 six-bit E3M2 codes of
-// k = 64 * kb + 32 * h + e as one 192-bit string.  A lane needs 32 consecutive k for that, but holds
+// The same, written as bf6 blocks (the operand form of the bf6 GEMM, see vdmq_bf6.hip): per row and 32
+// consecutive k = 64 * kb + 32 * h + e one 192-bit string of six-bit E3M2 codes, stored by panels of 8 rows
+// (bf6_piece in vdmq_internal.h).  A lane needs 32 consecutive k for that, but holds
 // 8 per chunk: four chunks at a time go through a wave-private LDS buffer in k order (16 bytes of
 // padding per 256 keep both the 16-byte writes and the 64-byte-per-lane reads free of bank
 // conflicts) and come back as 32 consecutive fp16 per lane.  Those are scaled, rounded to integers
@@ -273,8 +273,6 @@ __device__ __forceinline__ void quantize_held_row_bf6(u32x4 (&v)[NCH], int lane,
     // threads write the eight rows' parts of one string slot, 128 (and 64) contiguous bytes
     const int t = wave * kWaveSize + lane, srow = t % kBf6Rows, sidx = t / kBf6Rows;
     const int64_t grow = row0 + srow;
-    uint8_t *rowblk = blocks + (grow / 32) * static_cast<int64_t>(kblocks) * 1536;
-    const int slot = static_cast<int>(grow % 32);
     constexpr int NG = (NCH + 3) / 4;
 #pragma unroll
     for (int g = 0; g < NG; ++g) {
@@ -320,7 +318,8 @@ __device__ __forceinline__ void quantize_held_row_bf6(u32x4 (&v)[NCH], int lane,
         }
         const u32x6 str = __builtin_amdgcn_cvt_scalef32_pk32_bf6_f16(q, 1.0f);
         // per-lane stores would scatter 16-byte pieces over 64 cache lines per instruction (measured: 2x
-        // slower than the HBM-bound int4 quantizer): collect the workgroup's strings in LDS instead
+        // slower than the HBM-bound int4 quantizer): collect the workgroup's strings in LDS instead -- its
+        // eight rows are one panel, whose 128-byte and 64-byte runs of one k-block are adjacent in memory
         const int copy = phase & 1;
         ++phase;
         *reinterpret_cast<u32x4 *>(lds.part_a[copy][wave] + lane * 16) = u32x4{str[0], str[1], str[2], str[3]};
@@ -328,10 +327,11 @@ __device__ __forceinline__ void quantize_held_row_bf6(u32x4 (&v)[NCH], int lane,
         __syncthreads(); /* also orders this group's writes after every thread's reads of the group before last */
         const int k0 = 2048 * g + 32 * sidx;
         if (k0 < Kb && grow < M) {
-            uint8_t *blk = rowblk + static_cast<int64_t>(k0 >> 6) * 1536;
-            const int l = slot + 32 * ((k0 >> 5) & 1);
-            *reinterpret_cast<u32x4 *>(blk + l * 16) = *reinterpret_cast<const u32x4 *>(lds.part_a[copy][srow] + sidx * 16);
-            *reinterpret_cast<u32x2 *>(blk + 1024 + l * 8) = *reinterpret_cast<const u32x2 *>(lds.part_b[copy][srow] + sidx * 8);
+            const int kb = k0 >> 6, h = (k0 >> 5) & 1;
+            *reinterpret_cast<u32x4 *>(blocks + bf6_piece(grow, kb, h, false, kblocks)) =
+                *reinterpret_cast<const u32x4 *>(lds.part_a[copy][srow] + sidx * 16);
+            *reinterpret_cast<u32x2 *>(blocks + bf6_piece(grow, kb, h, true, kblocks)) =
+                *reinterpret_cast<const u32x2 *>(lds.part_b[copy][srow] + sidx * 8);
         }
     }
 }

@@ -171,9 +171,11 @@ int vdmq_linear_ln_w4a4(const void *x, int64_t M, int64_t K, int64_t ldx, float 
  * gfx950 multiplies 6-bit floats (E3M2) at twice its int8 rate, E3M2 holds every
  * int4 value exactly and fp32 accumulation of their products is exact for
  * K <= 65536, so the same GEMM can run on v_mfma_f32_32x32x64_f8f6f4 with
- * bit-identical results.  Operands are "bf6 blocks": 32 rows x 64 k per
- * 1536-byte block, row-block major, rows padded to 32 and K to 128 with zeros
- * (vdmq_bf6_bytes gives the size).  vdmq_native_to_bf6 converts a native int4
+ * bit-identical results.  Operands are "bf6 blocks": per row and 32 consecutive
+ * k one 192-bit string of six-bit codes, stored by panels of 8 rows (a panel holds
+ * its 64-deep k-blocks one after the other, 384 bytes each: [k half 0: 8 rows x
+ * 16 B][half 1: 8 x 16 B][half 0: 8 x 8 B][half 1: 8 x 8 B]), rows padded to 32
+ * and K to 128 with zeros (vdmq_bf6_bytes gives the size).  vdmq_native_to_bf6 converts a native int4
  * buffer (weights once per module; activations per call unless the quantizer
  * writes blocks itself); vdmq_gemm_w4a4_bf6 is vdmq_gemm_w4a4 on such operands
  * (fp16 output only), vdmq_gemm_w4a4_bf6_acc the int32 accumulator view.

@@ -311,20 +311,22 @@ def np_bf6_decode(code: np.ndarray) -> np.ndarray:
 
 
 def np_unpack_bf6_blocks(blocks: np.ndarray, rows: int, K: int) -> np.ndarray:
-    """bf6 block buffer (u8) -> values float64 [rows, K].  Layout: blocks of 32 rows x 64 k, row-block major, 1536
-    bytes each = [64 lanes x 16 bytes][64 lanes x 8 bytes]; lane (r % 32) + 32 h holds, as one 192-bit little-endian
-    string, the 32 six-bit codes of k = 64 kb + 32 h + e (code e at bits 6e..6e+5).  Also checks the zero padding."""
+    """bf6 operand buffer (u8) -> values float64 [rows, K].  Layout: rows padded to 32 and stored in panels of 8, K padded
+    to 128 and cut into k-blocks of 64; a panel holds its k-blocks one after the other, 384 bytes each =
+    [h = 0: 8 rows x 16 B][h = 1: 8 rows x 16 B][h = 0: 8 rows x 8 B][h = 1: 8 rows x 8 B].  A row's 16-byte and 8-byte
+    parts for (k-block, h) form one 192-bit little-endian string holding the 32 six-bit codes of k = 64 kb + 32 h + e
+    (code e at bits 6e..6e+5) -- the operand registers of lane (row % 32) + 32 h of v_mfma_f32_32x32x64_f8f6f4.
+    Also checks the zero padding."""
     kblocks = (K + 127) // 128 * 2
-    rbs = (rows + 31) // 32
-    b = blocks.reshape(rbs, kblocks, 1536)
-    lo = b[:, :, :1024].reshape(rbs, kblocks, 64, 16)
-    hi = b[:, :, 1024:].reshape(rbs, kblocks, 64, 8)
-    s = np.concatenate([lo, hi], axis=3)                      # 24 bytes per lane
-    bits = np.unpackbits(s, axis=3, bitorder="little")        # 192 bits per lane
-    codes = (bits.reshape(rbs, kblocks, 64, 32, 6) * (1 << np.arange(6))).sum(axis=4)
-    vals = np_bf6_decode(codes)                               # [rb, kb, lane, e]
-    vals = vals.reshape(rbs, kblocks, 2, 32, 32)              # lane = 32 h + r
-    full = vals.transpose(0, 3, 1, 2, 4).reshape(rbs * 32, kblocks * 64)
+    panels = (rows + 31) // 32 * 4
+    b = blocks.reshape(panels, kblocks, 384)
+    lo = b[:, :, :256].reshape(panels, kblocks, 2, 8, 16)
+    hi = b[:, :, 256:].reshape(panels, kblocks, 2, 8, 8)
+    s = np.concatenate([lo, hi], axis=4)                      # [panel, kb, h, row in panel, 24 bytes]
+    bits = np.unpackbits(s, axis=4, bitorder="little")        # 192 bits
+    codes = (bits.reshape(panels, kblocks, 2, 8, 32, 6) * (1 << np.arange(6))).sum(axis=5)
+    vals = np_bf6_decode(codes)                               # [panel, kb, h, j, e]
+    full = vals.transpose(0, 3, 1, 2, 4).reshape(panels * 8, kblocks * 64)
     assert not full[rows:].any() and not full[:, K:].any(), "padding must be zero"
     return full[:rows, :K]
 

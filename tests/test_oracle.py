@@ -456,8 +456,8 @@ def test_bf6_decoder_follows_the_format_and_holds_every_int4_value():
     rows, K = 40, 192
     want = (np.add.outer(np.arange(rows), np.arange(K)) % 16 - 8).astype(np.int64)
     enc = {int(v): int(c) for c, v in zip(codes, vals) if float(v).is_integer() and -8 <= v <= 8 and not (v == 0 and c >= 32)}
-    kblocks, rbs = (K + 127) // 128 * 2, (rows + 31) // 32
-    buf = np.zeros((rbs, kblocks, 1536), np.uint8)
+    kblocks, panels = (K + 127) // 128 * 2, (rows + 31) // 32 * 4
+    buf = np.zeros((panels, kblocks, 384), np.uint8)  # panels of 8 rows; per k-block [h0 16 B x 8][h1 16 B x 8][h0 8 B x 8][h1 8 B x 8]
     for r in range(rows):
         for kb in range(K // 64):
             for h in range(2):
@@ -466,7 +466,7 @@ def test_bf6_decoder_follows_the_format_and_holds_every_int4_value():
                     c = enc[int(want[r, 64 * kb + 32 * h + e])]
                     bits[6 * e: 6 * e + 6] = [(c >> i) & 1 for i in range(6)]
                 by = np.packbits(bits, bitorder="little")
-                lane = (r % 32) + 32 * h
-                buf[r // 32, kb, lane * 16: lane * 16 + 16] = by[:16]
-                buf[r // 32, kb, 1024 + lane * 8: 1024 + lane * 8 + 8] = by[16:]
+                a, b = h * 128 + (r % 8) * 16, 256 + h * 64 + (r % 8) * 8
+                buf[r // 8, kb, a: a + 16] = by[:16]
+                buf[r // 8, kb, b: b + 8] = by[16:]
     assert np.array_equal(O.np_unpack_bf6_blocks(buf.reshape(-1), rows, K), want.astype(np.float64))
