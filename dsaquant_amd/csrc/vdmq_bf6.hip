@@ -34,22 +34,23 @@ typedef _Float16 f16x8 __attribute__((ext_vector_type(8)));
 #define VDMQ_GLOBAL_PTR(p) ((const __attribute__((address_space(1))) void *)(p))
 #define VDMQ_LDS_PTR(p) ((__attribute__((address_space(3))) void *)(p))
 
-constexpr int waitcnt_imm(int vm, int lgkm) { return (vm & 15) | ((vm >> 4) << 14) | (7 << 4) | ((lgkm & 15) << 8); }
+[[maybe_unused]] constexpr int waitcnt_imm(int vm, int lgkm) { return (vm & 15) | ((vm >> 4) << 14) | (7 << 4) | ((lgkm & 15) << 8); }
 
-__device__ __forceinline__ void lds_barrier() {
+[[maybe_unused]] __device__ __forceinline__ void lds_barrier() {
     asm volatile("" ::: "memory");
     __builtin_amdgcn_s_barrier();
     asm volatile("" ::: "memory");
 }
 
 constexpr int kBlkBytes = 1536;                 /* 32 rows x 64 k */
-constexpr int kBlkPlaneB = 1024;                /* offset of the 8-byte plane */
+[[maybe_unused]] constexpr int kBlkPlaneB = 1024;                /* offset of the 8-byte plane */
 constexpr int KS = 128;                         /* K step: two k-blocks per stage */
 constexpr int kRbStage = (KS / 64) * kBlkBytes; /* bytes of one row-block per stage */
 constexpr int kXcds = 8;
 // per wave, beside the stage ring: the fp16 token scales of its 128 rows, the channel scales and the bias of its 64
 // columns, fetched when the tile starts so that the epilogue does not wait for them
-constexpr int kSideAs = 0, kSideWs = 256, kSideBias = 384, kSideBytes = 512;
+[[maybe_unused]] constexpr int kSideAs = 0, kSideWs = 256, kSideBias = 384;
+constexpr int kSideBytes = 512;
 
 // Tile configuration.  BM token rows x BN weight rows per workgroup, WAVES_M x WAVES_N waves (a wave owns
 // 128 x 64: 4 x 2 MFMA tiles), STAGES ring slots of (BM + BN) / 32 row-blocks, OCC workgroups per CU.  One
@@ -85,7 +86,7 @@ struct Bf6TileMap {
 };
 
 // workgroup b runs on XCD b % 8; each XCD walks super-tiles (see vdmq_gemm.hip)
-__device__ __forceinline__ bool map_tile(const Bf6TileMap &tm, int bid, int &tile_m, int &tile_n) {
+[[maybe_unused]] __device__ __forceinline__ bool map_tile(const Bf6TileMap &tm, int bid, int &tile_m, int &tile_n) {
     const int xcd = bid % kXcds, slot = bid / kXcds;
     const int st = (slot >> tm.per_log2) * kXcds + xcd, j = slot & ((1 << tm.per_log2) - 1);
     if (st >= tm.total_super) return false;
@@ -94,7 +95,7 @@ __device__ __forceinline__ bool map_tile(const Bf6TileMap &tm, int bid, int &til
     return tile_m < tm.tiles_m && tile_n < tm.tiles_n;
 }
 
-__device__ __forceinline__ v8i ld_frag(const uint8_t *p, uint32_t la, uint32_t lb) {
+[[maybe_unused]] __device__ __forceinline__ v8i ld_frag(const uint8_t *p, uint32_t la, uint32_t lb) {
     const u32x4 a = *reinterpret_cast<const u32x4 *>(p + la);
     const u32x2 b = *reinterpret_cast<const u32x2 *>(p + lb);
     v8i r = {(int)a.x, (int)a.y, (int)a.z, (int)a.w, (int)b.x, (int)b.y, 0, 0}; /* the MFMA reads six registers */
@@ -123,6 +124,7 @@ __global__ __launch_bounds__(Cfg::kWaves * 64, (Cfg::kWaves * Cfg::kOcc + 3) / 4
                                                                          const __half *__restrict__ bias, __half *out,
                                                                          int32_t *__restrict__ acc_out, int M, int N, int kblocks,
                                                                          int64_t ldo, Bf6TileMap tmap, GemmTail tail) {
+#if defined(__HIP_DEVICE_COMPILE__) /* the host pass needs the kernel's stub only; it does not know the buffer builtins */
     constexpr bool ACC_OUT = OUT_MODE == 2, STREAM_OUT = OUT_MODE == 1 || OUT_MODE == 4, TAIL = OUT_MODE >= 3;
     constexpr int BM = Cfg::BM, BN = Cfg::BN, S = Cfg::S, MI = Cfg::MI, NI = Cfg::NI, kWaves = Cfg::kWaves, kWavesN = Cfg::kWavesN;
     constexpr int kLoads = Cfg::kLoads, kStageBytes = Cfg::kStageBytes;
@@ -137,7 +139,11 @@ __global__ __launch_bounds__(Cfg::kWaves * 64, (Cfg::kWaves * Cfg::kOcc + 3) / 4
     // KiB (i * kWaves + wave) of it, 16 bytes per lane.  In LDS a row-block's two k-blocks lie as the MFMA reads them,
     // [64 lanes x 16 B][64 lanes x 8 B] each; in memory the operand is stored by panels of 8 rows (bf6_piece below), so
     // every lane finds its 16 bytes -- one lane's 16-byte part or two neighbouring rows' 8-byte parts -- on its own.
-    const uint8_t *src[kLoads];
+    // The source of a load is a base the whole wave shares (the row-block's first panel) plus a scalar offset that
+    // advances with K plus a 32-bit offset per lane that never changes -- a buffer load's three address parts, so the
+    // K loop spends no vector instruction on addresses (global_load_lds wants a 64-bit address per lane).
+    __amdgpu_buffer_rsrc_t src[kLoads];
+    uint32_t lane_off[kLoads];
 #pragma unroll
     for (int i = 0; i < kLoads; ++i) {
         const int idx = i * kWaves + wave, q = idx / 3;
@@ -146,14 +152,16 @@ __global__ __launch_bounds__(Cfg::kWaves * 64, (Cfg::kWaves * Cfg::kOcc + 3) / 4
         const bool part_b = in_blk >= kBlkPlaneB;
         const int l = part_b ? (in_blk - kBlkPlaneB) / 8 : in_blk / 16; /* lane of the MFMA operand: row % 32 + 32 * h */
         const int64_t rb = q < BN / 32 ? min(tile_n * (BN / 32) + q, last_rb_n) : min(tile_m * (BM / 32) + q - BN / 32, last_rb_m);
-        src[i] = (q < BN / 32 ? W : X) + bf6_piece(rb * 32 + (l & 31), kb, l >> 5, part_b, kblocks); /* rows past M or N re-read
-                                                                                       the last row-block and are never stored */
+        // rows past M or N re-read the last row-block and are never stored; the range covers the row-block's four panels
+        src[i] = __builtin_amdgcn_make_buffer_rsrc(const_cast<uint8_t *>((q < BN / 32 ? W : X) + bf6_piece(rb * 32, 0, 0, false, kblocks)), 0,
+                                                   4 * kblocks * kBf6PanelKb, 0x00020000 /* raw buffer of dwords */);
+        lane_off[i] = static_cast<uint32_t>(bf6_piece(l & 31, kb, l >> 5, part_b, kblocks));
     }
     auto issue = [&](int kt, int slot) __attribute__((always_inline)) {
 #pragma unroll
         for (int i = 0; i < kLoads; ++i)
-            __builtin_amdgcn_global_load_lds(VDMQ_GLOBAL_PTR(src[i] + static_cast<int64_t>(kt) * (KS / 64) * kBf6PanelKb),
-                                             VDMQ_LDS_PTR(lds + slot * kStageBytes + (i * kWaves + wave) * 1024), 16, 0, 0);
+            __builtin_amdgcn_raw_ptr_buffer_load_lds(src[i], VDMQ_LDS_PTR(lds + slot * kStageBytes + (i * kWaves + wave) * 1024), 16,
+                                                     lane_off[i], kt * (KS / 64) * kBf6PanelKb, 0, 0);
     };
     const uint32_t la = lane * 16, lb = kBlkPlaneB + lane * 8;
     auto read = [&](v8i (&wf)[NI], v8i (&xf)[MI], const uint8_t *stage, int kb) __attribute__((always_inline)) {
@@ -308,6 +316,7 @@ __global__ __launch_bounds__(Cfg::kWaves * 64, (Cfg::kWaves * Cfg::kOcc + 3) / 4
             }
         }
     }
+#endif
 }
 
 // E3M2 code of an int4 value given as a two's complement nibble: sign << 5 | exponent/mantissa of |q|
