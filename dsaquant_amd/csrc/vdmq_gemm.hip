@@ -47,9 +47,9 @@ typedef _Float16 f16x8 __attribute__((ext_vector_type(8)));
 
 
 // s_waitcnt immediate for gfx9: vmcnt[3:0] | expcnt[6:4] | lgkmcnt[11:8] | vmcnt[15:14]
-constexpr int waitcnt_imm(int vm, int lgkm) { return (vm & 15) | ((vm >> 4) << 14) | (7 << 4) | ((lgkm & 15) << 8); }
+[[maybe_unused]] constexpr int waitcnt_imm(int vm, int lgkm) { return (vm & 15) | ((vm >> 4) << 14) | (7 << 4) | ((lgkm & 15) << 8); }
 
-__device__ __forceinline__ void lds_barrier() {
+[[maybe_unused]] __device__ __forceinline__ void lds_barrier() {
     asm volatile("" ::: "memory");
 #ifndef VDMQ_DBG_NOBARRIER
     __builtin_amdgcn_s_barrier();
@@ -57,7 +57,7 @@ __device__ __forceinline__ void lds_barrier() {
     asm volatile("" ::: "memory");
 }
 
-__device__ __forceinline__ v4i widen(uint32_t p0, uint32_t p1) {
+[[maybe_unused]] __device__ __forceinline__ v4i widen(uint32_t p0, uint32_t p1) {
     v4i r;
     r[0] = static_cast<int>((p0 << 4) & 0xF0F0F0F0u);
     r[1] = static_cast<int>(p0 & 0xF0F0F0F0u);
@@ -107,16 +107,21 @@ struct GemmCfg {
 
 // Issue the direct-to-LDS loads of one stage.  `woff`/`xoff` are per-lane byte
 // offsets (clamped to valid rows) from the wave-uniform bases.
+#if defined(__HIP_DEVICE_COMPILE__) /* (the host pass does not know the buffer builtins) */
+// A buffer load takes its address in three parts -- the tile's first row (shared resource), the K position (scalar
+// offset) and the lane's row and piece (vector offset, fixed for the whole tile) -- so the K loop spends no vector
+// instruction on addresses; global_load_lds wants a 64-bit address per lane.
 template <typename Cfg>
-__device__ __forceinline__ void issue_stage(const uint8_t *wbase, const uint8_t *xbase, const uint32_t (&off)[Cfg::kLoads],
-                                            uint8_t *lds_stage, int wave) {
+__device__ __forceinline__ void issue_stage(__amdgpu_buffer_rsrc_t wsrc, __amdgpu_buffer_rsrc_t xsrc, int koff,
+                                            const uint32_t (&off)[Cfg::kLoads], uint8_t *lds_stage, int wave) {
 #pragma unroll
     for (int i = 0; i < Cfg::kLoads; ++i) {
         const int rb = i * Cfg::kWaves + wave; /* wave-uniform row block */
-        const uint8_t *base = (rb * Cfg::kDmaRows < Cfg::BN) ? wbase : xbase;
-        __builtin_amdgcn_global_load_lds(VDMQ_GLOBAL_PTR(base + off[i]), VDMQ_LDS_PTR(lds_stage + rb * 1024), 16, 0, 0);
+        __builtin_amdgcn_raw_ptr_buffer_load_lds((rb * Cfg::kDmaRows < Cfg::BN) ? wsrc : xsrc, VDMQ_LDS_PTR(lds_stage + rb * 1024), 16, off[i],
+                                                 koff, 0, 0);
     }
 }
+#endif
 
 template <typename Cfg>
 __device__ __forceinline__ void read_frags(u32x4 (&wf)[Cfg::kNI], u32x4 (&xf)[Cfg::kMI], const uint8_t *lds_stage, uint32_t waddr,
@@ -188,7 +193,7 @@ struct TileMap {
     int contig;           /* 1: those contiguous runs; 0: super-tiles dealt round-robin (start[kXcds] = their number) */
 };
 
-__device__ __forceinline__ bool map_tile(const TileMap &tm, int bid, int &tile_m, int &tile_n) {
+[[maybe_unused]] __device__ __forceinline__ bool map_tile(const TileMap &tm, int bid, int &tile_m, int &tile_n) {
     const int xcd = bid % kXcds, slot = bid / kXcds;
     const int per = kGroupM * kGroupN;
     const int j = slot % per;
@@ -237,6 +242,7 @@ __global__ __launch_bounds__(Cfg::kThreads, Cfg::kOccupancy * Cfg::kWaves / 4) v
                                                                   const __half *__restrict__ bias, void *out, int out_dtype,
                                                                   int32_t *__restrict__ acc_out, int M, int N, int ldk, int64_t ldo,
                                                                   TileMap tmap, GemmTail tail) {
+#if defined(__HIP_DEVICE_COMPILE__) /* the host pass needs the kernel's stub only */
     constexpr int BM = Cfg::BM, BN = Cfg::BN, S = Cfg::STAGES, L = Cfg::kLoads;
     constexpr bool ACC_OUT = OUT_MODE == 2, STREAM_OUT = OUT_MODE == 1 || OUT_MODE == 4, TAIL = OUT_MODE >= 3;
     extern __shared__ __attribute__((aligned(1024))) uint8_t lds[];
@@ -275,8 +281,11 @@ __global__ __launch_bounds__(Cfg::kThreads, Cfg::kOccupancy * Cfg::kWaves / 4) v
             goff[i] = static_cast<uint32_t>(rr) * static_cast<uint32_t>(ldk) + piece * 16;
         }
     }
-    const uint8_t *wbase = W + static_cast<int64_t>(n0) * ldk;
-    const uint8_t *xbase = A + static_cast<int64_t>(m0) * ldk;
+    // (rows of the tile that exist) x (bytes per row) each: the offsets above stay inside
+    const __amdgpu_buffer_rsrc_t wsrc = __builtin_amdgcn_make_buffer_rsrc(const_cast<uint8_t *>(W + static_cast<int64_t>(n0) * ldk), 0,
+                                                                          min(BN, N - n0) * ldk, 0x00020000 /* raw buffer of dwords */);
+    const __amdgpu_buffer_rsrc_t xsrc = __builtin_amdgcn_make_buffer_rsrc(const_cast<uint8_t *>(A + static_cast<int64_t>(m0) * ldk), 0,
+                                                                          min(BM, M - m0) * ldk, 0x00020000);
 
     // ---- LDS -> registers: per-lane fragment addresses for the R 128-bit reads
     // (j) of a stage; lanes 32..63 take the odd pieces.  Tile row offsets are
@@ -319,7 +328,7 @@ __global__ __launch_bounds__(Cfg::kThreads, Cfg::kOccupancy * Cfg::kWaves / 4) v
     // prologue: fill the ring (as far as K reaches), wait for stage 0
 #pragma unroll
     for (int s = 0; s < S; ++s)
-        if (s < ksteps) issue_stage<Cfg>(wbase + kpos(s) * RB, xbase + kpos(s) * RB, goff, lds + s * Cfg::kStageBytes, wave);
+        if (s < ksteps) issue_stage<Cfg>(wsrc, xsrc, kpos(s) * RB, goff, lds + s * Cfg::kStageBytes, wave);
     if (ksteps >= S)
         __builtin_amdgcn_s_waitcnt(waitcnt_imm(L * (S - 1), 15));
     else
@@ -382,7 +391,7 @@ __global__ __launch_bounds__(Cfg::kThreads, Cfg::kOccupancy * Cfg::kWaves / 4) v
             mma_step<Cfg>(acc, lo);
             schedule_region<Cfg, Cfg::kNI + Cfg::kMI, 0>();
 #ifndef VDMQ_DBG_NOLOAD
-            if (STEADY && j + 1 == R) issue_stage<Cfg>(wbase + kpos(kt + S) * RB, xbase + kpos(kt + S) * RB, goff, lds + cur * Cfg::kStageBytes, wave);
+            if (STEADY && j + 1 == R) issue_stage<Cfg>(wsrc, xsrc, kpos(kt + S) * RB, goff, lds + cur * Cfg::kStageBytes, wave);
 #endif
             widen_frags<Cfg, 0>(lo, wn, xn);
             mma_step<Cfg>(acc, hi);
@@ -536,6 +545,7 @@ __global__ __launch_bounds__(Cfg::kThreads, Cfg::kOccupancy * Cfg::kWaves / 4) v
             }
         }
     }
+#endif
 }
 
 template <typename Cfg>
