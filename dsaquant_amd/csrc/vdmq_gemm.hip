@@ -6,7 +6,7 @@
 // Data path.  Both operands are row-major packed int4; a K step takes 128 or
 // 256 k (64 or 128 bytes) of every row.  A workgroup owns a BM x BN output tile and walks K through
 // a ring of LDS stages filled by 128-bit direct-to-LDS loads
-// (global_load_lds_dwordx4: no VGPR staging, no ds_write).  A lane reads 16
+// (buffer_load_dwordx4 ... lds: no VGPR staging, no ds_write).  A lane reads 16
 // bytes (32 nibbles) of one row from LDS and widens each 32-bit word p into two
 // MFMA operand registers
 //     lo = (p << 4) & 0xF0F0F0F0   (even-k nibbles, as int8 = 16*q)
