@@ -592,6 +592,28 @@ def test_bf6_accumulators_exact(M, N, K):
     assert np.array_equal(acc.cpu().numpy(), O.np_gemm_i32(qx, qw))
 
 
+def test_both_matrix_paths_agree_on_random_shapes():
+    """Thirty seeded shapes (ragged M, every multiple of 128 / 64 allowed for N / K, up to several tiles and
+    super-tiles): the accumulators of the two matrix paths are the same integers, and the first shapes are also
+    checked against the integer product on the CPU."""
+    v = vk()
+    rng = np.random.default_rng(2024)
+    for i in range(30):
+        M = int(rng.integers(1, 2600))
+        N = 128 * int(rng.integers(1, 20))
+        K = 64 * int(rng.integers(1, 70))
+        qx = rng.integers(-8, 8, (M, K), dtype=np.int8)
+        qw = rng.integers(-8, 8, (N, K), dtype=np.int8)
+        Kp = v.k_padded(K)
+        print(f"paths agree M={M} N={N} K={K}", flush=True)
+        xn, wn = t16(pack_native(qx, Kp)), t16(pack_native(qw, Kp))
+        a8 = v.gemm_int32_accumulators(xn, wn, K, path="int8")
+        a6 = v.gemm_int32_accumulators(xn, wn, K, path="bf6")
+        assert torch.equal(a8, a6), (M, N, K)
+        if i < 6:
+            assert np.array_equal(a6.cpu().numpy(), O.np_gemm_i32(qx, qw))
+
+
 def test_bf6_extreme_values_stay_exact():
     """|acc| up to 64 * K = 2^20 * 0.875 with K = 14336: exact in the fp32 accumulator."""
     v = vk()
