@@ -83,13 +83,16 @@ constexpr int kValuPerMfma = 3; /* address arithmetic and operand assembly sprea
 struct Bf6TileMap {
     int tiles_m, tiles_n, super_n, total_super;
     int group_n_log2, per_log2; /* a super-tile is (per / group_n) x group_n tiles */
+    int contig;                 /* XCD x walks the super-tiles [start[x], start[x + 1]) instead of every eighth */
+    int start[kXcds + 1];
 };
 
 // workgroup b runs on XCD b % 8; each XCD walks super-tiles (see vdmq_gemm.hip)
 [[maybe_unused]] __device__ __forceinline__ bool map_tile(const Bf6TileMap &tm, int bid, int &tile_m, int &tile_n) {
     const int xcd = bid % kXcds, slot = bid / kXcds;
-    const int st = (slot >> tm.per_log2) * kXcds + xcd, j = slot & ((1 << tm.per_log2) - 1);
-    if (st >= tm.total_super) return false;
+    const int j = slot & ((1 << tm.per_log2) - 1);
+    const int st = tm.contig ? tm.start[xcd] + (slot >> tm.per_log2) : (slot >> tm.per_log2) * kXcds + xcd;
+    if (st >= (tm.contig ? tm.start[xcd + 1] : tm.total_super)) return false;
     tile_m = ((st / tm.super_n) << (tm.per_log2 - tm.group_n_log2)) + (j >> tm.group_n_log2);
     tile_n = ((st % tm.super_n) << tm.group_n_log2) + (j & ((1 << tm.group_n_log2) - 1));
     return tile_m < tm.tiles_m && tile_n < tm.tiles_n;
@@ -157,11 +160,15 @@ __global__ __launch_bounds__(Cfg::kWaves * 64, (Cfg::kWaves * Cfg::kOcc + 3) / 4
                                                    4 * kblocks * kBf6PanelKb, 0x00020000 /* raw buffer of dwords */);
         lane_off[i] = static_cast<uint32_t>(bf6_piece(l & 31, kb, l >> 5, part_b, kblocks));
     }
+    // every other super-tile of an XCD's run walks K backwards (sums of integers: any order gives the same result)
+    const bool k_reverse = tmap.contig && (((blockIdx.x / kXcds) >> tmap.per_log2) & 1) != 0;
+    const int ksteps_all = kblocks / (KS / 64);
     auto issue = [&](int kt, int slot) __attribute__((always_inline)) {
+        const int kpos = k_reverse ? ksteps_all - 1 - kt : kt;
 #pragma unroll
         for (int i = 0; i < kLoads; ++i)
             __builtin_amdgcn_raw_ptr_buffer_load_lds(src[i], VDMQ_LDS_PTR(lds + slot * kStageBytes + (i * kWaves + wave) * 1024), 16,
-                                                     lane_off[i], kt * (KS / 64) * kBf6PanelKb, 0, 0);
+                                                     lane_off[i], kpos * (KS / 64) * kBf6PanelKb, 0, 0);
     };
     const uint32_t la = lane * 16, lb = kBlkPlaneB + lane * 8;
     auto read = [&](v8i (&wf)[NI], v8i (&xf)[MI], const uint8_t *stage, int kb) __attribute__((always_inline)) {
@@ -406,7 +413,37 @@ int launch_bf6_cfg(const uint8_t *xblocks, const __half *ascale, const uint8_t *
     if (best_load < 0 || total_super * per + kXcds * per > (int64_t(1) << 30))
         return fail(VDMQ_ESHAPE, "M x N = %lld x %lld needs more workgroups than one launch can hold", (long long)M, (long long)N);
     tm.total_super = static_cast<int>(total_super);
-    const int rounds = static_cast<int>(ceil_div(total_super, kXcds));
+    int rounds = static_cast<int>(ceil_div(total_super, kXcds));
+    // Long K and wide N: every XCD takes one contiguous run of the super-tile sequence (n fastest), the runs cut so
+    // that they hold equal numbers of tiles; consecutive super-tiles of an XCD then share their token rows and,
+    // walking K in opposite directions, re-use what the previous one left in L2 (as in vdmq_gemm.hip).  Measured at
+    // M = 75600, K = 5120: 12...14 % fewer bytes from beyond L2 and 0...2 % less time for N = 13824 and 15360; with 20
+    // tile columns or fewer (N = 5120, 3072) it fetches 4 % more and is 3...5 % slower than taking turns.
+    tm.contig = K >= 2048 && tm.tiles_n >= 48;
+    if (tm.contig) {
+        const int gn = 1 << tm.group_n_log2, gm = per >> tm.group_n_log2;
+        const int64_t sm = total_super / tm.super_n;
+        const int64_t last_m = tm.tiles_m - (sm - 1) * gm;
+        auto tiles_before = [&](int64_t st) {
+            const int64_t r = st / tm.super_n, c = st % tm.super_n;
+            const int64_t rows_here = r == sm - 1 ? last_m : gm;
+            const int64_t cols_done = c * gn < tm.tiles_n ? c * gn : tm.tiles_n;
+            return r * gm * tm.tiles_n + rows_here * cols_done;
+        };
+        const int64_t all_tiles = static_cast<int64_t>(tm.tiles_m) * tm.tiles_n;
+        tm.start[0] = 0;
+        rounds = 0;
+        for (int x = 1; x <= kXcds; ++x) {
+            const int64_t want = (all_tiles * x + kXcds - 1) / kXcds;
+            int64_t lo = tm.start[x - 1], hi = total_super;
+            while (lo < hi) {
+                const int64_t mid = (lo + hi) / 2;
+                if (tiles_before(mid) >= want) hi = mid; else lo = mid + 1;
+            }
+            tm.start[x] = x == kXcds ? static_cast<int>(total_super) : static_cast<int>(lo);
+            rounds = rounds > tm.start[x] - tm.start[x - 1] ? rounds : tm.start[x] - tm.start[x - 1];
+        }
+    }
     const dim3 grid(static_cast<unsigned>(rounds) * kXcds * per), block(Cfg::kWaves * 64);
     const bool stream_out = M * N * 2 > (int64_t(224) << 20);
     const bool has_tail = tail.gate != nullptr || tail.residual != nullptr;
