@@ -45,11 +45,11 @@ FP6_PEAK_TOPS = 10100.0  # MI355X dense FP6 MFMA, published
 # gemm: (FETCH_SIZE 1377438 KiB x 2.0 + WRITE_SIZE 1455495 KiB x 1.0) x 1024; the reads are requests leaving L2
 # (Infinity Cache or HBM), 9x the operand bytes because every XCD fetches most of its super-tile's slabs once.
 # quant: (FETCH_SIZE 538736 KiB x 2.0 + WRITE_SIZE 269920 KiB x 1.0) x 1024 = 1.0005 x the algorithmic bytes.
-# bf6 path, same method: gemm (FETCH_SIZE 2520144 KiB x 2.0 + WRITE_SIZE 1456781 KiB x 1.0) x 1024 (6-bit operands and
-# no slab re-use between super-tiles: 11x the operand bytes); quant (538745 x 2.0 + 404284 x 1.0) x 1024 = 1.0002 x
+# bf6 path, same method: gemm (FETCH_SIZE 2334456 KiB x 2.0 + WRITE_SIZE 1456095 KiB x 1.0) x 1024 (6-bit operands and
+# little slab re-use between super-tiles: 10x the operand bytes); quant (538745 x 2.0 + 404284 x 1.0) x 1024 = 1.0002 x
 # the algorithmic bytes.
 MEASURED_TRAFFIC = {("wan14b_720p_block", "int8"): {"gemm": 4311418572, "quant": 1379729408},
-                    ("wan14b_720p_block", "bf6"): {"gemm": 6652997964, "quant": 1517336576}}
+                    ("wan14b_720p_block", "bf6"): {"gemm": 6272007654, "quant": 1517336576}}
 HBM_PEAK_GBS = 8000.0    # MI355X HBM3E, published
 
 # (name, K, N) at M tokens
