@@ -594,14 +594,19 @@ def test_bf6_accumulators_exact(M, N, K):
 
 def test_both_matrix_paths_agree_on_random_shapes():
     """Thirty seeded shapes (ragged M, every multiple of 128 / 64 allowed for N / K, up to several tiles and
-    super-tiles): the accumulators of the two matrix paths are the same integers, and the first shapes are also
-    checked against the integer product on the CPU."""
+    super-tiles) and three wide ones that take the bf6 kernel's contiguous tile order with ragged edges: the
+    accumulators of the two matrix paths are the same integers, and the first shapes are also checked against the
+    integer product on the CPU."""
     v = vk()
     rng = np.random.default_rng(2024)
-    for i in range(30):
-        M = int(rng.integers(1, 2600))
-        N = 128 * int(rng.integers(1, 20))
-        K = 64 * int(rng.integers(1, 70))
+    wide = [(260, 12544, 2048), (1100, 13824, 4096), (2300, 12288, 2112)]  # >= 48 tile columns, K >= 2048: contiguous runs
+    for i in range(30 + len(wide)):
+        if i >= 30:
+            M, N, K = wide[i - 30]
+        else:
+            M = int(rng.integers(1, 2600))
+            N = 128 * int(rng.integers(1, 20))
+            K = 64 * int(rng.integers(1, 70))
         qx = rng.integers(-8, 8, (M, K), dtype=np.int8)
         qw = rng.integers(-8, 8, (N, K), dtype=np.int8)
         Kp = v.k_padded(K)
