@@ -170,7 +170,7 @@ def linear_fused(
     GEMM epilogue as the two fp16 tensor operations of the reference's
     ``hidden_states + attn_output * gate`` (dit_block.py:102, :107, :112); either may
     be omitted.  Returns a new tensor; nothing is updated in place."""
-    lib = _k._load_ext()
+    _k._load_ext()  # raises when the library is missing
     if isinstance(x, LnInput):
         if act is not None:
             raise ValueError("an activation cannot be combined with a LayerNorm input")

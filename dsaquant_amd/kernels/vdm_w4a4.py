@@ -307,7 +307,7 @@ def _act_code(act: Optional[str]) -> int:
 
 def _linear_2d(x_2d: torch.Tensor, native_w: torch.Tensor, wscale: torch.Tensor, bias: Optional[torch.Tensor], clip_ratio: float,
                out_dtype: torch.dtype = torch.float16, act: Optional[str] = None) -> torch.Tensor:
-    lib = _load_ext()
+    _load_ext()  # raises when the library is missing
     M, K = x_2d.shape
     N = native_w.shape[0]
     dev = x_2d.device

@@ -28,7 +28,6 @@ reproduces, with the reference lines it follows:
 """
 from __future__ import annotations
 
-import math
 from dataclasses import dataclass
 from typing import Dict, List, Optional, Tuple
 
