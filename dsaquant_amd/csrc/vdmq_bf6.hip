@@ -196,7 +196,8 @@ __global__ __launch_bounds__(Cfg::kWaves * 64, (Cfg::kWaves * Cfg::kOcc + 3) / 4
     const int ksteps = kblocks / (KS / 64);
     const int m0 = tile_m * BM, n0 = tile_n * BN, wm0 = wm * MI * 32, wn0 = wn * NI * 32;
     uint8_t *side = lds + Cfg::kRingBytes + wave * kSideBytes;
-    _Float16 side_as[2] = {0, 0}, side_ws = 0, side_bias = 0;
+    // (no bias: -0, the one fp16 value whose addition changes no bit of any output)
+    _Float16 side_as[2] = {0, 0}, side_ws = 0, side_bias = static_cast<_Float16>(-0.0f);
     if (!ACC_OUT) { /* older than the stage loads below: complete before the first of those is waited for */
         const _Float16 *as_p = reinterpret_cast<const _Float16 *>(ascale);
         side_as[0] = as_p[min(m0 + wm0 + lane, M - 1)];
@@ -281,8 +282,16 @@ __global__ __launch_bounds__(Cfg::kWaves * 64, (Cfg::kWaves * Cfg::kOcc + 3) / 4
             for (int e = 0; e < 4; ++e) wsf[ni][rg][e] = static_cast<float>(w4[e]);
         }
     const int ncol = n0 + wn0 + (lane % PR) * 8;
-    f16x8 bv = {0, 0, 0, 0, 0, 0, 0, 0};
-    if (bias != nullptr) bv = *reinterpret_cast<const f16x8 *>(side + kSideBias + (lane % PR) * 16);
+    const f16x8 bv = *reinterpret_cast<const f16x8 *>(side + kSideBias + (lane % PR) * 16);
+    // The stores are buffer stores: the wave's corner of the output is the resource, whose size ends with the last
+    // row below M, so rows beyond are dropped by the range check instead of being predicated.  The check looks at the
+    // vector offset only (a scalar offset is added after it), so the row goes into the vector offset: one addition
+    // per store where a 64-bit address takes a multiplication and several additions.
+    const int wave_rows = min(max(M - (m0 + wm0), 0), MI * 32);
+    if (n0 + wn0 >= N || wave_rows == 0) return; /* the same for the whole wave */
+    const __amdgpu_buffer_rsrc_t out_rsrc = __builtin_amdgcn_make_buffer_rsrc(
+        out + static_cast<int64_t>(m0 + wm0) * ldo + n0 + wn0, 0, wave_rows * static_cast<int>(ldo) * 2, 0x00020000);
+    const int out_voff = ((lane / PR) * static_cast<int>(ldo) + (lane % PR) * 8) * 2;
 #pragma unroll
     for (int mi = 0; mi < MI; ++mi) {
         const float as = static_cast<float>(*reinterpret_cast<const _Float16 *>(side + kSideAs + (mi * 32 + l32) * 2));
@@ -310,17 +319,13 @@ __global__ __launch_bounds__(Cfg::kWaves * 64, (Cfg::kWaves * Cfg::kOcc + 3) / 4
         for (int it = 0; it < PR / 2; ++it) {
             const int row = it * (64 / PR) + lane / PR;
             f16x8 hv = *reinterpret_cast<const f16x8 *>(stg + row * RS + (lane % PR) * 16);
-            if (bias != nullptr) hv += bv;
+            hv += bv;
             const int mrow = m0 + wm0 + mi * 32 + row;
-            if (TAIL && tail.gate != nullptr && mrow < M && ncol < N) hv *= gv[it];
-            if (TAIL && tail.residual != nullptr && mrow < M && ncol < N) hv = rv[it] + hv;
-            if (mrow < M && ncol < N) {
-                f16x8 *dst = reinterpret_cast<f16x8 *>(out + static_cast<int64_t>(mrow) * ldo + ncol);
-                if (STREAM_OUT)
-                    __builtin_nontemporal_store(hv, dst);
-                else
-                    *dst = hv;
-            }
+            if (TAIL && tail.gate != nullptr && mrow < M) hv *= gv[it];
+            if (TAIL && tail.residual != nullptr && mrow < M) hv = rv[it] + hv;
+            __builtin_amdgcn_raw_buffer_store_b128(__builtin_bit_cast(u32x4, hv), out_rsrc,
+                                                   out_voff + (mi * 32 + it * (64 / PR)) * static_cast<int>(ldo) * 2, 0,
+                                                   STREAM_OUT ? 2 /* nt */ : 0);
         }
     }
 #endif
