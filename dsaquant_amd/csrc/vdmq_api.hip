@@ -31,6 +31,7 @@ int launch_act_to_native(const void *qact_v1, const void *ascales_v1, int64_t M,
 namespace {
 
 constexpr int64_t kMaxK = 65536;      /* keeps 256 * sum(q*q) inside int32 */
+constexpr int64_t kMaxLdo = 1 << 22;  /* a wave's 128 output rows stay inside the 32-bit offsets of its buffer stores */
 constexpr int64_t kMaxDim = 1 << 30;  /* int indexing inside the kernels */
 
 int check_k(int64_t K) {
@@ -201,7 +202,8 @@ static int gemm_checked(const void *qact, const void *ascale, const void *wq, co
         VDMQ_TRY(check_ptr(out, "out"));
         if (bias != nullptr) VDMQ_TRY(check_ptr(bias, "bias"));
         if (out_dtype != VDMQ_OUT_F16 && out_dtype != VDMQ_OUT_BF16) return fail(VDMQ_EINVAL, "unknown out_dtype %d", out_dtype);
-        if (ldo < N || ldo % 8 != 0) return fail(VDMQ_ESHAPE, "ldo must be >= N and a multiple of 8 (got %lld)", (long long)ldo);
+        if (ldo < N || ldo % 8 != 0 || ldo > kMaxLdo)
+            return fail(VDMQ_ESHAPE, "ldo must be >= N, a multiple of 8 and at most %lld (got %lld)", (long long)kMaxLdo, (long long)ldo);
         if (tail.gate != nullptr || tail.residual != nullptr) {
             if (out_dtype != VDMQ_OUT_F16) return fail(VDMQ_EINVAL, "gate and residual need an fp16 output");
             VDMQ_TRY(check_tail(tail, N));
@@ -305,7 +307,8 @@ static int gemm_bf6_checked(const void *xblocks, const void *ascale, const void 
         VDMQ_TRY(check_ptr(wscale, "wscale"));
         VDMQ_TRY(check_ptr(out, "out"));
         if (bias != nullptr) VDMQ_TRY(check_ptr(bias, "bias"));
-        if (ldo < N || ldo % 8 != 0) return fail(VDMQ_ESHAPE, "ldo must be >= N and a multiple of 8 (got %lld)", (long long)ldo);
+        if (ldo < N || ldo % 8 != 0 || ldo > kMaxLdo)
+            return fail(VDMQ_ESHAPE, "ldo must be >= N, a multiple of 8 and at most %lld (got %lld)", (long long)kMaxLdo, (long long)ldo);
         VDMQ_TRY(check_tail(tail, N));
     } else {
         VDMQ_TRY(check_ptr(acc, "acc"));

@@ -317,7 +317,8 @@ __global__ __launch_bounds__(Cfg::kThreads, Cfg::kOccupancy * Cfg::kWaves / 4) v
 
     uint8_t *side = lds + Cfg::kRingBytes + wave * Cfg::kSideBytes;
     const bool f16_out = !ACC_OUT && out_dtype == VDMQ_OUT_F16;
-    _Float16 side_as[(Cfg::kWaveM + 63) / 64] = {}, side_ws = 0, side_bias = 0;
+    // (no bias: -0, the one fp16 value whose addition changes no bit of any output)
+    _Float16 side_as[(Cfg::kWaveM + 63) / 64] = {}, side_ws = 0, side_bias = static_cast<_Float16>(-0.0f);
     if (f16_out) { /* older than the stage loads below: complete before the first of those is waited for */
 #pragma unroll
         for (int i = 0; i < (Cfg::kWaveM + 63) / 64; ++i)
@@ -441,8 +442,19 @@ __global__ __launch_bounds__(Cfg::kThreads, Cfg::kOccupancy * Cfg::kWaves / 4) v
                 for (int e = 0; e < 4; ++e) wsf[ni][rg][e] = static_cast<float>(w4[e]);
             }
         const int ncol = n0 + wn0 + (lane % PR) * 8;
-        f16x8 bv = {0, 0, 0, 0, 0, 0, 0, 0};
-        if (bias != nullptr) bv = *reinterpret_cast<const f16x8 *>(side + Cfg::kSideBias + (lane % PR) * 16);
+        const f16x8 bv = *reinterpret_cast<const f16x8 *>(side + Cfg::kSideBias + (lane % PR) * 16); /* -0 without a bias */
+        // The stores are buffer stores: the wave's corner of the output is the resource, whose size ends with the
+        // last row below M, so rows beyond are dropped by the range check instead of being predicated.  The check
+        // looks at the vector offset only (a scalar offset is added after it), so the row goes into the vector
+        // offset: one addition per store where a 64-bit address takes a multiplication and several additions.
+        const int wave_rows = min(max(M - (m0 + wm0), 0), Cfg::kWaveM);
+        if (n0 + wn0 >= N || wave_rows == 0) {
+            VDMQ_STAMP(3);
+            return; /* the same for the whole wave */
+        }
+        const __amdgpu_buffer_rsrc_t out_rsrc = __builtin_amdgcn_make_buffer_rsrc(
+            static_cast<__half *>(out) + static_cast<int64_t>(m0 + wm0) * ldo + n0 + wn0, 0, wave_rows * static_cast<int>(ldo) * 2, 0x00020000);
+        const int out_voff = ((lane / PR) * static_cast<int>(ldo) + (lane % PR) * 8) * 2;
 #pragma unroll
         for (int mi = 0; mi < Cfg::kMI; ++mi) {
             // The accumulator holds 256*acc.  float(256*acc) = 256*float(acc) exactly (|acc| < 2^24),
@@ -478,26 +490,20 @@ __global__ __launch_bounds__(Cfg::kThreads, Cfg::kOccupancy * Cfg::kWaves / 4) v
             for (int it = 0; it < PR / 2; ++it) {
                 const int row = it * (64 / PR) + lane / PR;
                 f16x8 hv = *reinterpret_cast<const f16x8 *>(stg + row * RS + (lane % PR) * 16);
-                if (bias != nullptr) hv += bv; /* one fp16 add per element */
+                hv += bv; /* one fp16 add per element */
                 const int mrow = m0 + wm0 + mi * 32 + row;
                 // out = residual + y * gate: the block's gated residual update, two more fp16
                 // operations per element, each rounded like the fp16 tensor operations they replace
-                if (TAIL && tail.gate != nullptr && mrow < M && ncol < N) hv *= gv[it];
-                if (TAIL && tail.residual != nullptr && mrow < M && ncol < N) hv = rv[it] + hv;
-#ifdef VDMQ_DBG_NOSTORE
-                if (mrow < 0 && ncol < N) {
-#else
-                if (mrow < M && ncol < N) {
+                if (TAIL && tail.gate != nullptr && mrow < M) hv *= gv[it];
+                if (TAIL && tail.residual != nullptr && mrow < M) hv = rv[it] + hv;
+#ifndef VDMQ_DBG_NOSTORE
+                // A large output is not re-read before it falls out of the caches anyway: streaming it (nt) keeps
+                // the operands (and the next quantizer's writes) in the Infinity Cache (measured: next quantizer
+                // 5.76 -> 6.01 TB/s).
+                __builtin_amdgcn_raw_buffer_store_b128(__builtin_bit_cast(u32x4, hv), out_rsrc,
+                                                       out_voff + (mi * 32 + it * (64 / PR)) * static_cast<int>(ldo) * 2, 0,
+                                                       STREAM_OUT ? 2 /* nt */ : 0);
 #endif
-                    f16x8 *dst = reinterpret_cast<f16x8 *>(static_cast<__half *>(out) + static_cast<int64_t>(mrow) * ldo + ncol);
-                    // A large output is not re-read before it falls out of the caches anyway:
-                    // streaming it keeps the operands (and the next quantizer's writes) in
-                    // the Infinity Cache (measured: next quantizer 5.76 -> 6.01 TB/s).
-                    if (STREAM_OUT)
-                        __builtin_nontemporal_store(hv, dst);
-                    else
-                        *dst = hv;
-                }
             }
         }
         VDMQ_STAMP(3);

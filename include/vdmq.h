@@ -120,7 +120,7 @@ int vdmq_ln_f16(const void *x, int64_t M, int64_t K, int64_t ldx, float eps, int
  *              then, with a bias, one more fp16 addition of bias[n]
  *   qact u8 [M, Kp/2] native; ascale fp16 [M]; wq u8 [N, Kp/2] native;
  *   wscale fp16 [N]; bias fp16 [N] or NULL; out [M, N] with row stride ldo
- *   elements (ldo % 8 == 0), out_dtype VDMQ_OUT_F16 or VDMQ_OUT_BF16.
+ *   elements (ldo % 8 == 0, ldo <= 4194304), out_dtype VDMQ_OUT_F16 or VDMQ_OUT_BF16.
  * Preconditions: K % 64 == 0, N % 128 == 0, K <= 65536. */
 int vdmq_gemm_w4a4(const void *qact, const void *ascale, const void *wq, const void *wscale, const void *bias, void *out,
                    int out_dtype, int64_t M, int64_t N, int64_t K, int64_t ldo, vdmq_stream_t stream);
