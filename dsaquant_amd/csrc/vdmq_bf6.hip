@@ -292,6 +292,16 @@ __global__ __launch_bounds__(Cfg::kWaves * 64, (Cfg::kWaves * Cfg::kOcc + 3) / 4
     const __amdgpu_buffer_rsrc_t out_rsrc = __builtin_amdgcn_make_buffer_rsrc(
         out + static_cast<int64_t>(m0 + wm0) * ldo + n0 + wn0, 0, wave_rows * static_cast<int>(ldo) * 2, 0x00020000);
     const int out_voff = ((lane / PR) * static_cast<int>(ldo) + (lane % PR) * 8) * 2;
+    // Row of the gate vectors for output row m = m / rows_per_gate, without a division per element: one vector per
+    // token is the row itself, and with at least as many rows per vector as the wave owns the wave's rows meet at
+    // most one boundary, found by comparing with the first row's remainder.
+    const int gate_rows = TAIL ? tail.rows_per_gate : 1;
+    const int gate_first = __builtin_amdgcn_readfirstlane((m0 + wm0) / gate_rows), gate_rem = m0 + wm0 - gate_first * gate_rows;
+    auto gate_row = [&](int mrow) -> int64_t {
+        if (gate_rows == 1) return mrow;
+        if (gate_rows >= MI * 32) return gate_first + (gate_rem + (mrow - m0 - wm0) >= gate_rows ? 1 : 0);
+        return mrow / gate_rows;
+    };
 #pragma unroll
     for (int mi = 0; mi < MI; ++mi) {
         const float as = static_cast<float>(*reinterpret_cast<const _Float16 *>(side + kSideAs + (mi * 32 + l32) * 2));
@@ -302,7 +312,7 @@ __global__ __launch_bounds__(Cfg::kWaves * 64, (Cfg::kWaves * Cfg::kOcc + 3) / 4
             const int mrow = m0 + wm0 + mi * 32 + it * (64 / PR) + lane / PR;
             const bool live = mrow < M && ncol < N;
             if (tail.gate != nullptr && live)
-                gv[it] = *reinterpret_cast<const f16x8 *>(tail.gate + static_cast<int64_t>(mrow / tail.rows_per_gate) * tail.ldg + ncol);
+                gv[it] = *reinterpret_cast<const f16x8 *>(tail.gate + gate_row(mrow) * tail.ldg + ncol);
             if (tail.residual != nullptr && live)
                 rv[it] = *reinterpret_cast<const f16x8 *>(tail.residual + static_cast<int64_t>(mrow) * tail.ldr + ncol);
         }

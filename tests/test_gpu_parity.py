@@ -461,6 +461,7 @@ def test_fused_layer_norm_argument_errors():
     (1, 8197, 2048, 8448, "token"),     # 256 x 256 tiles, one gate vector per token
     (3, 100, 320, 256, "none"),         # residual only (the attn2 update)
     (1, 257, 640, 384, "gate_only"),
+    (8, 40, 320, 256, "batch"),         # fewer rows per gate vector than a wave owns
 ])
 def test_gated_residual_epilogue_bit_exact(B, L, K, N, gate_kind):
     from dsaquant_amd import fused_ops
