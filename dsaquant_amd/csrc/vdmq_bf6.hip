@@ -78,6 +78,9 @@ struct Bf6Cfg {
     static_assert(kLdsBytes * kOcc <= 160 * 1024, "the CU's LDS holds OCC workgroups");
 };
 using Bf6Big = Bf6Cfg<256, 256, 2, 4, 3, 1>;
+#ifndef VDMQ_BF6_PERSISTENT
+#define VDMQ_BF6_PERSISTENT 1
+#endif
 constexpr int kValuPerMfma = 3; /* address arithmetic and operand assembly spread between the MFMAs */
 
 struct Bf6TileMap {
@@ -341,6 +344,257 @@ __global__ __launch_bounds__(Cfg::kWaves * 64, (Cfg::kWaves * Cfg::kOcc + 3) / 4
 #endif
 }
 
+// The same GEMM as a persistent kernel: one workgroup per CU position (XCD x, place j of a super-tile) walks that
+// place of every super-tile of its XCD.  While a tile's epilogue converts and stores, the first two K steps of the
+// next tile are already on their way into the two ring slots the epilogue's staging does not use; nothing is
+// dispatched, and no kernel argument re-read, between tiles.
+template <class Cfg, int OUT_MODE>
+__global__ __launch_bounds__(Cfg::kWaves * 64, (Cfg::kWaves * Cfg::kOcc + 3) / 4) void gemm_bf6_persistent_kernel(
+    const uint8_t *__restrict__ X, const uint8_t *__restrict__ W, const __half *__restrict__ ascale, const __half *__restrict__ wscale,
+    const __half *__restrict__ bias, __half *out, int M, int N, int kblocks, int64_t ldo, Bf6TileMap tmap, GemmTail tail) {
+#if defined(__HIP_DEVICE_COMPILE__)
+    constexpr bool STREAM_OUT = OUT_MODE == 1 || OUT_MODE == 4, TAIL = OUT_MODE >= 3;
+    constexpr int BM = Cfg::BM, BN = Cfg::BN, S = Cfg::S, MI = Cfg::MI, NI = Cfg::NI, kWaves = Cfg::kWaves, kWavesN = Cfg::kWavesN;
+    constexpr int kLoads = Cfg::kLoads, kStageBytes = Cfg::kStageBytes;
+    constexpr int PR = Cfg::kPiecesPerRow, RS = Cfg::kStageRowBytes;
+    static_assert(S == 3, "the prefetch under the epilogue uses ring slots 1 and 2");
+    extern __shared__ __attribute__((aligned(1024))) uint8_t lds[];
+    const int lane = threadIdx.x & 63, wave = __builtin_amdgcn_readfirstlane(threadIdx.x >> 6);
+    const int wn = wave % kWavesN, wm = wave / kWavesN;
+    const int l32 = lane & 31, lh = lane >> 5;
+    const int wm0 = wm * MI * 32, wn0 = wn * NI * 32;
+    const int last_rb_m = (M + 31) / 32 - 1, last_rb_n = N / 32 - 1;
+    const int ksteps = kblocks / (KS / 64);
+    const int xcd = blockIdx.x % kXcds, place = blockIdx.x / kXcds; /* gridDim.x = kXcds << per_log2 */
+    const int st_end = tmap.contig ? tmap.start[xcd + 1] : tmap.total_super;
+    // the seq-th super-tile of this XCD, and this workgroup's tile in it (false: none left; a super-tile at a ragged
+    // edge may have no tile at this place: tile_m = -1)
+    auto locate = [&](int seq, int &tile_m, int &tile_n) -> bool {
+        const int st = tmap.contig ? tmap.start[xcd] + seq : seq * kXcds + xcd;
+        if (st >= st_end) return false;
+        tile_m = ((st / tmap.super_n) << (tmap.per_log2 - tmap.group_n_log2)) + (place >> tmap.group_n_log2);
+        tile_n = ((st % tmap.super_n) << tmap.group_n_log2) + (place & ((1 << tmap.group_n_log2) - 1));
+        if (tile_m >= tmap.tiles_m || tile_n >= tmap.tiles_n) tile_m = -1;
+        return true;
+    };
+    auto next_tile = [&](int &seq, int &tile_m, int &tile_n) -> bool { /* advances seq to the next existing tile */
+        for (;;) {
+            ++seq;
+            if (!locate(seq, tile_m, tile_n)) return false;
+            if (tile_m >= 0) return true;
+        }
+    };
+    uint32_t lane_off[kLoads];
+#pragma unroll
+    for (int i = 0; i < kLoads; ++i) {
+        const int off = ((i * kWaves + wave) % 3) * 1024 + lane * 16;
+        const int kb = off >= kBlkBytes ? 1 : 0, in_blk = off - kb * kBlkBytes;
+        const bool part_b = in_blk >= kBlkPlaneB;
+        const int l = part_b ? (in_blk - kBlkPlaneB) / 8 : in_blk / 16;
+        lane_off[i] = static_cast<uint32_t>(bf6_piece(l & 31, kb, l >> 5, part_b, kblocks));
+    }
+    auto sources = [&](__amdgpu_buffer_rsrc_t (&src)[kLoads], int tile_m, int tile_n) __attribute__((always_inline)) {
+#pragma unroll
+        for (int i = 0; i < kLoads; ++i) {
+            const int q = (i * kWaves + wave) / 3;
+            const int64_t rb = q < BN / 32 ? min(tile_n * (BN / 32) + q, last_rb_n) : min(tile_m * (BM / 32) + q - BN / 32, last_rb_m);
+            src[i] = __builtin_amdgcn_make_buffer_rsrc(const_cast<uint8_t *>((q < BN / 32 ? W : X) + bf6_piece(rb * 32, 0, 0, false, kblocks)), 0,
+                                                       4 * kblocks * kBf6PanelKb, 0x00020000);
+        }
+    };
+    auto issue = [&](const __amdgpu_buffer_rsrc_t (&src)[kLoads], bool k_reverse, int kt, int slot) __attribute__((always_inline)) {
+        const int kpos = k_reverse ? ksteps - 1 - kt : kt;
+#pragma unroll
+        for (int i = 0; i < kLoads; ++i)
+            __builtin_amdgcn_raw_ptr_buffer_load_lds(src[i], VDMQ_LDS_PTR(lds + slot * kStageBytes + (i * kWaves + wave) * 1024), 16,
+                                                     lane_off[i], kpos * (KS / 64) * kBf6PanelKb, 0, 0);
+    };
+    struct Side {
+        _Float16 as[2], ws, bias;
+    };
+    auto side_fetch = [&](int tile_m, int tile_n) __attribute__((always_inline)) {
+        Side sd;
+        const int m0 = tile_m * BM, n0 = tile_n * BN;
+        const _Float16 *as_p = reinterpret_cast<const _Float16 *>(ascale);
+        sd.as[0] = as_p[min(m0 + wm0 + lane, M - 1)];
+        sd.as[1] = as_p[min(m0 + wm0 + 64 + lane, M - 1)];
+        sd.ws = reinterpret_cast<const _Float16 *>(wscale)[min(n0 + wn0 + lane, N - 1)];
+        sd.bias = static_cast<_Float16>(-0.0f);
+        if (bias != nullptr) sd.bias = reinterpret_cast<const _Float16 *>(bias)[min(n0 + wn0 + lane, N - 1)];
+        return sd;
+    };
+    uint8_t *side = lds + Cfg::kRingBytes + wave * kSideBytes;
+    auto side_publish = [&](const Side &sd) __attribute__((always_inline)) {
+        *reinterpret_cast<_Float16 *>(side + kSideAs + lane * 2) = sd.as[0];
+        *reinterpret_cast<_Float16 *>(side + kSideAs + 128 + lane * 2) = sd.as[1];
+        *reinterpret_cast<_Float16 *>(side + kSideWs + lane * 2) = sd.ws;
+        *reinterpret_cast<_Float16 *>(side + kSideBias + lane * 2) = sd.bias;
+    };
+    const uint32_t la = lane * 16, lb = kBlkPlaneB + lane * 8;
+    auto read = [&](v8i (&wf)[NI], v8i (&xf)[MI], const uint8_t *stage, int kb) __attribute__((always_inline)) {
+#pragma unroll
+        for (int ni = 0; ni < NI; ++ni) wf[ni] = ld_frag(stage + ((wn * NI + ni) * 2 + kb) * kBlkBytes, la, lb);
+#pragma unroll
+        for (int mi = 0; mi < MI; ++mi) xf[mi] = ld_frag(stage + ((BN / 32 + wm * MI + mi) * 2 + kb) * kBlkBytes, la, lb);
+    };
+    v16f acc[NI][MI];
+    auto mma = [&](const v8i (&wf)[NI], const v8i (&xf)[MI]) __attribute__((always_inline)) {
+#pragma unroll
+        for (int ni = 0; ni < NI; ++ni)
+#pragma unroll
+            for (int mi = 0; mi < MI; ++mi)
+                acc[ni][mi] = __builtin_amdgcn_mfma_scale_f32_32x32x64_f8f6f4(wf[ni], xf[mi], acc[ni][mi], 3, 3, 0, 0, 0, 0);
+    };
+
+    int seq = -1, tile_m = -1, tile_n = 0;
+    if (!next_tile(seq, tile_m, tile_n)) return;
+    __amdgpu_buffer_rsrc_t src[kLoads];
+    sources(src, tile_m, tile_n);
+    bool k_reverse = tmap.contig && (seq & 1) != 0;
+    {
+        const Side sd = side_fetch(tile_m, tile_n);
+#pragma unroll
+        for (int s = 0; s < S; ++s)
+            if (s < ksteps) issue(src, k_reverse, s, s);
+        if (ksteps >= S)
+            __builtin_amdgcn_s_waitcnt(waitcnt_imm(kLoads * (S - 1), 15));
+        else
+            __builtin_amdgcn_s_waitcnt(waitcnt_imm(0, 15));
+        lds_barrier();
+        side_publish(sd);
+    }
+    int cur = 0; /* ring slot of the tile's K step under work */
+    v8i wfa[NI], xfa[MI], wfb[NI], xfb[MI];
+    for (;;) {
+#pragma unroll
+        for (int ni = 0; ni < NI; ++ni)
+#pragma unroll
+            for (int mi = 0; mi < MI; ++mi)
+#pragma unroll
+                for (int r = 0; r < 16; ++r) acc[ni][mi][r] = 0.f;
+        read(wfa, xfa, lds + cur * kStageBytes, 0);
+        auto k_step = [&](int kt, auto steady_tag) __attribute__((always_inline)) {
+            constexpr bool STEADY = decltype(steady_tag)::value;
+            const uint8_t *stage = lds + cur * kStageBytes;
+            const int nxt = cur + 1 == S ? 0 : cur + 1;
+            read(wfb, xfb, stage, 1);
+            mma(wfa, xfa);
+            schedule_region<2 * (NI + MI), 0>();
+            if (STEADY)
+                __builtin_amdgcn_s_waitcnt(waitcnt_imm(kLoads * (S - 2), 0));
+            else
+                __builtin_amdgcn_s_waitcnt(waitcnt_imm(0, 0));
+            lds_barrier();
+            if (STEADY || kt + 1 < ksteps) read(wfa, xfa, lds + nxt * kStageBytes, 0);
+            if (STEADY) issue(src, k_reverse, kt + S, cur);
+            mma(wfb, xfb);
+            if (STEADY)
+                schedule_region<2 * (NI + MI), kLoads>();
+            else
+                schedule_region<2 * (NI + MI), 0>();
+            cur = nxt;
+        };
+        int kt = 0;
+        for (; kt + S < ksteps; ++kt) k_step(kt, std::true_type{});
+        for (; kt < ksteps; ++kt) k_step(kt, std::false_type{});
+
+        // ---- the next tile: its first two K steps go into slots 1 and 2 now (every wave is past the last barrier of
+        // the K loop, behind which nothing reads the ring any more); slot 0 holds the epilogue's staging
+        const int m0 = tile_m * BM, n0 = tile_n * BN;
+        int next_m = -1, next_n = 0;
+        const bool more = next_tile(seq, next_m, next_n);
+        Side next_side = {};
+        bool next_reverse = false;
+        if (more) {
+            sources(src, next_m, next_n);
+            next_reverse = tmap.contig && (seq & 1) != 0;
+            next_side = side_fetch(next_m, next_n);
+            issue(src, next_reverse, 0, 1);
+            if (ksteps > 1) issue(src, next_reverse, 1, 2);
+        }
+
+        // ---- fp16 epilogue of this tile (see gemm_bf6_kernel)
+        uint8_t *stg = lds + wave * Cfg::kStagingBytes;
+        const int wave_rows = min(max(M - (m0 + wm0), 0), MI * 32);
+        if (n0 + wn0 < N && wave_rows > 0) { /* the same for the whole wave */
+            float wsf[NI][4][4];
+#pragma unroll
+            for (int ni = 0; ni < NI; ++ni)
+#pragma unroll
+                for (int rg = 0; rg < 4; ++rg) {
+                    const f16x4 w4 = *reinterpret_cast<const f16x4 *>(side + kSideWs + (ni * 32 + rg * 8 + lh * 4) * 2);
+#pragma unroll
+                    for (int e = 0; e < 4; ++e) wsf[ni][rg][e] = static_cast<float>(w4[e]);
+                }
+            const int ncol = n0 + wn0 + (lane % PR) * 8;
+            const f16x8 bv = *reinterpret_cast<const f16x8 *>(side + kSideBias + (lane % PR) * 16);
+            const __amdgpu_buffer_rsrc_t out_rsrc = __builtin_amdgcn_make_buffer_rsrc(
+                out + static_cast<int64_t>(m0 + wm0) * ldo + n0 + wn0, 0, wave_rows * static_cast<int>(ldo) * 2, 0x00020000);
+            const int out_voff = ((lane / PR) * static_cast<int>(ldo) + (lane % PR) * 8) * 2;
+            const int gate_rows = TAIL ? tail.rows_per_gate : 1;
+            const int gate_first = __builtin_amdgcn_readfirstlane((m0 + wm0) / gate_rows), gate_rem = m0 + wm0 - gate_first * gate_rows;
+            auto gate_row = [&](int mrow) -> int64_t {
+                if (gate_rows == 1) return mrow;
+                if (gate_rows >= MI * 32) return gate_first + (gate_rem + (mrow - m0 - wm0) >= gate_rows ? 1 : 0);
+                return mrow / gate_rows;
+            };
+#pragma unroll
+            for (int mi = 0; mi < MI; ++mi) {
+                const float as = static_cast<float>(*reinterpret_cast<const _Float16 *>(side + kSideAs + (mi * 32 + l32) * 2));
+                f16x8 gv[PR / 2], rv[PR / 2];
+#pragma unroll
+                for (int it = 0; TAIL && it < PR / 2; ++it) {
+                    const int mrow = m0 + wm0 + mi * 32 + it * (64 / PR) + lane / PR;
+                    const bool live = mrow < M && ncol < N;
+                    if (tail.gate != nullptr && live)
+                        gv[it] = *reinterpret_cast<const f16x8 *>(tail.gate + gate_row(mrow) * tail.ldg + ncol);
+                    if (tail.residual != nullptr && live)
+                        rv[it] = *reinterpret_cast<const f16x8 *>(tail.residual + static_cast<int64_t>(mrow) * tail.ldr + ncol);
+                }
+#pragma unroll
+                for (int ni = 0; ni < NI; ++ni)
+#pragma unroll
+                    for (int rg = 0; rg < 4; ++rg) {
+                        f16x4 h;
+#pragma unroll
+                        for (int e = 0; e < 4; ++e) h[e] = static_cast<_Float16>(acc[ni][mi][rg * 4 + e] * (as * wsf[ni][rg][e]));
+                        *reinterpret_cast<f16x4 *>(stg + l32 * RS + (ni * 32 + rg * 8 + lh * 4) * 2) = h;
+                    }
+                // The prefetched steps have to be in LDS, for every wave, before the next tile reads them.  Loads and
+                // stores share one counter, so the wave waits for its loads here, before its first store -- by now
+                // they have had the first strip's conversion to arrive -- and the barrier after the epilogue
+                // publishes them.
+                if (mi == 0 && more) __builtin_amdgcn_s_waitcnt(waitcnt_imm(0, 15));
+#pragma unroll
+                for (int it = 0; it < PR / 2; ++it) {
+                    const int row = it * (64 / PR) + lane / PR;
+                    f16x8 hv = *reinterpret_cast<const f16x8 *>(stg + row * RS + (lane % PR) * 16);
+                    hv += bv;
+                    const int mrow = m0 + wm0 + mi * 32 + row;
+                    if (TAIL && tail.gate != nullptr && mrow < M) hv *= gv[it];
+                    if (TAIL && tail.residual != nullptr && mrow < M) hv = rv[it] + hv;
+                    __builtin_amdgcn_raw_buffer_store_b128(__builtin_bit_cast(u32x4, hv), out_rsrc,
+                                                           out_voff + (mi * 32 + it * (64 / PR)) * static_cast<int>(ldo) * 2, 0,
+                                                           STREAM_OUT ? 2 : 0);
+                }
+            }
+        }
+        else if (more) {
+            __builtin_amdgcn_s_waitcnt(waitcnt_imm(0, 15)); /* a wave without columns to store waits for its loads here */
+        }
+        if (!more) break;
+        __builtin_amdgcn_s_waitcnt(waitcnt_imm(63, 0)); /* the staging reads of this wave are done */
+        lds_barrier();
+        side_publish(next_side);
+        if (ksteps > 2) issue(src, next_reverse, 2, 0);
+        tile_m = next_m;
+        tile_n = next_n;
+        k_reverse = next_reverse;
+        cur = 1;
+    }
+#endif
+}
+
 // E3M2 code of an int4 value given as a two's complement nibble: sign << 5 | exponent/mantissa of |q|
 __device__ __forceinline__ uint32_t bf6_code(uint32_t nib) {
     const int q = static_cast<int>(nib << 28) >> 28;
@@ -476,6 +730,30 @@ int launch_bf6_cfg(const uint8_t *xblocks, const __half *ascale, const uint8_t *
                                            Cfg::kLdsBytes);
         if (e != hipSuccess) return fail(VDMQ_ELAUNCH, "hipFuncSetAttribute(%d bytes of LDS): %s", Cfg::kLdsBytes, hipGetErrorString(e));
         attr_done[dev][which] = true;
+    }
+    // The persistent kernel gives every CU position a fixed share -- its place in each super-tile of the XCD's
+    // sequence -- where the hardware dispatcher would refill a CU as soon as it is free: it pays when no XCD has many
+    // partly empty super-tiles (a ragged last row of super-tiles spread over an XCD's run costs whole rounds:
+    // measured -16 % on M = 27280, N = 14336, where that takes a third more rounds), i.e. when its rounds are within 15 % of
+    // the busiest XCD's tiles / places (M = 32760, N = 4608: 10 rounds for 9, still +4 %).
+    const int64_t all_tiles = static_cast<int64_t>(tm.tiles_m) * tm.tiles_n;
+    const int64_t busiest = tm.contig || best_load == 0 ? ceil_div(all_tiles, kXcds) : best_load;
+    const bool persistent = VDMQ_BF6_PERSISTENT && which < 2 && /* with the gated residual tail it needs more registers than there are: 10 % slower */
+                             static_cast<int64_t>(rounds) * 100 <= ceil_div(busiest, per) * 115;
+    if (persistent) {
+        using PKernel = void (*)(const uint8_t *, const uint8_t *, const __half *, const __half *, const __half *, __half *, int, int, int,
+                                 int64_t, Bf6TileMap, GemmTail);
+        const PKernel pk[2] = {gemm_bf6_persistent_kernel<Cfg, 0>, gemm_bf6_persistent_kernel<Cfg, 1>};
+        static bool pattr[kMaxDevices][2] = {};
+        if (!pattr[dev][which]) {
+            hipError_t e = hipFuncSetAttribute(reinterpret_cast<const void *>(pk[which]), hipFuncAttributeMaxDynamicSharedMemorySize,
+                                               Cfg::kLdsBytes);
+            if (e != hipSuccess) return fail(VDMQ_ELAUNCH, "hipFuncSetAttribute: %s", hipGetErrorString(e));
+            pattr[dev][which] = true;
+        }
+        hipLaunchKernelGGL(pk[which], dim3(kXcds * per), block, Cfg::kLdsBytes, s, xblocks, wblocks, ascale, wscale, bias, out,
+                           static_cast<int>(M), static_cast<int>(N), static_cast<int>(bf6_kblocks(K)), ldo, tm, tail);
+        return check_launch("gemm_bf6_persistent_kernel");
     }
     hipLaunchKernelGGL(kernels[which], grid, block, Cfg::kLdsBytes, s, xblocks, wblocks, ascale, wscale, bias, out, acc_out,
                        static_cast<int>(M), static_cast<int>(N), static_cast<int>(bf6_kblocks(K)), ldo, tm, tail);
