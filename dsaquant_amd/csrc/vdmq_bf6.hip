@@ -121,6 +121,86 @@ __device__ __forceinline__ void schedule_region() {
     }
 }
 
+#if defined(__HIP_DEVICE_COMPILE__) /* (the host pass does not know the buffer builtins) */
+// fp16 epilogue of one wave's 128 x 64 corner of a tile, as in the int8 kernel:
+// out = fp16(float(acc) * (float(as) * float(ws))) (+ bias in fp16) [then residual + y * gate]; one 32-row strip at
+// a time is transposed through the wave's staging area so that rows leave as whole 128-byte lines.  `side` holds the
+// wave's token scales, channel scales and bias; (m0, n0) is the corner's first output element.  `before_first_store`
+// runs once, after the first strip has been converted and staged.
+template <class Cfg, bool STREAM_OUT, bool TAIL, class Hook>
+__device__ __forceinline__ void bf6_epilogue(const v16f (&acc)[Cfg::NI][Cfg::MI], const uint8_t *side, uint8_t *stg, int lane, int m0, int n0,
+                                             __half *out, int64_t ldo, int M, int N, const GemmTail &tail, Hook &&before_first_store) {
+    constexpr int MI = Cfg::MI, NI = Cfg::NI, PR = Cfg::kPiecesPerRow, RS = Cfg::kStageRowBytes;
+    const int l32 = lane & 31, lh = lane >> 5;
+    float wsf[NI][4][4];
+#pragma unroll
+    for (int ni = 0; ni < NI; ++ni)
+#pragma unroll
+        for (int rg = 0; rg < 4; ++rg) {
+            const f16x4 w4 = *reinterpret_cast<const f16x4 *>(side + kSideWs + (ni * 32 + rg * 8 + lh * 4) * 2);
+#pragma unroll
+            for (int e = 0; e < 4; ++e) wsf[ni][rg][e] = static_cast<float>(w4[e]);
+        }
+    const int ncol = n0 + (lane % PR) * 8;
+    const f16x8 bv = *reinterpret_cast<const f16x8 *>(side + kSideBias + (lane % PR) * 16); /* -0 without a bias */
+    // The stores are buffer stores: the wave's corner of the output is the resource, whose size ends with the last
+    // row below M, so rows beyond are dropped by the range check instead of being predicated.  The check looks at the
+    // vector offset only (a scalar offset is added after it), so the row goes into the vector offset: one addition
+    // per store where a 64-bit address takes a multiplication and several additions.
+    const int wave_rows = min(M - m0, MI * 32);
+    const __amdgpu_buffer_rsrc_t out_rsrc =
+        __builtin_amdgcn_make_buffer_rsrc(out + static_cast<int64_t>(m0) * ldo + n0, 0, wave_rows * static_cast<int>(ldo) * 2, 0x00020000);
+    const int out_voff = ((lane / PR) * static_cast<int>(ldo) + (lane % PR) * 8) * 2;
+    // Row of the gate vectors for output row m = m / rows_per_gate, without a division per element: one vector per
+    // token is the row itself, and with at least as many rows per vector as the wave owns the wave's rows meet at
+    // most one boundary, found by comparing with the first row's remainder.
+    const int gate_rows = TAIL ? tail.rows_per_gate : 1;
+    const int gate_first = __builtin_amdgcn_readfirstlane(m0 / gate_rows), gate_rem = m0 - gate_first * gate_rows;
+    auto gate_row = [&](int mrow) -> int64_t {
+        if (gate_rows == 1) return mrow;
+        if (gate_rows >= MI * 32) return gate_first + (gate_rem + (mrow - m0) >= gate_rows ? 1 : 0);
+        return mrow / gate_rows;
+    };
+#pragma unroll
+    for (int mi = 0; mi < MI; ++mi) {
+        const float as = static_cast<float>(*reinterpret_cast<const _Float16 *>(side + kSideAs + (mi * 32 + l32) * 2));
+        // gate and residual pieces of this strip, requested before the strip is converted and staged
+        f16x8 gv[PR / 2], rv[PR / 2];
+#pragma unroll
+        for (int it = 0; TAIL && it < PR / 2; ++it) {
+            const int mrow = m0 + mi * 32 + it * (64 / PR) + lane / PR;
+            const bool live = mrow < M && ncol < N;
+            if (tail.gate != nullptr && live)
+                gv[it] = *reinterpret_cast<const f16x8 *>(tail.gate + gate_row(mrow) * tail.ldg + ncol);
+            if (tail.residual != nullptr && live)
+                rv[it] = *reinterpret_cast<const f16x8 *>(tail.residual + static_cast<int64_t>(mrow) * tail.ldr + ncol);
+        }
+#pragma unroll
+        for (int ni = 0; ni < NI; ++ni)
+#pragma unroll
+            for (int rg = 0; rg < 4; ++rg) {
+                f16x4 h;
+#pragma unroll
+                for (int e = 0; e < 4; ++e) h[e] = static_cast<_Float16>(acc[ni][mi][rg * 4 + e] * (as * wsf[ni][rg][e]));
+                *reinterpret_cast<f16x4 *>(stg + l32 * RS + (ni * 32 + rg * 8 + lh * 4) * 2) = h;
+            }
+        if (mi == 0) before_first_store();
+#pragma unroll
+        for (int it = 0; it < PR / 2; ++it) {
+            const int row = it * (64 / PR) + lane / PR;
+            f16x8 hv = *reinterpret_cast<const f16x8 *>(stg + row * RS + (lane % PR) * 16);
+            hv += bv;
+            const int mrow = m0 + mi * 32 + row;
+            if (TAIL && tail.gate != nullptr && mrow < M) hv *= gv[it];
+            if (TAIL && tail.residual != nullptr && mrow < M) hv = rv[it] + hv;
+            __builtin_amdgcn_raw_buffer_store_b128(__builtin_bit_cast(u32x4, hv), out_rsrc,
+                                                   out_voff + (mi * 32 + it * (64 / PR)) * static_cast<int>(ldo) * 2, 0,
+                                                   STREAM_OUT ? 2 /* nt */ : 0);
+        }
+    }
+}
+#endif
+
 // OUT_MODE: 0 = scaled fp16 output, 1 = the same with non-temporal stores, 2 = raw accumulators as int32,
 // 3 / 4 = 0 / 1 followed by the gated residual update out = residual + y * gate (see vdmq_gemm.hip)
 template <class Cfg, int OUT_MODE>
@@ -134,7 +214,7 @@ __global__ __launch_bounds__(Cfg::kWaves * 64, (Cfg::kWaves * Cfg::kOcc + 3) / 4
     constexpr bool ACC_OUT = OUT_MODE == 2, STREAM_OUT = OUT_MODE == 1 || OUT_MODE == 4, TAIL = OUT_MODE >= 3;
     constexpr int BM = Cfg::BM, BN = Cfg::BN, S = Cfg::S, MI = Cfg::MI, NI = Cfg::NI, kWaves = Cfg::kWaves, kWavesN = Cfg::kWavesN;
     constexpr int kLoads = Cfg::kLoads, kStageBytes = Cfg::kStageBytes;
-    constexpr int kPiecesPerRow = Cfg::kPiecesPerRow, kStageRowBytes = Cfg::kStageRowBytes, kStagingBytes = Cfg::kStagingBytes;
+    constexpr int kStagingBytes = Cfg::kStagingBytes;
     extern __shared__ __attribute__((aligned(1024))) uint8_t lds[];
     int tile_m, tile_n;
     if (!map_tile(tmap, blockIdx.x, tile_m, tile_n)) return;
@@ -271,76 +351,8 @@ __global__ __launch_bounds__(Cfg::kWaves * 64, (Cfg::kWaves * Cfg::kOcc + 3) / 4
         }
         return;
     }
-    // fp16 epilogue, as in the int8 kernel: out = fp16(float(acc) * (float(as) * float(ws))) (+ bias in fp16);
-    // one 32-row strip at a time is transposed through LDS so that rows leave as whole 128-byte lines
-    constexpr int PR = kPiecesPerRow, RS = kStageRowBytes;
-    uint8_t *stg = lds + wave * kStagingBytes;
-    float wsf[NI][4][4];
-#pragma unroll
-    for (int ni = 0; ni < NI; ++ni)
-#pragma unroll
-        for (int rg = 0; rg < 4; ++rg) {
-            const f16x4 w4 = *reinterpret_cast<const f16x4 *>(side + kSideWs + (ni * 32 + rg * 8 + lh * 4) * 2);
-#pragma unroll
-            for (int e = 0; e < 4; ++e) wsf[ni][rg][e] = static_cast<float>(w4[e]);
-        }
-    const int ncol = n0 + wn0 + (lane % PR) * 8;
-    const f16x8 bv = *reinterpret_cast<const f16x8 *>(side + kSideBias + (lane % PR) * 16);
-    // The stores are buffer stores: the wave's corner of the output is the resource, whose size ends with the last
-    // row below M, so rows beyond are dropped by the range check instead of being predicated.  The check looks at the
-    // vector offset only (a scalar offset is added after it), so the row goes into the vector offset: one addition
-    // per store where a 64-bit address takes a multiplication and several additions.
-    const int wave_rows = min(max(M - (m0 + wm0), 0), MI * 32);
-    if (n0 + wn0 >= N || wave_rows == 0) return; /* the same for the whole wave */
-    const __amdgpu_buffer_rsrc_t out_rsrc = __builtin_amdgcn_make_buffer_rsrc(
-        out + static_cast<int64_t>(m0 + wm0) * ldo + n0 + wn0, 0, wave_rows * static_cast<int>(ldo) * 2, 0x00020000);
-    const int out_voff = ((lane / PR) * static_cast<int>(ldo) + (lane % PR) * 8) * 2;
-    // Row of the gate vectors for output row m = m / rows_per_gate, without a division per element: one vector per
-    // token is the row itself, and with at least as many rows per vector as the wave owns the wave's rows meet at
-    // most one boundary, found by comparing with the first row's remainder.
-    const int gate_rows = TAIL ? tail.rows_per_gate : 1;
-    const int gate_first = __builtin_amdgcn_readfirstlane((m0 + wm0) / gate_rows), gate_rem = m0 + wm0 - gate_first * gate_rows;
-    auto gate_row = [&](int mrow) -> int64_t {
-        if (gate_rows == 1) return mrow;
-        if (gate_rows >= MI * 32) return gate_first + (gate_rem + (mrow - m0 - wm0) >= gate_rows ? 1 : 0);
-        return mrow / gate_rows;
-    };
-#pragma unroll
-    for (int mi = 0; mi < MI; ++mi) {
-        const float as = static_cast<float>(*reinterpret_cast<const _Float16 *>(side + kSideAs + (mi * 32 + l32) * 2));
-        // gate and residual pieces of this strip, requested before the strip is converted and staged
-        f16x8 gv[PR / 2], rv[PR / 2];
-#pragma unroll
-        for (int it = 0; TAIL && it < PR / 2; ++it) {
-            const int mrow = m0 + wm0 + mi * 32 + it * (64 / PR) + lane / PR;
-            const bool live = mrow < M && ncol < N;
-            if (tail.gate != nullptr && live)
-                gv[it] = *reinterpret_cast<const f16x8 *>(tail.gate + gate_row(mrow) * tail.ldg + ncol);
-            if (tail.residual != nullptr && live)
-                rv[it] = *reinterpret_cast<const f16x8 *>(tail.residual + static_cast<int64_t>(mrow) * tail.ldr + ncol);
-        }
-#pragma unroll
-        for (int ni = 0; ni < NI; ++ni)
-#pragma unroll
-            for (int rg = 0; rg < 4; ++rg) {
-                f16x4 h;
-#pragma unroll
-                for (int e = 0; e < 4; ++e) h[e] = static_cast<_Float16>(acc[ni][mi][rg * 4 + e] * (as * wsf[ni][rg][e]));
-                *reinterpret_cast<f16x4 *>(stg + l32 * RS + (ni * 32 + rg * 8 + lh * 4) * 2) = h;
-            }
-#pragma unroll
-        for (int it = 0; it < PR / 2; ++it) {
-            const int row = it * (64 / PR) + lane / PR;
-            f16x8 hv = *reinterpret_cast<const f16x8 *>(stg + row * RS + (lane % PR) * 16);
-            hv += bv;
-            const int mrow = m0 + wm0 + mi * 32 + row;
-            if (TAIL && tail.gate != nullptr && mrow < M) hv *= gv[it];
-            if (TAIL && tail.residual != nullptr && mrow < M) hv = rv[it] + hv;
-            __builtin_amdgcn_raw_buffer_store_b128(__builtin_bit_cast(u32x4, hv), out_rsrc,
-                                                   out_voff + (mi * 32 + it * (64 / PR)) * static_cast<int>(ldo) * 2, 0,
-                                                   STREAM_OUT ? 2 /* nt */ : 0);
-        }
-    }
+    if (n0 + wn0 >= N || m0 + wm0 >= M) return; /* nothing to store: the same for the whole wave */
+    bf6_epilogue<Cfg, STREAM_OUT, TAIL>(acc, side, lds + wave * kStagingBytes, lane, m0 + wm0, n0 + wn0, out, ldo, M, N, tail, [] {});
 #endif
 }
 
@@ -356,12 +368,10 @@ __global__ __launch_bounds__(Cfg::kWaves * 64, (Cfg::kWaves * Cfg::kOcc + 3) / 4
     constexpr bool STREAM_OUT = OUT_MODE == 1 || OUT_MODE == 4, TAIL = OUT_MODE >= 3;
     constexpr int BM = Cfg::BM, BN = Cfg::BN, S = Cfg::S, MI = Cfg::MI, NI = Cfg::NI, kWaves = Cfg::kWaves, kWavesN = Cfg::kWavesN;
     constexpr int kLoads = Cfg::kLoads, kStageBytes = Cfg::kStageBytes;
-    constexpr int PR = Cfg::kPiecesPerRow, RS = Cfg::kStageRowBytes;
     static_assert(S == 3, "the prefetch under the epilogue uses ring slots 1 and 2");
     extern __shared__ __attribute__((aligned(1024))) uint8_t lds[];
     const int lane = threadIdx.x & 63, wave = __builtin_amdgcn_readfirstlane(threadIdx.x >> 6);
     const int wn = wave % kWavesN, wm = wave / kWavesN;
-    const int l32 = lane & 31, lh = lane >> 5;
     const int wm0 = wm * MI * 32, wn0 = wn * NI * 32;
     const int last_rb_m = (M + 31) / 32 - 1, last_rb_n = N / 32 - 1;
     const int ksteps = kblocks / (KS / 64);
@@ -513,75 +523,17 @@ __global__ __launch_bounds__(Cfg::kWaves * 64, (Cfg::kWaves * Cfg::kOcc + 3) / 4
             if (ksteps > 1) issue(src, next_reverse, 1, 2);
         }
 
-        // ---- fp16 epilogue of this tile (see gemm_bf6_kernel)
-        uint8_t *stg = lds + wave * Cfg::kStagingBytes;
-        const int wave_rows = min(max(M - (m0 + wm0), 0), MI * 32);
-        if (n0 + wn0 < N && wave_rows > 0) { /* the same for the whole wave */
-            float wsf[NI][4][4];
-#pragma unroll
-            for (int ni = 0; ni < NI; ++ni)
-#pragma unroll
-                for (int rg = 0; rg < 4; ++rg) {
-                    const f16x4 w4 = *reinterpret_cast<const f16x4 *>(side + kSideWs + (ni * 32 + rg * 8 + lh * 4) * 2);
-#pragma unroll
-                    for (int e = 0; e < 4; ++e) wsf[ni][rg][e] = static_cast<float>(w4[e]);
-                }
-            const int ncol = n0 + wn0 + (lane % PR) * 8;
-            const f16x8 bv = *reinterpret_cast<const f16x8 *>(side + kSideBias + (lane % PR) * 16);
-            const __amdgpu_buffer_rsrc_t out_rsrc = __builtin_amdgcn_make_buffer_rsrc(
-                out + static_cast<int64_t>(m0 + wm0) * ldo + n0 + wn0, 0, wave_rows * static_cast<int>(ldo) * 2, 0x00020000);
-            const int out_voff = ((lane / PR) * static_cast<int>(ldo) + (lane % PR) * 8) * 2;
-            const int gate_rows = TAIL ? tail.rows_per_gate : 1;
-            const int gate_first = __builtin_amdgcn_readfirstlane((m0 + wm0) / gate_rows), gate_rem = m0 + wm0 - gate_first * gate_rows;
-            auto gate_row = [&](int mrow) -> int64_t {
-                if (gate_rows == 1) return mrow;
-                if (gate_rows >= MI * 32) return gate_first + (gate_rem + (mrow - m0 - wm0) >= gate_rows ? 1 : 0);
-                return mrow / gate_rows;
-            };
-#pragma unroll
-            for (int mi = 0; mi < MI; ++mi) {
-                const float as = static_cast<float>(*reinterpret_cast<const _Float16 *>(side + kSideAs + (mi * 32 + l32) * 2));
-                f16x8 gv[PR / 2], rv[PR / 2];
-#pragma unroll
-                for (int it = 0; TAIL && it < PR / 2; ++it) {
-                    const int mrow = m0 + wm0 + mi * 32 + it * (64 / PR) + lane / PR;
-                    const bool live = mrow < M && ncol < N;
-                    if (tail.gate != nullptr && live)
-                        gv[it] = *reinterpret_cast<const f16x8 *>(tail.gate + gate_row(mrow) * tail.ldg + ncol);
-                    if (tail.residual != nullptr && live)
-                        rv[it] = *reinterpret_cast<const f16x8 *>(tail.residual + static_cast<int64_t>(mrow) * tail.ldr + ncol);
-                }
-#pragma unroll
-                for (int ni = 0; ni < NI; ++ni)
-#pragma unroll
-                    for (int rg = 0; rg < 4; ++rg) {
-                        f16x4 h;
-#pragma unroll
-                        for (int e = 0; e < 4; ++e) h[e] = static_cast<_Float16>(acc[ni][mi][rg * 4 + e] * (as * wsf[ni][rg][e]));
-                        *reinterpret_cast<f16x4 *>(stg + l32 * RS + (ni * 32 + rg * 8 + lh * 4) * 2) = h;
-                    }
-                // The prefetched steps have to be in LDS, for every wave, before the next tile reads them.  Loads and
-                // stores share one counter, so the wave waits for its loads here, before its first store -- by now
-                // they have had the first strip's conversion to arrive -- and the barrier after the epilogue
-                // publishes them.
-                if (mi == 0 && more) __builtin_amdgcn_s_waitcnt(waitcnt_imm(0, 15));
-#pragma unroll
-                for (int it = 0; it < PR / 2; ++it) {
-                    const int row = it * (64 / PR) + lane / PR;
-                    f16x8 hv = *reinterpret_cast<const f16x8 *>(stg + row * RS + (lane % PR) * 16);
-                    hv += bv;
-                    const int mrow = m0 + wm0 + mi * 32 + row;
-                    if (TAIL && tail.gate != nullptr && mrow < M) hv *= gv[it];
-                    if (TAIL && tail.residual != nullptr && mrow < M) hv = rv[it] + hv;
-                    __builtin_amdgcn_raw_buffer_store_b128(__builtin_bit_cast(u32x4, hv), out_rsrc,
-                                                           out_voff + (mi * 32 + it * (64 / PR)) * static_cast<int>(ldo) * 2, 0,
-                                                           STREAM_OUT ? 2 : 0);
-                }
-            }
-        }
-        else if (more) {
-            __builtin_amdgcn_s_waitcnt(waitcnt_imm(0, 15)); /* a wave without columns to store waits for its loads here */
-        }
+        // ---- fp16 epilogue of this tile.  The prefetched steps have to be in LDS, for every wave, before the next tile
+        // reads them.  Loads and stores share one counter, so the wave waits for its loads before its first store --
+        // by then they have had the first strip's conversion to arrive -- and the barrier below publishes them.
+        auto prefetch_landed = [&] {
+            if (more) __builtin_amdgcn_s_waitcnt(waitcnt_imm(0, 15));
+        };
+        if (n0 + wn0 < N && m0 + wm0 < M) /* the same for the whole wave */
+            bf6_epilogue<Cfg, STREAM_OUT, TAIL>(acc, side, lds + wave * Cfg::kStagingBytes, lane, m0 + wm0, n0 + wn0, out, ldo, M, N, tail,
+                                                prefetch_landed);
+        else
+            prefetch_landed();
         if (!more) break;
         __builtin_amdgcn_s_waitcnt(waitcnt_imm(63, 0)); /* the staging reads of this wave are done */
         lds_barrier();
