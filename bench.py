@@ -41,15 +41,15 @@ FP6_PEAK_TOPS = 10100.0  # MI355X dense FP6 MFMA, published
 # HBM bytes per launch of the dominant kernels on the default workload, from rocprofv3 --pmc FETCH_SIZE and
 # WRITE_SIZE runs of this program (mean over the four launches of a step; the summary with the scaling by
 # the copy kernel's readings is profiles/gemm_w4a4_kernel+quantize_rows_kernel.wan14b_720p_block.md for the int8
-# path and profiles/gemm_bf6_kernel+quantize_rows_kernel.wan14b_720p_block.md for the bf6 path)
+# path and profiles/gemm_bf6_persistent_kernel+quantize_rows_kernel.wan14b_720p_block.md for the bf6 path)
 # gemm: (FETCH_SIZE 1377438 KiB x 2.0 + WRITE_SIZE 1455495 KiB x 1.0) x 1024; the reads are requests leaving L2
 # (Infinity Cache or HBM), 9x the operand bytes because every XCD fetches most of its super-tile's slabs once.
 # quant: (FETCH_SIZE 538736 KiB x 2.0 + WRITE_SIZE 269920 KiB x 1.0) x 1024 = 1.0005 x the algorithmic bytes.
-# bf6 path, same method: gemm (FETCH_SIZE 2334456 KiB x 2.0 + WRITE_SIZE 1456095 KiB x 1.0) x 1024 (6-bit operands and
-# little slab re-use between super-tiles: 10x the operand bytes); quant (538745 x 2.0 + 404284 x 1.0) x 1024 = 1.0002 x
+# bf6 path, same method: gemm (FETCH_SIZE 2692746 KiB x 2.0 + WRITE_SIZE 1456313 KiB x 1.0) x 1024 (6-bit operands and
+# little slab re-use between super-tiles: 12x the operand bytes); quant (538745 x 2.0 + 404284 x 1.0) x 1024 = 1.0002 x
 # the algorithmic bytes.
 MEASURED_TRAFFIC = {("wan14b_720p_block", "int8"): {"gemm": 4311418572, "quant": 1379729408},
-                    ("wan14b_720p_block", "bf6"): {"gemm": 6272007654, "quant": 1517336576}}
+                    ("wan14b_720p_block", "bf6"): {"gemm": 7006008524, "quant": 1517336576}}
 HBM_PEAK_GBS = 8000.0    # MI355X HBM3E, published
 
 # (name, K, N) at M tokens
@@ -225,7 +225,7 @@ def main():
     path = paths[0] if len(paths) == 1 else "mixed"
     # a step that mixes both kinds of launches is priced against the higher peak
     peak = INT8_PEAK_TOPS if path == "int8" else FP6_PEAK_TOPS
-    gemm_kernel = {"int8": "gemm_w4a4_kernel", "bf6": "gemm_bf6_kernel"}.get(path, "gemm_w4a4_kernel + gemm_bf6_kernel")
+    gemm_kernel = {"int8": "gemm_w4a4_kernel", "bf6": "gemm_bf6_persistent_kernel"}.get(path, "gemm_w4a4_kernel + gemm_bf6_persistent_kernel")
     traffic = MEASURED_TRAFFIC.get((args.workload, path), {})
     value = total_ops / (ms_per_step * 1e-3) / 1e12
 
