@@ -620,6 +620,45 @@ def test_both_matrix_paths_agree_on_random_shapes():
             assert np.array_equal(a6.cpu().numpy(), O.np_gemm_i32(qx, qw))
 
 
+def test_matrix_paths_give_the_same_fp16_outputs():
+    """Twenty seeded problems through the whole linear (quantizer, GEMM, epilogue) on either matrix path: the fp16
+    outputs are the same bits, with and without bias, plain and with the gated residual tail.  The shapes cover what
+    the bf6 launcher chooses between: several rounds of tiles per CU (the kernel that walks tiles), few tiles, long
+    K, wide N, ragged M throughout."""
+    from dsaquant_amd import fused_ops
+
+    v = vk()
+    rng = np.random.default_rng(77)
+    old = v.matrix_path()
+    try:
+        for i in range(20):
+            kind = i % 4
+            if kind == 0:
+                M, N, K = int(rng.integers(3000, 12000)), 128 * int(rng.integers(8, 36)), 64 * int(rng.integers(1, 16))
+            elif kind == 1:
+                M, N, K = int(rng.integers(1, 3000)), 128 * int(rng.integers(1, 16)), 64 * int(rng.integers(40, 225))
+            elif kind == 2:
+                M, N, K = int(rng.integers(1, 700)), 128 * int(rng.integers(1, 12)), 64 * int(rng.integers(1, 40))
+            else:
+                M, N, K = int(rng.integers(200, 3000)), 128 * int(rng.integers(60, 120)), 64 * int(rng.integers(8, 40))
+            x, qw, ws, bias = O.synth_linear(M, K, N, seed=i)
+            tail = i % 3
+            print(f"same fp16 outputs M={M} N={N} K={K} tail={tail}", flush=True)
+            args = (t16(x), t16(O.np_pack_wgt_v1(qw)), t16(O.np_pack_wscales_v1(ws, K)), t16(bias) if i % 2 else None)
+            res = t16(rng.standard_normal((M, N)).astype(np.float16)) if tail else None
+            gate = t16(rng.standard_normal((1, N)).astype(np.float16)) if tail == 2 else None
+            got = {}
+            for path in ("int8", "bf6"):
+                v.set_matrix_path(path)
+                got[path] = (fused_ops.linear_fused(*args, clip_ratio=0.95, residual=res, gate=gate) if tail
+                             else v.linear_vdm_w4a4(*args, clip_ratio=0.95))
+            torch.cuda.synchronize()
+            assert torch.equal(got["int8"].view(torch.int16), got["bf6"].view(torch.int16)), (M, N, K, tail)
+            v.clear_native_cache()
+    finally:
+        v.set_matrix_path(old)
+
+
 def test_bf6_extreme_values_stay_exact():
     """|acc| up to 64 * K = 2^20 * 0.875 with K = 14336: exact in the fp32 accumulator."""
     v = vk()
