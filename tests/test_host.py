@@ -5,6 +5,7 @@ No compute call is made on the library here (there is no GPU)."""
 import re
 from pathlib import Path
 
+import numpy as np
 import pytest
 import torch
 import torch.nn as nn
@@ -253,3 +254,99 @@ def test_fused_qkv_dispatch_falls_through_to_separate_projections_on_cpu():
     attn.to_qkv = nn.Linear(128, 384)
     q, k, v = get_qkv_projections(attn, x, None)
     assert torch.equal(torch.cat([q, k, v], -1), attn.to_qkv(x))
+
+
+# ---- the reference's torch floating-point path, from vectors recorded with its own quant_linear.py ----
+
+_QL_FIXTURE = Path(__file__).parent / "golden" / "quantlinear_fp_path.npz"
+_QL_QUANTIZERS = {
+    "sym_per_channel": dict(bit=4, sym=True),
+    "sym_clip": dict(bit=4, sym=True, clip_ratio=0.9),
+    "sym_per_token_3d": dict(bit=4, sym=True, granularity="per_token"),
+    "sym_per_channel_3d": dict(bit=4, sym=True),
+    "sym_per_tensor": dict(bit=8, sym=True, granularity="per_tensor"),
+    "sym_per_group": dict(bit=4, sym=True, granularity="per_group", group_size=8),
+    "asym_round_zero": dict(bit=4, sym=False),
+    "asym_no_round_zero": dict(bit=4, sym=False, round_zero=False),
+    "sym_fp16": dict(bit=4, sym=True),
+}
+
+
+def _bits(a: np.ndarray) -> np.ndarray:
+    return a.view({2: np.uint16, 4: np.uint32}[a.dtype.itemsize])
+
+
+@pytest.mark.parametrize("name", sorted(_QL_QUANTIZERS))
+def test_uniform_quantizer_reproduces_the_reference_vectors(name):
+    """UniformQuantizer on the recorded inputs: scale, zero point and both fake-quantized tensors (the second one
+    with the parameters frozen by the first) are the reference's bits -- elementwise IEEE operations only
+    (tests/golden/make_quantlinear_fixture.py wrote the vectors from quant_linear.py:6-86)."""
+    from dsaquant_amd.quantization.quant_linear import UniformQuantizer
+
+    g = np.load(_QL_FIXTURE)
+    q = UniformQuantizer(**_QL_QUANTIZERS[name])
+    y = q(torch.from_numpy(g[f"q.{name}.x"]))
+    y2 = q(torch.from_numpy(g[f"q.{name}.x2"]))
+    assert np.array_equal(_bits(q.scale.numpy()), _bits(g[f"q.{name}.scale"]))
+    if f"q.{name}.zero_point" in g.files:
+        assert np.array_equal(_bits(q.zero_point.numpy()), _bits(g[f"q.{name}.zero_point"]))
+    else:
+        assert q.zero_point is None
+    assert np.array_equal(_bits(y.numpy()), _bits(g[f"q.{name}.y"]))
+    assert np.array_equal(_bits(y2.numpy()), _bits(g[f"q.{name}.y2"]))
+
+
+@pytest.mark.parametrize("name,bias", [("bias_2d", True), ("nobias_2d", False), ("bias_3d", True)])
+def test_quantlinear_fp_path_reproduces_the_reference_vectors(name, bias):
+    """QuantLinear.forward without the kernel on the recorded layer and inputs (quant_linear.py:162-178): plain,
+    weight-only, weight + activation, and a second input under the activation scale the first one froze.  The
+    quantizer scales are exact; the outputs go through F.linear, whose fp32 summation order belongs to the torch
+    build, hence 1e-5 of the largest output."""
+    from dsaquant_amd.quantization.quant_linear import QuantLinear
+
+    g = np.load(_QL_FIXTURE)
+    layer = nn.Linear(40, 24, bias=bias)
+    with torch.no_grad():
+        layer.weight.copy_(torch.from_numpy(g[f"l.{name}.weight"]))
+        if bias:
+            layer.bias.copy_(torch.from_numpy(g[f"l.{name}.bias"]))
+    m = QuantLinear(layer, {"w": "lsq", "act": "dynamic"}, {"w": {"bit": 4, "sym": True}, "act": {"bit": 4, "sym": True}})
+    x, x2 = torch.from_numpy(g[f"l.{name}.x"]), torch.from_numpy(g[f"l.{name}.x2"])
+    with torch.no_grad():
+        got = {"plain": m(x)}
+        m.set_quant_state(True, False)
+        got["w_only"] = m(x)
+        m.set_quant_state(True, True)
+        got["both"] = m(x)
+        got["both2"] = m(x2)
+    assert np.array_equal(_bits(m.wquantizer.scale.numpy()), _bits(g[f"l.{name}.wscale"]))
+    assert np.array_equal(_bits(m.aquantizer.scale.numpy()), _bits(g[f"l.{name}.ascale"]))
+    for key, y in got.items():
+        want = g[f"l.{name}.{key}"]
+        assert y.shape == want.shape
+        assert np.abs(y.numpy() - want).max() <= 1e-5 * np.abs(want).max(), key
+    assert m.extra_repr() == str(g[f"l.{name}.repr"])
+
+
+def test_cpu_baseline_restatement_matches_the_reference_vectors():
+    """oracle/quantlinear_torch.py (the timed CPU baseline) on the recorded 2-D cases: its scales are the reference's
+    bits; with `dynamic=False` (scale frozen by the first call, as the reference does) both outputs agree to the
+    F.linear tolerance, and `dynamic=True` differs from the reference only by recomputing the scale per call."""
+    from oracle.quantlinear_torch import QuantLinearTorchPath, sym_scale
+
+    g = np.load(_QL_FIXTURE)
+    for name, bias in (("bias_2d", True), ("nobias_2d", False)):
+        w = torch.from_numpy(g[f"l.{name}.weight"])
+        b = torch.from_numpy(g[f"l.{name}.bias"]) if bias else None
+        x, x2 = torch.from_numpy(g[f"l.{name}.x"]), torch.from_numpy(g[f"l.{name}.x2"])
+        p = QuantLinearTorchPath(w, b, dynamic=False)
+        y, y2 = p(x), p(x2)
+        assert np.array_equal(_bits(p.wscale.numpy()), _bits(g[f"l.{name}.wscale"]))
+        assert np.array_equal(_bits(p.ascale.numpy()), _bits(g[f"l.{name}.ascale"]))
+        for got, key in ((y, "both"), (y2, "both2")):
+            want = g[f"l.{name}.{key}"]
+            assert np.abs(got.numpy() - want).max() <= 1e-5 * np.abs(want).max(), (name, key)
+        d = QuantLinearTorchPath(w, b, dynamic=True)
+        assert np.abs(d(x).numpy() - g[f"l.{name}.both"]).max() <= 1e-5 * np.abs(g[f"l.{name}.both"]).max()
+        d(x2)
+        assert np.array_equal(_bits(d.ascale.numpy()), _bits(sym_scale(x2).numpy()))
