@@ -922,3 +922,42 @@ def test_hip_path_reproduces_the_committed_emulation_fixture():
     native_w, _ = v._native_weights(t16(f["qweight"]), t16(f["wscales_packed"]))
     acc = v.gemm_int32_accumulators(native_x, native_w, 128)
     assert np.array_equal(acc.cpu().numpy(), f["acc"])
+
+
+@pytest.mark.gpu
+@pytest.mark.parametrize("tag", ["v1", "legacy"])
+def test_reference_written_checkpoint_runs_through_the_kernels(tag):
+    """The checkpoint the reference's own save_packed_checkpoint wrote (tests/golden/make_checkpoint_fixture.py), loaded
+    with the kernel required: both QuantLinear layers give the oracle's fp16 bits for the integers and scales the
+    file holds, at the module's clip ratio of 0.95 (quant_linear.py:121, :163-172)."""
+    import importlib.util
+    from pathlib import Path
+
+    from dsaquant_amd.checkpoints import packed_checkpoint as pc
+    from dsaquant_amd.quantization.quant_linear import QuantLinear
+
+    vk()
+    golden = Path(__file__).parent / "golden"
+    spec = importlib.util.spec_from_file_location("_make_checkpoint_fixture", golden / "make_checkpoint_fixture.py")
+    gen = importlib.util.module_from_spec(spec)
+    spec.loader.exec_module(gen)
+    ckpt = pc.load_quant_checkpoint(str(golden / f"reference_written_packed_{tag}.pt"), dcp_loader=None)
+    model = gen.build_toy(QuantLinear, seed=3)
+    missing, unexpected = pc.load_packed_quantized_model(model, ckpt, quant_linear_cls=QuantLinear, dtype=torch.float16,
+                                                        device=torch.device("cuda:0"))
+    assert missing == [] and unexpected == []
+    rng = np.random.default_rng(5)
+    for layer in (model.q1, model.q2):
+        N, K = layer.out_features, layer.in_features
+        x = rng.standard_normal((33, K)).astype(np.float16)
+        x[:, 5] *= np.float16(20.0)
+        x[7] = 0
+        print(f"reference-written checkpoint {tag}: layer {K}->{N}", flush=True)
+        y = layer(t16(x))
+        torch.cuda.synchronize()
+        qw = O.np_unpack_wgt_v1(layer.vdm_weight_packed.cpu().numpy(), N, K)
+        ws = layer.vdm_weight_scale.cpu().numpy()
+        assert np.array_equal(O.np_unpack_wscales_v1(layer.vdm_weight_scale_packed.cpu().numpy(), N, K), ws)
+        bias = None if layer.bias is None else layer.bias.detach().cpu().numpy()
+        want = O.np_linear(x, qw, ws, bias, 0.95)[0]
+        assert y.dtype == torch.float16 and np.array_equal(y.cpu().numpy().view(np.uint16), want.view(np.uint16))

@@ -350,3 +350,92 @@ def test_cpu_baseline_restatement_matches_the_reference_vectors():
         assert np.abs(d(x).numpy() - g[f"l.{name}.both"]).max() <= 1e-5 * np.abs(g[f"l.{name}.both"]).max()
         d(x2)
         assert np.array_equal(_bits(d.ascale.numpy()), _bits(sym_scale(x2).numpy()))
+
+
+# ---- a checkpoint written by the reference's own writer, and what its own loader makes of it ----
+
+def _checkpoint_fixture():
+    import importlib.util
+    import json
+
+    golden = Path(__file__).parent / "golden"
+    spec = importlib.util.spec_from_file_location("_make_checkpoint_fixture", golden / "make_checkpoint_fixture.py")
+    gen = importlib.util.module_from_spec(spec)
+    spec.loader.exec_module(gen)  # for build_toy and describe only; its main() is what touches the reference
+    return golden, gen, json.loads((golden / "reference_loader_outcome.json").read_text())
+
+
+@pytest.mark.parametrize("tag", ["v1", "legacy"])
+def test_reference_written_checkpoint_loads_as_the_reference_loads_it(tag):
+    """tests/golden/reference_written_packed_{v1,legacy}.pt were written by the reference's save_packed_checkpoint
+    (packed_checkpoint.py:190-215) from a toy model of its own QuantLinear layers; reference_loader_outcome.json is
+    what its load_packed_quantized_model (:52-148) left behind.  This repository's loader on this repository's
+    QuantLinear ends in the same state: missing / unexpected keys, every flag of the layers, dropped fp weight and
+    quantizers, buffer names, dtypes and shapes of the state dict, and the keys a re-export would write."""
+    from dsaquant_amd.checkpoints import packed_checkpoint as pc
+    from dsaquant_amd.quantization.quant_linear import QuantLinear
+
+    golden, gen, want = _checkpoint_fixture()
+    path = str(golden / f"reference_written_packed_{tag}.pt")
+    ckpt = pc.load_quant_checkpoint(path, dcp_loader=None)
+    assert pc.is_packed_checkpoint(ckpt) == want["is_packed_checkpoint"][tag] is True
+    if tag == "v1":
+        assert ckpt["format"] == want["format"] == pc.PACKED_CHECKPOINT_FORMAT and ckpt["metadata"] == want["metadata"]
+        assert {k: [str(v.dtype), list(v.shape)] for k, v in ckpt["model"].items()} == want["saved_keys"]
+    model = gen.build_toy(QuantLinear, seed=1)
+    missing, unexpected = pc.load_packed_quantized_model(model, ckpt, quant_linear_cls=QuantLinear, dtype=torch.float16,
+                                                        device=torch.device("cpu"), require_vdm_kernel=False)
+    got = gen.describe(model, QuantLinear)
+    ref = want["loads"][tag]
+    assert list(missing) == ref["missing"] and list(unexpected) == ref["unexpected"]
+    assert got["layers"] == ref["layers"]
+    assert got["state_dict"] == ref["state_dict"]
+    assert {k: [str(v.dtype), list(v.shape)] for k, v in pc.packed_state_dict_from_model(model).items()} == ref["re_export"]
+    # the tensors themselves are the file's
+    sfx = dict(zip(pc.VDM_BUFFER_SUFFIXES, pc._LEGACY_BUFFER_SUFFIXES if tag == "legacy" else pc.VDM_BUFFER_SUFFIXES))
+    for name in ("q1", "q2"):
+        for new, stored in sfx.items():
+            assert torch.equal(getattr(getattr(model, name), new), ckpt["model"][f"{name}.{stored}"])
+    assert torch.equal(model.pre.weight, ckpt["model"]["pre.weight"]) and torch.equal(model.q1.bias, ckpt["model"]["q1.bias"])
+
+
+def test_writer_writes_what_the_reference_writer_wrote(tmp_path):
+    """save_packed_checkpoint on the model loaded from the reference-written file gives a file with the same
+    format string and, key for key, the same dtypes, shapes and bytes as the reference's re-export would hold."""
+    from dsaquant_amd.checkpoints import packed_checkpoint as pc
+    from dsaquant_amd.quantization.quant_linear import QuantLinear
+
+    golden, gen, want = _checkpoint_fixture()
+    ckpt = torch.load(str(golden / "reference_written_packed_v1.pt"), map_location="cpu", weights_only=True)
+    model = gen.build_toy(QuantLinear, seed=2)
+    pc.load_packed_quantized_model(model, ckpt, quant_linear_cls=QuantLinear, dtype=torch.float16, device=torch.device("cpu"),
+                                   require_vdm_kernel=False)
+    out = str(tmp_path / "rewritten.pt")
+    pc.save_packed_checkpoint(model, out, metadata=ckpt["metadata"])
+    again = torch.load(out, map_location="cpu", weights_only=True)
+    assert again["format"] == want["format"] and again["metadata"] == want["metadata"]
+    assert {k: [str(v.dtype), list(v.shape)] for k, v in again["model"].items()} == want["loads"]["v1"]["re_export"]
+    for k, v in again["model"].items():
+        assert torch.equal(v, ckpt["model"][k]), k
+
+
+def test_loader_errors_read_as_the_reference_loader_errors():
+    from dsaquant_amd.checkpoints import packed_checkpoint as pc
+    from dsaquant_amd.quantization.quant_linear import QuantLinear
+
+    golden, gen, want = _checkpoint_fixture()
+    ckpt = torch.load(str(golden / "reference_written_packed_v1.pt"), map_location="cpu", weights_only=True)
+    kw = dict(quant_linear_cls=QuantLinear, dtype=torch.float16, device=torch.device("cpu"), require_vdm_kernel=False)
+    plain = nn.Sequential(nn.Linear(4, 4))
+    cases = {
+        "missing_buffer": lambda: pc.load_packed_quantized_model(
+            gen.build_toy(QuantLinear), dict(ckpt, model={k: v for k, v in ckpt["model"].items() if k != "q2.vdm_weight_scale"}), **kw),
+        "other_format": lambda: pc.load_packed_quantized_model(gen.build_toy(QuantLinear), {"format": "other", "model": {}}, **kw),
+        "not_a_dict": lambda: pc.load_packed_quantized_model(gen.build_toy(QuantLinear), [1, 2], **kw),
+        "no_quant_layers": lambda: pc.load_packed_quantized_model(plain, {"format": pc.PACKED_CHECKPOINT_FORMAT, "model": plain.state_dict()}, **kw),
+    }
+    assert set(cases) == set(want["errors"])
+    for name, fn in cases.items():
+        with pytest.raises(Exception) as info:
+            fn()
+        assert [type(info.value).__name__, str(info.value)] == want["errors"][name], name
