@@ -69,6 +69,27 @@ def _to_kernel_mode(module: nn.Module) -> None:
             setattr(module, q, None)
 
 
+def _found_format(ckpt: Any):
+    return ckpt.get("format") if isinstance(ckpt, dict) else type(ckpt)
+
+
+def _stored_names(layer_name: str, state_dict: dict) -> dict:
+    """buffer name -> the key it is stored under: the current name if present, else the legacy one."""
+    names = {}
+    for current, legacy in zip(VDM_BUFFER_SUFFIXES, _LEGACY_BUFFER_SUFFIXES):
+        key = _key(layer_name, current)
+        names[current] = key if key in state_dict else _key(layer_name, legacy)
+    return names
+
+
+def _ordinary_entries(state_dict: dict, fp_weight_keys: set) -> dict:
+    """What goes through load_state_dict: everything but packed buffers (either naming), quantizer state, cached
+    fp16 biases and the fp weights of the quantized layers (packed_checkpoint.py:84-93)."""
+    packed = VDM_BUFFER_SUFFIXES + _LEGACY_BUFFER_SUFFIXES
+    skip = lambda k: k.endswith(packed) or _is_quantizer_state(k) or k.endswith("._bias_half") or k in fp_weight_keys  # noqa: E731
+    return {k: v for k, v in state_dict.items() if not skip(k)}
+
+
 def load_packed_quantized_model(model: nn.Module, packed_ckpt: dict, *, quant_linear_cls: type, dtype: torch.dtype,
                                 device: torch.device, require_vdm_kernel: bool = True) -> tuple:
     """Populate a freshly built model (Linear layers already swapped for
@@ -77,11 +98,12 @@ def load_packed_quantized_model(model: nn.Module, packed_ckpt: dict, *, quant_li
 
     Raises ValueError for an unknown format, AssertionError when the kernel
     library is required but unavailable, KeyError when a QuantLinear lacks any of
-    its three buffers, RuntimeError when no QuantLinear was populated.
+    its three buffers, RuntimeError when no QuantLinear was populated.  The outcome
+    on a file the reference's writer wrote is held to what the reference's loader
+    leaves behind (tests/golden/reference_loader_outcome.json).
     """
     if not is_packed_checkpoint(packed_ckpt):
-        found = packed_ckpt.get("format") if isinstance(packed_ckpt, dict) else type(packed_ckpt)
-        raise ValueError(f"Unsupported checkpoint format: {found}")
+        raise ValueError(f"Unsupported checkpoint format: {_found_format(packed_ckpt)}")
     if require_vdm_kernel:
         from dsaquant_amd.kernels.vdm_w4a4 import is_available, load_error
 
@@ -90,45 +112,39 @@ def load_packed_quantized_model(model: nn.Module, packed_ckpt: dict, *, quant_li
     state_dict = packed_ckpt["model"]
     quant_layers = {name: m for name, m in model.named_modules() if isinstance(m, quant_linear_cls)}
     fp_weight_keys = {_key(name, "weight") for name in quant_layers}
-    packed_suffixes = VDM_BUFFER_SUFFIXES + _LEGACY_BUFFER_SUFFIXES
 
-    plain_state = {
-        k: v for k, v in state_dict.items()
-        if not k.endswith(packed_suffixes) and not _is_quantizer_state(k) and not k.endswith("._bias_half") and k not in fp_weight_keys
-    }
-    missing, unexpected = model.load_state_dict(plain_state, strict=False, assign=True)
-    missing = [k for k in missing if k not in fp_weight_keys and not _is_quantizer_state(k)]
+    # 1. everything that is not W4A4 state, through the ordinary route
+    report = model.load_state_dict(_ordinary_entries(state_dict, fp_weight_keys), strict=False, assign=True)
+    missing = [k for k in report.missing_keys if k not in fp_weight_keys and not _is_quantizer_state(k)]
 
+    # 2. the packed buffers, attached layer by layer; a layer with any buffer absent is reported, not half-loaded
     absent: list = []
     populated = 0
     for name, module in quant_layers.items():
-        resolved = {}
-        for suffix, legacy in zip(VDM_BUFFER_SUFFIXES, _LEGACY_BUFFER_SUFFIXES):
-            k = _key(name, suffix)
-            resolved[suffix] = k if k in state_dict else _key(name, legacy)
-        gone = [k for k in resolved.values() if k not in state_dict]
+        stored = _stored_names(name, state_dict)
+        gone = [key for key in stored.values() if key not in state_dict]
         if gone:
-            absent.extend(gone)
+            absent += gone
             continue
-        for suffix, k in resolved.items():
-            _attach_buffer(module, suffix, state_dict[k])
+        for buffer_name, key in stored.items():
+            _attach_buffer(module, buffer_name, state_dict[key])
         _to_kernel_mode(module)
         populated += 1
-
     if absent:
         raise KeyError(f"Packed checkpoint is missing {len(absent)} VDM buffers, e.g. {', '.join(absent[:8])}")
-    if populated == 0:
+    if not populated:
         raise RuntimeError("No QuantLinear layers were populated from the packed checkpoint")
 
-    del state_dict, plain_state
+    del state_dict
     gc.collect()
 
+    # 3. dtype / device, then the fp16 bias each kernel call takes
     model = model.to(dtype).to(device)
     for module in model.modules():
         if isinstance(module, quant_linear_cls) and module.bias is not None:
             module._bias_half = module.bias.half().contiguous()
     print(f"Loaded packed DSAQuant W4A4 checkpoint: {populated} QuantLinear layers")
-    return list(missing), list(unexpected)
+    return list(missing), list(report.unexpected_keys)
 
 
 def enable_quant_kernels(model: nn.Module, *, quant_linear_cls: type) -> None:
