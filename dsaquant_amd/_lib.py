@@ -52,6 +52,7 @@ SIGNATURES = {
     "vdmq_quantize_act_bf6": (_int, [_p, _i64, _i64, _i64, _f32, _int, _p, _p, _p]),
     "vdmq_quantize_act_ln_bf6": (_int, [_p, _i64, _i64, _i64, _f32, _int, _p, _p, _i64, _i64, _f32, _p, _p, _p]),
     "vdmq_workspace_bytes_bf6": (_i64, [_i64, _i64]),
+    "vdmq_bf6_pays": (_int, [_i64, _i64, _i64]),
     "vdmq_linear_w4a4_bf6": (_int, [_p, _i64, _i64, _i64, _f32, _int, _p, _p, _p, _p, _i64, _i64, _p, _i64, _p]),
     "vdmq_native_to_bf6": (_int, [_p, _i64, _i64, _p, _p]),
     "vdmq_gemm_w4a4_bf6": (_int, [_p, _p, _p, _p, _p, _p, _i64, _i64, _i64, _i64, _p]),

@@ -336,6 +336,16 @@ int vdmq_gemm_w4a4_bf6_acc(const void *xblocks, const void *wblocks, int32_t *ac
     return gemm_bf6_checked(xblocks, nullptr, wblocks, nullptr, nullptr, nullptr, acc, M, N, K, N, GemmTail{}, stream);
 }
 
+int vdmq_bf6_pays(int64_t M, int64_t N, int64_t K) {
+    if (M <= 0 || N <= 0 || K <= 0) return 0;
+    // Measured, quantizer + GEMM, int8 time / bf6 time: 4096 x 1536 -> 4608 (288 tiles) 0.90, 8192 x 1536 -> 4608 (576)
+    // 1.05, 32760 x 1536 -> 1536 (768) 1.03, 2048 x 5120 -> 5120 (160) 1.15, 4096 x 8960 -> 1536 (96) 0.93,
+    // 32760 x 8960 -> 1536 1.22, 75600 x 5120 -> 15360 1.17.
+    constexpr int64_t kMinTiles = 512, kLongK = 4096;
+    const int64_t tiles = ((M + 255) / 256) * ((N + 255) / 256);
+    return tiles >= kMinTiles || (K >= kLongK && 4 * tiles >= kMinTiles) ? 1 : 0;
+}
+
 int64_t vdmq_workspace_bytes_bf6(int64_t M, int64_t K) {
     if (M < 0 || K <= 0) return 0;
     return (bf6_bytes(M, K) + 255) / 256 * 256 + (M * 2 + 255) / 256 * 256;

@@ -147,14 +147,9 @@ def clear_native_cache() -> None:
 # ------------------------------------------------- which matrix instructions run the GEMM
 # "int8": v_mfma_i32_32x32x32_i8 on nibbles widened in registers.  "bf6": v_mfma_f32_32x32x64_f8f6f4 on 6-bit
 # floats (twice the rate, no widening work; every int4 value is exact in E3M2, so is the fp32 accumulation).
-# Both give bit-identical results.  "auto" takes bf6 where it is faster (its kernel has one tile shape, 256 x 256):
-# problems with at least _BF6_MIN_TILES output tiles, or a quarter of that when K is long enough for the K loop
-# to outweigh a tile's prologue and epilogue.  Measured, quantizer + GEMM, int8 time / bf6 time: 4096 x 1536 ->
-# 4608 (288 tiles) 0.90, 8192 x 1536 -> 4608 (576) 1.05, 32760 x 1536 -> 1536 (768) 1.03, 2048 x 5120 -> 5120 (160)
-# 1.15, 4096 x 8960 -> 1536 (96) 0.93, 32760 x 8960 -> 1536 1.22, 75600 x 5120 -> 15360 1.17.
+# Both give bit-identical results.  "auto" asks the library (vdmq_bf6_pays: bf6 for problems with enough 256 x 256
+# output tiles, fewer when K is long).
 _MATRIX_PATH = os.environ.get("VDMQ_MATRIX_PATH", "auto")
-_BF6_MIN_TILES = 512
-_BF6_LONG_K = 4096
 
 
 def set_matrix_path(name: str) -> None:
@@ -173,8 +168,7 @@ def _use_bf6(M: int, N: int, K: int, out_dtype: torch.dtype = torch.float16) -> 
         return False
     if _MATRIX_PATH == "bf6":
         return True
-    tiles = ((M + 255) // 256) * ((N + 255) // 256)
-    return tiles >= _BF6_MIN_TILES or (K >= _BF6_LONG_K and 4 * tiles >= _BF6_MIN_TILES)
+    return bool(_load_ext().vdmq_bf6_pays(M, N, K))
 
 
 _BF6_CACHE: Dict[tuple, torch.Tensor] = {}

@@ -439,3 +439,17 @@ def test_loader_errors_read_as_the_reference_loader_errors():
         with pytest.raises(Exception) as info:
             fn()
         assert [type(info.value).__name__, str(info.value)] == want["errors"][name], name
+
+
+def test_library_says_where_the_fp6_path_pays():
+    """vdmq_bf6_pays is a pure function of the sizes (no GPU work): the BASELINE shapes and the measured crossovers."""
+    from dsaquant_amd import _lib
+
+    lib = _lib.load()
+    pays = lambda M, N, K: bool(lib.vdmq_bf6_pays(M, N, K))  # noqa: E731
+    assert pays(75600, 15360, 5120) and pays(75600, 5120, 13824) and pays(32760, 1536, 1536) and pays(27280, 3072, 14336)
+    assert pays(2048, 5120, 5120)            # 160 tiles, long K
+    assert not pays(4096, 4608, 1536)        # config 0: 288 tiles, short K
+    assert not pays(4096, 1536, 8960)        # 96 tiles
+    assert not pays(512, 10240, 5120)        # the skinny cross-attention K/V case: 80 tiles
+    assert not pays(0, 128, 64) and not pays(-1, 128, 64)
