@@ -78,9 +78,6 @@ struct Bf6Cfg {
     static_assert(kLdsBytes * kOcc <= 160 * 1024, "the CU's LDS holds OCC workgroups");
 };
 using Bf6Big = Bf6Cfg<256, 256, 2, 4, 3, 1>;
-#ifndef VDMQ_BF6_PERSISTENT
-#define VDMQ_BF6_PERSISTENT 1
-#endif
 constexpr int kValuPerMfma = 3; /* address arithmetic and operand assembly spread between the MFMAs */
 
 struct Bf6TileMap {
@@ -690,7 +687,7 @@ int launch_bf6_cfg(const uint8_t *xblocks, const __half *ascale, const uint8_t *
     // the busiest XCD's tiles / places (M = 32760, N = 4608: 10 rounds for 9, still +4 %).
     const int64_t all_tiles = static_cast<int64_t>(tm.tiles_m) * tm.tiles_n;
     const int64_t busiest = tm.contig || best_load == 0 ? ceil_div(all_tiles, kXcds) : best_load;
-    const bool persistent = VDMQ_BF6_PERSISTENT && which < 2 && /* with the gated residual tail it needs more registers than there are: 10 % slower */
+    const bool persistent = which < 2 && /* with the gated residual tail it needs more registers than there are: 10 % slower */
                              static_cast<int64_t>(rounds) * 100 <= ceil_div(busiest, per) * 115;
     if (persistent) {
         using PKernel = void (*)(const uint8_t *, const uint8_t *, const __half *, const __half *, const __half *, __half *, int, int, int,

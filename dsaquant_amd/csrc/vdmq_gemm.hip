@@ -51,9 +51,7 @@ typedef _Float16 f16x8 __attribute__((ext_vector_type(8)));
 
 [[maybe_unused]] __device__ __forceinline__ void lds_barrier() {
     asm volatile("" ::: "memory");
-#ifndef VDMQ_DBG_NOBARRIER
     __builtin_amdgcn_s_barrier();
-#endif
     asm volatile("" ::: "memory");
 }
 
@@ -181,11 +179,7 @@ __device__ __forceinline__ void schedule_region() {
 // "super-tiles" of kGroupM x kGroupN tiles (32 = its CU count): the tiles that are
 // resident on an XCD together share kGroupM token row-blocks and kGroupN weight
 // row-blocks.
-#ifndef VDMQ_GROUP_M
-#define VDMQ_GROUP_M 8
-#define VDMQ_GROUP_N 4
-#endif
-constexpr int kXcds = 8, kGroupM = VDMQ_GROUP_M, kGroupN = VDMQ_GROUP_N;
+constexpr int kXcds = 8, kGroupM = 8, kGroupN = 4;
 
 struct TileMap {
     int tiles_m, tiles_n, super_n;
@@ -210,28 +204,10 @@ struct TileMap {
         st = (slot / per) * kXcds + xcd;
         if (st >= tm.start[kXcds]) return false;
     }
-#ifdef VDMQ_ORDER_M_FIRST
-    // consecutive super-tiles run down the token axis: an XCD keeps its weight super-column in L2
-    const int super_m = tm.start[kXcds] / tm.super_n;
-    tile_m = (st % super_m) * kGroupM + j / kGroupN;
-    tile_n = (st / super_m) * kGroupN + j % kGroupN;
-#else
     tile_m = (st / tm.super_n) * kGroupM + j / kGroupN;
     tile_n = (st % tm.super_n) * kGroupN + j % kGroupN;
-#endif
     return tile_m < tm.tiles_m && tile_n < tm.tiles_n;
 }
-
-#ifdef VDMQ_DBG_TIMELINE
-// debug build only: per-workgroup cycle stamps (entry, first stage landed, K loop done, epilogue done)
-__device__ unsigned long long g_timeline[4 * 32768];
-#define VDMQ_STAMP(i)                                                                                         \
-    do {                                                                                                      \
-        if (threadIdx.x == 0 && blockIdx.x < 32768) g_timeline[blockIdx.x * 4 + (i)] = __builtin_readcyclecounter(); \
-    } while (0)
-#else
-#define VDMQ_STAMP(i)
-#endif
 
 // OUT_MODE: 0 = scaled output, 1 = scaled output with non-temporal stores, 2 = raw int32 accumulators,
 // 3 / 4 = 0 / 1 followed by the gated residual update (a separate instantiation: carrying the tail's
@@ -249,17 +225,6 @@ __global__ __launch_bounds__(Cfg::kThreads, Cfg::kOccupancy * Cfg::kWaves / 4) v
 
     int tile_m, tile_n;
     if (!map_tile(tmap, blockIdx.x, tile_m, tile_n)) return;
-    VDMQ_STAMP(0);
-#ifdef VDMQ_STAGGER
-    // Two workgroups share a CU.  The first grid-wide wave of workgroups fills slot
-    // one of every CU, the next one slot two: hold the latter back by about half a
-    // tile so that one workgroup's epilogue runs under the other's MFMAs.  Later
-    // workgroups inherit the phase of the slot they fill.
-    if (Cfg::kOccupancy == 2 && blockIdx.x >= VDMQ_STAGGER && blockIdx.x < 2 * VDMQ_STAGGER) {
-        const int naps = (ldk / Cfg::kRowBytes) * Cfg::kKStepElems / 1024;
-        for (int i = 0; i < naps; ++i) __builtin_amdgcn_s_sleep(127);
-    }
-#endif
     const int m0 = tile_m * BM, n0 = tile_n * BN;
     const int lane = threadIdx.x & 63;
     const int wave = __builtin_amdgcn_readfirstlane(threadIdx.x >> 6);
@@ -335,7 +300,6 @@ __global__ __launch_bounds__(Cfg::kThreads, Cfg::kOccupancy * Cfg::kWaves / 4) v
     else
         __builtin_amdgcn_s_waitcnt(waitcnt_imm(0, 15));
     lds_barrier();
-    VDMQ_STAMP(1);
     if (f16_out) { /* wave-private: the epilogue's reads follow these writes in the wave's own LDS queue */
 #pragma unroll
         for (int i = 0; i < (Cfg::kWaveM + 63) / 64; ++i)
@@ -391,9 +355,7 @@ __global__ __launch_bounds__(Cfg::kThreads, Cfg::kOccupancy * Cfg::kWaves / 4) v
             widen_frags<Cfg, 1>(hi, wc, xc);
             mma_step<Cfg>(acc, lo);
             schedule_region<Cfg, Cfg::kNI + Cfg::kMI, 0>();
-#ifndef VDMQ_DBG_NOLOAD
             if (STEADY && j + 1 == R) issue_stage<Cfg>(wsrc, xsrc, kpos(kt + S) * RB, goff, lds + cur * Cfg::kStageBytes, wave);
-#endif
             widen_frags<Cfg, 0>(lo, wn, xn);
             mma_step<Cfg>(acc, hi);
             if (STEADY && j + 1 == R)
@@ -406,23 +368,9 @@ __global__ __launch_bounds__(Cfg::kThreads, Cfg::kOccupancy * Cfg::kWaves / 4) v
     int kt = 0;
     for (; kt + S < ksteps; ++kt) k_step(kt, std::true_type{});
     for (; kt < ksteps; ++kt) k_step(kt, std::false_type{});
-    VDMQ_STAMP(2);
 
     // Epilogue.  Accumulator register r of a 32x32 tile holds
     // n = 8*(r/4) + 4*(lane/32) + r%4, m = lane%32.
-#ifdef VDMQ_DBG_NOEPI
-    if (!ACC_OUT) {
-        int sum = 0;
-#pragma unroll
-        for (int ni = 0; ni < Cfg::kNI; ++ni)
-#pragma unroll
-            for (int mi = 0; mi < Cfg::kMI; ++mi)
-#pragma unroll
-                for (int r = 0; r < 16; ++r) sum ^= acc[ni][mi][r];
-        if (sum == 0x12345678) static_cast<int *>(out)[threadIdx.x] = sum;
-        return;
-    }
-#endif
     if (!ACC_OUT && out_dtype == VDMQ_OUT_F16) {
         // fp16 path: scale in the accumulator layout, round to fp16, transpose one
         // 32-row strip at a time through LDS (the stage ring is idle: every wave
@@ -448,10 +396,7 @@ __global__ __launch_bounds__(Cfg::kThreads, Cfg::kOccupancy * Cfg::kWaves / 4) v
         // looks at the vector offset only (a scalar offset is added after it), so the row goes into the vector
         // offset: one addition per store where a 64-bit address takes a multiplication and several additions.
         const int wave_rows = min(max(M - (m0 + wm0), 0), Cfg::kWaveM);
-        if (n0 + wn0 >= N || wave_rows == 0) {
-            VDMQ_STAMP(3);
-            return; /* the same for the whole wave */
-        }
+        if (n0 + wn0 >= N || wave_rows == 0) return; /* the same for the whole wave */
         const __amdgpu_buffer_rsrc_t out_rsrc = __builtin_amdgcn_make_buffer_rsrc(
             static_cast<__half *>(out) + static_cast<int64_t>(m0 + wm0) * ldo + n0 + wn0, 0, wave_rows * static_cast<int>(ldo) * 2, 0x00020000);
         const int out_voff = ((lane / PR) * static_cast<int>(ldo) + (lane % PR) * 8) * 2;
@@ -506,17 +451,14 @@ __global__ __launch_bounds__(Cfg::kThreads, Cfg::kOccupancy * Cfg::kWaves / 4) v
                 // operations per element, each rounded like the fp16 tensor operations they replace
                 if (TAIL && tail.gate != nullptr && mrow < M) hv *= gv[it];
                 if (TAIL && tail.residual != nullptr && mrow < M) hv = rv[it] + hv;
-#ifndef VDMQ_DBG_NOSTORE
                 // A large output is not re-read before it falls out of the caches anyway: streaming it (nt) keeps
                 // the operands (and the next quantizer's writes) in the Infinity Cache (measured: next quantizer
                 // 5.76 -> 6.01 TB/s).
                 __builtin_amdgcn_raw_buffer_store_b128(__builtin_bit_cast(u32x4, hv), out_rsrc,
                                                        out_voff + (mi * 32 + it * (64 / PR)) * static_cast<int>(ldo) * 2, 0,
                                                        STREAM_OUT ? 2 /* nt */ : 0);
-#endif
             }
         }
-        VDMQ_STAMP(3);
         return;
     }
 #pragma unroll
@@ -607,11 +549,7 @@ int launch_cfg(const uint8_t *qact, const __half *ascale, const uint8_t *wq, con
     // A large output is not re-read before it falls out of the caches anyway:
     // streaming it keeps the operands (and the next quantizer's writes) in the
     // Infinity Cache.
-#ifdef VDMQ_DBG_NOSTREAM
-    const bool stream_out = false;
-#else
     const bool stream_out = M * N * 2 > (int64_t(224) << 20);
-#endif
     const bool has_tail = tail.gate != nullptr || tail.residual != nullptr;
     const int which = acc_out != nullptr ? 2 : (stream_out ? 1 : 0) + (has_tail ? 3 : 0);
     using Kernel = void (*)(const uint8_t *, const uint8_t *, const __half *, const __half *, const __half *, void *, int, int32_t *, int,
@@ -639,34 +577,19 @@ int launch_cfg(const uint8_t *qact, const __half *ascale, const uint8_t *wq, con
 int launch_gemm(const uint8_t *qact, const __half *ascale, const uint8_t *wq, const __half *wscale, const __half *bias, void *out,
                 int out_dtype, int32_t *acc_out, int64_t M, int64_t N, int64_t K, int64_t ldo, const GemmTail &tail, hipStream_t s) {
     if (M == 0 || N == 0) return VDMQ_OK;
-#ifndef VDMQ_GEMM_CFG
-#define VDMQ_GEMM_CFG 256, 256, 2, 4, 2, 1, 256
-#endif
-#ifndef VDMQ_GEMM_MID_CFG
-#define VDMQ_GEMM_MID_CFG 256, 128, 2, 2, 3, 2, 128
-#endif
-#ifndef VDMQ_GEMM_SMALL_CFG
-#define VDMQ_GEMM_SMALL_CFG 128, 128, 2, 2, 3, 2, 128
-#endif
     // One 8-wave workgroup per CU with a 256 x 256 tile is the fastest steady state, but its
     // prologue and epilogue run with the matrix pipes idle.  When a CU sees only a few such
     // tiles, or K is short, two 4-wave workgroups per CU (one's epilogue under the other's K
     // loop) win: 256 x 128 tiles (Wan-1.3B: o-proj +19 %, FFN-down +12 %, QKV +4 %).  With
     // fewer than two large tiles per CU (M = 512 text tokens) 128 x 128 tiles fill the chip.
-    using Big = GemmCfg<VDMQ_GEMM_CFG>;
+    using Big = GemmCfg<256, 256, 2, 4, 2, 1, 256>;
+    using Mid = GemmCfg<256, 128, 2, 2, 3, 2, 128>;
+    using Small = GemmCfg<128, 128, 2, 2, 3, 2, 128>;
     const int64_t big_tiles = ceil_div(M, Big::BM) * ceil_div(N, Big::BN);
-#ifndef VDMQ_DBG_ONE_CFG
-    if (big_tiles < 512) return launch_cfg<GemmCfg<VDMQ_GEMM_SMALL_CFG>>(qact, ascale, wq, wscale, bias, out, out_dtype, acc_out, M, N, K, ldo, tail, s);
+    if (big_tiles < 512) return launch_cfg<Small>(qact, ascale, wq, wscale, bias, out, out_dtype, acc_out, M, N, K, ldo, tail, s);
     if (big_tiles < 1024 || (K < 2048 && big_tiles < 4096))
-        return launch_cfg<GemmCfg<VDMQ_GEMM_MID_CFG>>(qact, ascale, wq, wscale, bias, out, out_dtype, acc_out, M, N, K, ldo, tail, s);
-#endif
+        return launch_cfg<Mid>(qact, ascale, wq, wscale, bias, out, out_dtype, acc_out, M, N, K, ldo, tail, s);
     return launch_cfg<Big>(qact, ascale, wq, wscale, bias, out, out_dtype, acc_out, M, N, K, ldo, tail, s);
 }
 
 }  // namespace vdmq
-
-#ifdef VDMQ_DBG_TIMELINE
-extern "C" int vdmq_debug_timeline(void *host_out, long long bytes) {
-    return hipMemcpyFromSymbol(host_out, HIP_SYMBOL(vdmq::g_timeline), bytes) == hipSuccess ? 0 : -1;
-}
-#endif

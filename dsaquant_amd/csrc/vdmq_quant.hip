@@ -234,10 +234,7 @@ struct Bf6Scratch { /* LDS of one workgroup */
 // row has gone to the transpose buffer and its registers are free: a workgroup that walks several
 // row groups loads the next row's chunk there, so those loads overlap the rest of this row's
 // conversion.  `phase` counts the groups this workgroup has staged (it picks the staging copy).
-#ifndef VDMQ_BF6_WALK_MIN_CHUNKS
-#define VDMQ_BF6_WALK_MIN_CHUNKS 17
-#endif
-constexpr bool bf6_walks(int nch) { return nch >= VDMQ_BF6_WALK_MIN_CHUNKS; }
+constexpr bool bf6_walks(int nch) { return nch >= 17; } /* rows longer than 8192: one workgroup per CU, which walks row groups */
 struct NoRefill {
     __device__ __forceinline__ void operator()(int) const {}
 };
@@ -616,7 +613,7 @@ int launch_reg(const __half *x, int64_t M, int64_t K, int64_t ldx, float clip, i
         const int64_t resident = !bf6_walks(NCH) ? groups
                                  : resident_workgroups(reinterpret_cast<const void *>(&quantize_rows_kernel<NCH, false, ACT, 1>),
                                                        kBf6Rows * kWaveSize, cache);
-        if (resident <= 0) return VDMQ_ELAUNCH;
+        if (resident <= 0) return fail(VDMQ_ELAUNCH, "quantize_rows_kernel: the occupancy query for the current device failed");
         hipLaunchKernelGGL((quantize_rows_kernel<NCH, false, ACT, 1>), dim3(static_cast<unsigned>(!bf6_walks(NCH) || groups < resident ? groups : resident)),
                            dim3(kBf6Rows * kWaveSize), 0, s, x, ldx, static_cast<int>(M), static_cast<int>(K),
                            static_cast<int>(bf6_kblocks(K) * 64), clip, qact, scale_h);
