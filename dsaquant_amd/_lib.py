@@ -40,6 +40,7 @@ SIGNATURES = {
     "vdmq_workspace_bytes": (_i64, [_i64, _i64]),
     "vdmq_linear_w4a4": (_int, [_p, _i64, _i64, _i64, _f32, _p, _p, _p, _p, _int, _i64, _i64, _p, _i64, _p]),
     "vdmq_linear_w4a4_ex": (_int, [_p, _i64, _i64, _i64, _f32, _int, _p, _p, _p, _p, _int, _i64, _i64, _p, _i64, _p]),
+    "vdmq_linear_w4a4_noalloc": (_int, [_p, _i64, _i64, _i64, _f32, _p, _p, _p, _p, _int, _i64, _i64, _p]),
     "vdmq_weight_v1_to_native": (_int, [_p, _p, _i64, _i64, _p]),
     "vdmq_weight_native_to_v1": (_int, [_p, _p, _i64, _i64, _p]),
     "vdmq_wscale_v1_to_plain": (_int, [_p, _p, _i64, _i64, _p]),

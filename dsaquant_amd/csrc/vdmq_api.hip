@@ -70,6 +70,38 @@ inline hipStream_t as_stream(vdmq_stream_t s) { return static_cast<hipStream_t>(
 
 using namespace vdmq;
 
+// Workspace of vdmq_linear_w4a4_noalloc: the quantized activation rows and the token scales of one call.  Every
+// device the library runs on holds its own copy of the array, at its own address, until the process ends.  In host
+// code the name stands for the symbol only (HIP_SYMBOL): the device address comes from hipGetSymbolAddress, once per
+// device, and that pointer is what reaches the kernels.
+static __device__ __align__(256) unsigned char scratch[VDMQ_NOALLOC_SCRATCH_BYTES];
+
+namespace {
+
+constexpr int kScratchMaxDevices = 64;
+void *g_scratch_ptr[kScratchMaxDevices]; /* device address of `scratch` on device i, 0 = not asked yet */
+
+int scratch_of_current_device(void **ptr) {
+    int dev = -1;
+    if (hipGetDevice(&dev) != hipSuccess || dev < 0 || dev >= kScratchMaxDevices) {
+        (void)hipGetLastError();
+        return fail(VDMQ_ELAUNCH, "no current HIP device");
+    }
+    void *p = __atomic_load_n(&g_scratch_ptr[dev], __ATOMIC_ACQUIRE);
+    if (p == nullptr) {
+        const hipError_t e = hipGetSymbolAddress(&p, HIP_SYMBOL(scratch));
+        if (e != hipSuccess || p == nullptr) {
+            (void)hipGetLastError();
+            return fail(VDMQ_ELAUNCH, "hipGetSymbolAddress(scratch) on device %d: %s", dev, hipGetErrorString(e));
+        }
+        __atomic_store_n(&g_scratch_ptr[dev], p, __ATOMIC_RELEASE); /* racing first calls store the same address */
+    }
+    *ptr = p;
+    return VDMQ_OK;
+}
+
+}  // namespace
+
 extern "C" {
 
 int vdmq_version(void) { return 1; }
@@ -278,6 +310,23 @@ int vdmq_linear_w4a4(const void *x, int64_t M, int64_t K, int64_t ldx, float cli
                      vdmq_stream_t stream) {
     return vdmq_linear_w4a4_ex(x, M, K, ldx, clip, VDMQ_ACT_NONE, wq, wscale, bias, out, out_dtype, N, ldo, workspace, workspace_bytes,
                                stream);
+}
+
+int vdmq_linear_w4a4_noalloc(const void *x, int64_t M, int64_t K, int64_t ldx, float clip, const void *wq, const void *wscale,
+                             const void *bias, void *out, int out_dtype, int64_t N, int64_t ldo, vdmq_stream_t stream) {
+    VDMQ_TRY(check_k(K));
+    VDMQ_TRY(check_n(N));
+    VDMQ_TRY(check_m(M));
+    const int64_t need = vdmq_workspace_bytes(M, K);
+    if (need > static_cast<int64_t>(VDMQ_NOALLOC_SCRATCH_BYTES))
+        return fail(VDMQ_ENOSPACE, "an [M = %lld, K = %lld] input needs %lld bytes of scratch, the built-in buffer holds %lld",
+                    (long long)M, (long long)K, (long long)need, (long long)VDMQ_NOALLOC_SCRATCH_BYTES);
+    if (M == 0) return VDMQ_OK;
+    void *ws = nullptr;
+    VDMQ_TRY(scratch_of_current_device(&ws));
+    // the quantizer writes every byte the GEMM reads (all M rows with their padding, all M scales): nothing of the
+    // previous call's contents is seen, nothing has to be cleared
+    return vdmq_linear_w4a4_ex(x, M, K, ldx, clip, VDMQ_ACT_NONE, wq, wscale, bias, out, out_dtype, N, ldo, ws, need, stream);
 }
 
 int64_t vdmq_bf6_bytes(int64_t rows, int64_t K) {

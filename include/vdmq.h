@@ -167,6 +167,22 @@ int vdmq_linear_ln_w4a4(const void *x, int64_t M, int64_t K, int64_t ldx, float 
                         int64_t ldv, int64_t rows_per_vec, float clip, const void *wq, const void *wscale, const void *bias, void *out,
                         int out_dtype, int64_t N, int64_t ldo, void *workspace, int64_t workspace_bytes, vdmq_stream_t stream);
 
+/* vdmq_linear_w4a4 for callers that cannot allocate device memory (code under
+ * HIP graph capture, tight serving loops, harnesses that forbid hipMalloc): no
+ * counterpart in the reference, whose entry points allocate their scratch with
+ * torch::empty on every call.  The workspace is a buffer of
+ * VDMQ_NOALLOC_SCRATCH_BYTES built into the library's device code (every GPU the
+ * library is used on holds one copy until the process ends); the call allocates
+ * and frees nothing.  Inputs with vdmq_workspace_bytes(M, K) beyond that size
+ * are refused with VDMQ_ENOSPACE before anything is launched.  All calls on one
+ * GPU share that buffer: calls that may overlap there (different streams, or
+ * threads) race; calls on one stream are ordered and safe.  The first call on a
+ * device looks the buffer's address up (and, like every first launch of a GEMM
+ * kernel, sets its LDS size attribute): make it before a graph capture starts. */
+#define VDMQ_NOALLOC_SCRATCH_BYTES (64 << 20)
+int vdmq_linear_w4a4_noalloc(const void *x, int64_t M, int64_t K, int64_t ldx, float clip, const void *wq, const void *wscale,
+                             const void *bias, void *out, int out_dtype, int64_t N, int64_t ldo, vdmq_stream_t stream);
+
 /* ---- bf6 matrix path (optional; no counterpart in the reference).
  * gfx950 multiplies 6-bit floats (E3M2) at twice its int8 rate, E3M2 holds every
  * int4 value exactly and fp32 accumulation of their products is exact for

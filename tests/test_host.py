@@ -47,6 +47,9 @@ def test_abi_rejects_bad_shapes_without_touching_the_gpu():
     assert lib.vdmq_gemm_w4a4(fake, fake, fake, fake, None, fake, 7, 4, 128, 128, 128, None) == -1
     assert lib.vdmq_linear_w4a4(fake, 4, 128, 128, 1.0, fake, fake, None, fake, 0, 128, 128, fake, 16, None) == -4
     assert lib.vdmq_act_v1_to_native(fake, fake, 100, 128, fake, fake, None) == -2
+    # the entry point with the built-in workspace refuses what does not fit it, before it looks for a device
+    assert lib.vdmq_linear_w4a4_noalloc(fake, 75600, 5120, 5120, 1.0, fake, fake, None, fake, 0, 128, 128, None) == -4
+    assert b"scratch" in lib.vdmq_last_error()
     assert lib.vdmq_quantize_act(fake, 0, 128, 128, 1.0, fake, fake, None) == 0  # empty input is fine
     with pytest.raises(_lib.VdmqError):
         _lib.check(-2)
