@@ -21,6 +21,15 @@ VDMQ_ACT_GELU_TANH = 1
 VDMQ_LN_MODULATE = 1
 VDMQ_LN_AFFINE = 2
 
+class GemmLaunchInfo(ctypes.Structure):
+    """vdmq_gemm_launch_info of include/vdmq.h."""
+    _fields_ = [("kernel", ctypes.c_int), ("tile_m", ctypes.c_int), ("tile_n", ctypes.c_int), ("group_m", ctypes.c_int),
+                ("group_n", ctypes.c_int), ("contiguous_runs", ctypes.c_int), ("split_k_tiles", ctypes.c_int),
+                ("workgroups", ctypes.c_int64)]
+
+
+KERNEL_GEMM_W4A4, KERNEL_GEMM_BF6, KERNEL_GEMM_BF6_PERSISTENT = 1, 2, 3
+
 # name -> (restype, argtypes); every symbol include/vdmq.h declares
 _i64, _p, _f32, _int = ctypes.c_int64, ctypes.c_void_p, ctypes.c_float, ctypes.c_int
 SIGNATURES = {
@@ -37,6 +46,7 @@ SIGNATURES = {
     "vdmq_gemm_w4a4": (_int, [_p, _p, _p, _p, _p, _p, _int, _i64, _i64, _i64, _i64, _p]),
     "vdmq_gemm_w4a4_ex": (_int, [_p, _p, _p, _p, _p, _p, _i64, _i64, _p, _i64, _p, _int, _i64, _i64, _i64, _i64, _p]),
     "vdmq_gemm_w4a4_acc": (_int, [_p, _p, _p, _i64, _i64, _i64, _p]),
+    "vdmq_last_gemm_launch": (_int, [ctypes.POINTER(GemmLaunchInfo)]),
     "vdmq_workspace_bytes": (_i64, [_i64, _i64]),
     "vdmq_linear_w4a4": (_int, [_p, _i64, _i64, _i64, _f32, _p, _p, _p, _p, _int, _i64, _i64, _p, _i64, _p]),
     "vdmq_linear_w4a4_ex": (_int, [_p, _i64, _i64, _i64, _f32, _int, _p, _p, _p, _p, _int, _i64, _i64, _p, _i64, _p]),
@@ -94,6 +104,13 @@ def load() -> ctypes.CDLL:
         fn.argtypes = argtypes
     _LIB = lib
     return lib
+
+
+def last_gemm_launch() -> GemmLaunchInfo:
+    """What the library chose for the last GEMM launched on this thread."""
+    info = GemmLaunchInfo()
+    check(load().vdmq_last_gemm_launch(ctypes.byref(info)))
+    return info
 
 
 def check(rc: int) -> None:

@@ -16,6 +16,10 @@ int fail(int code, const char *fmt, ...) {
     return code;
 }
 
+static thread_local vdmq_gemm_launch_info g_last_launch = {};
+
+void record_gemm_launch(const vdmq_gemm_launch_info &info) { g_last_launch = info; }
+
 int check_launch(const char *what) {
     hipError_t e = hipGetLastError();
     if (e != hipSuccess) return fail(VDMQ_ELAUNCH, "%s: launch failed: %s", what, hipGetErrorString(e));
@@ -147,12 +151,13 @@ int vdmq_gelu_tanh_f16(const void *x, void *y, int64_t n, vdmq_stream_t stream) 
 }
 
 static int ln_checked(const void *x, int64_t M, int64_t K, int64_t ldx, int ln_mode, const void *a, const void *b, int64_t ldv,
-                      int64_t rows_per_vec) {
+                      int64_t &rows_per_vec) {
     VDMQ_TRY(check_k(K));
     VDMQ_TRY(check_m(M));
     if (K > 16384) return fail(VDMQ_ESHAPE, "the fused LayerNorm needs K <= 16384 (got %lld)", (long long)K);
     if (ln_mode != VDMQ_LN_MODULATE && ln_mode != VDMQ_LN_AFFINE) return fail(VDMQ_EINVAL, "unknown ln_mode %d", ln_mode);
     if (rows_per_vec <= 0) return fail(VDMQ_ESHAPE, "rows_per_vec must be positive (got %lld)", (long long)rows_per_vec);
+    if (rows_per_vec > (int64_t(1) << 30)) rows_per_vec = int64_t(1) << 30; /* "one vector for every row": the kernels index with int */
     if (ldv < K || ldv % 8 != 0) return fail(VDMQ_ESHAPE, "ldv must be >= K and a multiple of 8 (got %lld)", (long long)ldv);
     if (ldx < K || ldx % 8 != 0) return fail(VDMQ_ESHAPE, "ldx must be >= K and a multiple of 8 (got %lld)", (long long)ldx);
     if (M == 0) return VDMQ_OK;
@@ -263,6 +268,13 @@ int vdmq_gemm_w4a4_ex(const void *qact, const void *ascale, const void *wq, cons
 int vdmq_gemm_w4a4_acc(const void *qact, const void *wq, int32_t *acc, int64_t M, int64_t N, int64_t K, vdmq_stream_t stream) {
     if (acc == nullptr && M != 0) return fail(VDMQ_EINVAL, "acc is null");
     return gemm_checked(qact, nullptr, wq, nullptr, nullptr, nullptr, VDMQ_OUT_F16, acc, M, N, K, N, GemmTail{}, stream);
+}
+
+int vdmq_last_gemm_launch(vdmq_gemm_launch_info *info) {
+    if (info == nullptr) return fail(VDMQ_EINVAL, "info is null");
+    if (g_last_launch.kernel == 0) return fail(VDMQ_EINVAL, "no GEMM was launched on this thread yet");
+    *info = g_last_launch;
+    return VDMQ_OK;
 }
 
 int64_t vdmq_workspace_bytes(int64_t M, int64_t K) {

@@ -616,12 +616,13 @@ int launch_bf6_cfg(const uint8_t *xblocks, const __half *ascale, const uint8_t *
         const int64_t sm = ceil_div(tm.tiles_m, gm), sn = ceil_div(tm.tiles_n, gn);
         const int64_t last_m = tm.tiles_m - (sm - 1) * gm, last_n = tm.tiles_n - (sn - 1) * gn;
         int64_t load[kXcds] = {};
-        if (sm * sn <= 4096) /* beyond that the edges no longer matter: the first shape is taken */
+        const bool modelled = sm * sn <= 4096; /* beyond that the edges no longer matter: the first shape is taken */
+        if (modelled)
             for (int64_t st = 0; st < sm * sn; ++st)
                 load[st % kXcds] += (st / sn == sm - 1 ? last_m : gm) * (st % sn == sn - 1 ? last_n : gn);
         int64_t worst = 0;
         for (int x = 0; x < kXcds; ++x) worst = load[x] > worst ? load[x] : worst;
-        if (best_load < 0 || worst * 10 <= best_load * 9) {
+        if (best_load < 0 || (modelled && best_load > 0 && worst * 10 <= best_load * 9)) {
             best_load = worst;
             tm.group_n_log2 = gn_log2;
             tm.super_n = static_cast<int>(sn);
@@ -702,10 +703,14 @@ int launch_bf6_cfg(const uint8_t *xblocks, const __half *ascale, const uint8_t *
         }
         hipLaunchKernelGGL(pk[which], dim3(kXcds * per), block, Cfg::kLdsBytes, s, xblocks, wblocks, ascale, wscale, bias, out,
                            static_cast<int>(M), static_cast<int>(N), static_cast<int>(bf6_kblocks(K)), ldo, tm, tail);
+        record_gemm_launch({VDMQ_KERNEL_GEMM_BF6_PERSISTENT, Cfg::BM, Cfg::BN, per >> tm.group_n_log2, 1 << tm.group_n_log2, tm.contig, 0,
+                            static_cast<int64_t>(kXcds * per)});
         return check_launch("gemm_bf6_persistent_kernel");
     }
     hipLaunchKernelGGL(kernels[which], grid, block, Cfg::kLdsBytes, s, xblocks, wblocks, ascale, wscale, bias, out, acc_out,
                        static_cast<int>(M), static_cast<int>(N), static_cast<int>(bf6_kblocks(K)), ldo, tm, tail);
+    record_gemm_launch({VDMQ_KERNEL_GEMM_BF6, Cfg::BM, Cfg::BN, per >> tm.group_n_log2, 1 << tm.group_n_log2, tm.contig, 0,
+                        static_cast<int64_t>(grid.x)});
     return check_launch("gemm_bf6_kernel");
 }
 

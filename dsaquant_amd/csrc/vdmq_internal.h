@@ -17,6 +17,7 @@ constexpr int kWaveSize = 64;
 
 int fail(int code, const char *fmt, ...) __attribute__((format(printf, 2, 3)));
 int check_launch(const char *what);
+void record_gemm_launch(const vdmq_gemm_launch_info &info); /* what vdmq_last_gemm_launch reports */
 
 inline int64_t k_padded(int64_t K) { return (K + kKStep - 1) / kKStep * kKStep; }
 inline int64_t ceil_div(int64_t a, int64_t b) { return (a + b - 1) / b; }

@@ -144,6 +144,26 @@ int vdmq_gemm_w4a4_ex(const void *qact, const void *ascale, const void *wq, cons
  * holds in `ipsum` before finalize_int_accum (vdm_w4a4_kernel.cu:650, :684). */
 int vdmq_gemm_w4a4_acc(const void *qact, const void *wq, int32_t *acc, int64_t M, int64_t N, int64_t K, vdmq_stream_t stream);
 
+/* What the library chose for the last GEMM it launched on this thread (any of the
+ * vdmq_gemm_* / vdmq_linear_* entry points): which kernel, its output tile, the
+ * shape of the groups of tiles ("super-tiles") an XCD works on together, whether
+ * every XCD walks one contiguous run of them, and the grid.  No counterpart in
+ * the reference (one kernel, one tile shape, vdm_w4a4_kernel.cu:819); for tests
+ * and tuning: the choice never changes a result bit.  Returns VDMQ_EINVAL when
+ * nothing was launched yet. */
+#define VDMQ_KERNEL_GEMM_W4A4 1           /* int8 matrix path */
+#define VDMQ_KERNEL_GEMM_BF6 2            /* bf6 matrix path, one workgroup per tile */
+#define VDMQ_KERNEL_GEMM_BF6_PERSISTENT 3 /* bf6 matrix path, one workgroup per CU walking tiles */
+typedef struct vdmq_gemm_launch_info {
+    int kernel;                 /* VDMQ_KERNEL_* */
+    int tile_m, tile_n;         /* output tile of one workgroup: token rows x channels */
+    int group_m, group_n;       /* super-tile, in tiles */
+    int contiguous_runs;        /* 1: each XCD walks one contiguous run of super-tiles, K direction alternating */
+    int split_k_tiles;          /* tiles of the last, partly filled round whose K range was split over idle CUs */
+    int64_t workgroups;         /* grid size */
+} vdmq_gemm_launch_info;
+int vdmq_last_gemm_launch(vdmq_gemm_launch_info *info);
+
 /* Bytes of caller workspace vdmq_linear_w4a4 needs for an [M, K] input. */
 int64_t vdmq_workspace_bytes(int64_t M, int64_t K);
 
