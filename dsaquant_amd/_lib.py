@@ -8,8 +8,7 @@ from pathlib import Path
 from typing import Optional
 
 _PKG = Path(__file__).resolve().parent
-# VDMQ_LIBRARY points at another build of the same C ABI (e.g. a tuning variant)
-LIB_PATH = Path(os.environ.get("VDMQ_LIBRARY", str(_PKG / "libvdmq.so")))
+LIB_PATH = _PKG / "libvdmq.so"
 CSRC = _PKG / "csrc"
 
 _LIB: Optional[ctypes.CDLL] = None
@@ -66,6 +65,7 @@ SIGNATURES = {
     "vdmq_bf6_pays": (_int, [_i64, _i64, _i64]),
     "vdmq_linear_w4a4_bf6": (_int, [_p, _i64, _i64, _i64, _f32, _int, _p, _p, _p, _p, _i64, _i64, _p, _i64, _p]),
     "vdmq_native_to_bf6": (_int, [_p, _i64, _i64, _p, _p]),
+    "vdmq_weight_v1_to_bf6": (_int, [_p, _p, _i64, _i64, _p]),
     "vdmq_gemm_w4a4_bf6": (_int, [_p, _p, _p, _p, _p, _p, _i64, _i64, _i64, _i64, _p]),
     "vdmq_gemm_w4a4_bf6_ex": (_int, [_p, _p, _p, _p, _p, _p, _i64, _i64, _p, _i64, _p, _i64, _i64, _i64, _i64, _p]),
     "vdmq_gemm_w4a4_bf6_acc": (_int, [_p, _p, _p, _i64, _i64, _i64, _p]),

@@ -8,8 +8,10 @@ where, for every QuantLinear ``<name>``, the state dict holds
 ``<name>.vdm_weight_packed`` (u8 [N, K/2]), ``<name>.vdm_weight_scale_packed``
 (fp16 [N, K/64]), ``<name>.vdm_weight_scale`` (fp16 [N]) and ``<name>.bias``
 but no fp ``<name>.weight`` and no quantizer state.  Buffers stay in the v1
-byte layout in the module (they are the state-dict contract); the gfx950
-kernels relayout them once on first use.
+byte layout in the module (they are the state-dict contract); the loader
+relays each of them once, as it puts the model on the GPU, into the one form
+the gfx950 kernels stream for that layer (bf6 blocks or native int4 rows,
+3/4 or 1/2 byte per weight beside the v1 buffer).
 """
 from __future__ import annotations
 
@@ -143,8 +145,21 @@ def load_packed_quantized_model(model: nn.Module, packed_ckpt: dict, *, quant_li
     for module in model.modules():
         if isinstance(module, quant_linear_cls) and module.bias is not None:
             module._bias_half = module.bias.half().contiguous()
+    _prepare_for_kernels(model, device)
     print(f"Loaded packed DSAQuant W4A4 checkpoint: {populated} QuantLinear layers")
     return list(missing), list(report.unexpected_keys)
+
+
+def _prepare_for_kernels(model: nn.Module, device) -> None:
+    """The point at which the reference has its buffers attached and on the device (packed_checkpoint.py:102-148):
+    relay them now, on the current stream, rather than inside the first forward (which may be under graph
+    capture).  Nothing to do on a machine without the kernel library or for a model kept on the CPU."""
+    if torch.device(device).type != "cuda":
+        return
+    from dsaquant_amd.kernels import vdm_w4a4
+
+    if vdm_w4a4.is_available():
+        vdm_w4a4.prepare_model(model)
 
 
 def enable_quant_kernels(model: nn.Module, *, quant_linear_cls: type) -> None:
@@ -173,6 +188,23 @@ def enable_fused_qkv(model: nn.Module, *, quant_linear_cls: type, attention_cls:
         if all(isinstance(p, quant_linear_cls) and p.use_vdm_kernel for p in qkv):
             module.use_fused_qkv_kernel = True
             module.qkv_kernel_backend = "vdm"
+            _prepare_fused(module)
+
+
+def _prepare_fused(attention: nn.Module) -> None:
+    """The concatenated q|k|v (self-attention) or k|v (cross-attention) weight in the kernels' form, relaid from the
+    projections' packed buffers; those projections are never called on their own from now on, so what was prepared
+    for each of them alone is released."""
+    from dsaquant_amd.fused_qkv import fused_parts
+    from dsaquant_amd.kernels import vdm_w4a4
+
+    for names in fused_parts(attention):
+        layers = [getattr(attention, n) for n in names]
+        if not all(l.vdm_weight_packed.is_cuda for l in layers) or not vdm_w4a4.is_available():
+            continue
+        for l in layers:
+            vdm_w4a4.release_prepared(l.vdm_weight_packed)
+        vdm_w4a4.prepare_model(attention)
 
 
 def packed_state_dict_from_model(model: nn.Module, *, float_dtype: torch.dtype = torch.float16) -> dict:

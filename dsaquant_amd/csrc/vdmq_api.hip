@@ -355,6 +355,14 @@ int vdmq_native_to_bf6(const void *native, int64_t rows, int64_t K, void *blocks
     return launch_nibbles_to_bf6(static_cast<const uint8_t *>(native), rows, K, static_cast<uint8_t *>(blocks), as_stream(stream));
 }
 
+int vdmq_weight_v1_to_bf6(const void *qweight_v1, void *wblocks, int64_t N, int64_t K, vdmq_stream_t stream) {
+    VDMQ_TRY(check_k(K));
+    VDMQ_TRY(check_n(N));
+    VDMQ_TRY(check_ptr(qweight_v1, "qweight_v1"));
+    VDMQ_TRY(check_ptr(wblocks, "wblocks"));
+    return launch_weight_v1_to_bf6(static_cast<const uint8_t *>(qweight_v1), N, K, static_cast<uint8_t *>(wblocks), as_stream(stream));
+}
+
 static int gemm_bf6_checked(const void *xblocks, const void *ascale, const void *wblocks, const void *wscale, const void *bias, void *out,
                             int32_t *acc, int64_t M, int64_t N, int64_t K, int64_t ldo, const GemmTail &tail, vdmq_stream_t stream) {
     VDMQ_TRY(check_k(K));

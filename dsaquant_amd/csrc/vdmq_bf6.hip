@@ -554,7 +554,11 @@ __device__ __forceinline__ uint32_t bf6_code(uint32_t nib) {
     return (q < 0 ? 32u : 0u) | mag;
 }
 
-// native int4 rows (row-major, low nibble = even k) -> bf6 blocks; one thread per (row-block, k-block, lane)
+// int4 rows -> bf6 blocks; one thread per (row-block, k-block, lane).  The source is either native (row-major, low
+// nibble = even k, rows of src_row_bytes) or, for V1, a checkpoint's weight buffer in the v1 word order
+// (vdmq_layout.hip): the four 32-bit words that hold row n, k = 64 * kb + 32 * h + 8 * t ... + 7 (t = 0..3) are words
+// 2 * (r / 8) + h of the 16-byte groups ((n / 128 * KG + kb) * 8 + n / 16 % 8) * 32 + 4 * (r % 8) + t, r = n % 16.
+template <bool V1>
 __global__ __launch_bounds__(256) void nibbles_to_bf6_kernel(const uint8_t *__restrict__ src, int64_t rows, int64_t src_row_bytes,
                                                              int kblocks, int src_kblocks, uint8_t *__restrict__ dst, int64_t total) {
     const int64_t idx = static_cast<int64_t>(blockIdx.x) * blockDim.x + threadIdx.x;
@@ -567,8 +571,17 @@ __global__ __launch_bounds__(256) void nibbles_to_bf6_kernel(const uint8_t *__re
     const int h = l >> 5;
     uint32_t regs[6] = {0, 0, 0, 0, 0, 0};
     if (r < rows && kb < src_kblocks) {
-        const u32x4 v = *reinterpret_cast<const u32x4 *>(src + r * src_row_bytes + kb * 32 + h * 16); /* 32 nibbles */
-        const uint32_t w[4] = {v.x, v.y, v.z, v.w};
+        uint32_t w[4];
+        if (V1) {
+            const int r16 = static_cast<int>(r & 15);
+            const int64_t group = (((r >> 7) * src_kblocks + kb) * 8 + ((r >> 4) & 7)) * 32 + 4 * (r16 & 7);
+            const uint32_t *words = reinterpret_cast<const uint32_t *>(src);
+#pragma unroll
+            for (int t = 0; t < 4; ++t) w[t] = words[(group + t) * 4 + 2 * (r16 >> 3) + h];
+        } else {
+            const u32x4 v = *reinterpret_cast<const u32x4 *>(src + r * src_row_bytes + kb * 32 + h * 16); /* 32 nibbles */
+            w[0] = v.x, w[1] = v.y, w[2] = v.z, w[3] = v.w;
+        }
 #pragma unroll
         for (int e = 0; e < 32; ++e) {
             const uint64_t code = bf6_code((w[e / 8] >> (4 * (e % 8))) & 0xFu);
@@ -590,8 +603,17 @@ int launch_nibbles_to_bf6(const uint8_t *native, int64_t rows, int64_t K, uint8_
     if (rows == 0) return VDMQ_OK;
     const int64_t kblocks = bf6_kblocks(K);
     const int64_t total = (rows + 31) / 32 * kblocks * 64;
-    hipLaunchKernelGGL(nibbles_to_bf6_kernel, dim3(static_cast<unsigned>(ceil_div(total, 256))), dim3(256), 0, s, native, rows,
+    hipLaunchKernelGGL(nibbles_to_bf6_kernel<false>, dim3(static_cast<unsigned>(ceil_div(total, 256))), dim3(256), 0, s, native, rows,
                        k_padded(K) / 2, static_cast<int>(kblocks), static_cast<int>(k_padded(K) / 64), blocks, total);
+    return check_launch("nibbles_to_bf6_kernel");
+}
+
+int launch_weight_v1_to_bf6(const uint8_t *qweight_v1, int64_t N, int64_t K, uint8_t *blocks, hipStream_t s) {
+    if (N == 0) return VDMQ_OK;
+    const int64_t kblocks = bf6_kblocks(K);
+    const int64_t total = (N + 31) / 32 * kblocks * 64;
+    hipLaunchKernelGGL(nibbles_to_bf6_kernel<true>, dim3(static_cast<unsigned>(ceil_div(total, 256))), dim3(256), 0, s, qweight_v1, N,
+                       K / 2, static_cast<int>(kblocks), static_cast<int>(K / 64), blocks, total);
     return check_launch("nibbles_to_bf6_kernel");
 }
 

@@ -61,6 +61,7 @@ __host__ __device__ __forceinline__ int64_t bf6_piece(int64_t row, int kb, int h
 int64_t bf6_kblocks(int64_t K);
 int64_t bf6_bytes(int64_t rows, int64_t K);
 int launch_nibbles_to_bf6(const uint8_t *native, int64_t rows, int64_t K, uint8_t *blocks, hipStream_t stream);
+int launch_weight_v1_to_bf6(const uint8_t *qweight_v1, int64_t N, int64_t K, uint8_t *blocks, hipStream_t stream);
 int launch_gemm_bf6(const uint8_t *xblocks, const __half *ascale, const uint8_t *wblocks, const __half *wscale, const __half *bias,
                     __half *out, int32_t *acc_out, int64_t M, int64_t N, int64_t K, int64_t ldo, const GemmTail &tail,
                     hipStream_t stream);

@@ -151,8 +151,8 @@ class QuantizedInput:
 
 def linear_fused(
     x,
-    qweight: torch.Tensor,
-    wscales: torch.Tensor,
+    qweight,
+    wscales: Optional[torch.Tensor],
     bias: Optional[torch.Tensor] = None,
     clip_ratio: float = 1.0,
     bias_half: Optional[torch.Tensor] = None,
@@ -169,7 +169,8 @@ def linear_fused(
     or per token) and ``residual`` (fp16, shaped like the output) are folded into the
     GEMM epilogue as the two fp16 tensor operations of the reference's
     ``hidden_states + attn_output * gate`` (dit_block.py:102, :107, :112); either may
-    be omitted.  Returns a new tensor; nothing is updated in place."""
+    be omitted.  ``qweight`` may be a ``PreparedWeight`` (then ``wscales`` is ignored): the concatenated weight of a
+    fused projection.  Returns a new tensor; nothing is updated in place."""
     _k._load_ext()  # raises when the library is missing
     if isinstance(x, LnInput):
         if act is not None:
@@ -184,17 +185,21 @@ def linear_fused(
     else:
         pre = None
         x_2d, lead = _k._as_2d_half_contiguous(x)
+    prepared = isinstance(qweight, _k.PreparedWeight)
     if x_2d is not None:
-        _k._check_linear_shapes(x_2d, qweight, wscales)
         _k._require(x_2d.is_cuda, "input must be a CUDA tensor")
         M, K = x_2d.shape
         dev = x_2d.device
     else:
         M, K, dev = pre.M, pre.K, pre.device
+    if prepared:
+        if qweight.K != K:
+            raise ValueError("qweight shape must be [N, K/2]")
+    else:
         _k._check_packed_weight(qweight, wscales, K)
     act_code = _k._act_code(act)
-    native_w, wscale = _k._native_weights(qweight.contiguous(), wscales.contiguous())
-    N = native_w.shape[0]
+    weight = qweight if prepared else _k._prepared_weight(qweight, wscales)
+    N = weight.N
     b = bias_half if bias_half is not None else bias
     if b is not None:
         b = b.half().contiguous().view(-1)
@@ -218,11 +223,11 @@ def linear_fused(
     with torch.cuda.device(dev):
         out = torch.empty((M, N), dtype=torch.float16, device=dev)
         if M and isinstance(pre, QuantizedInput):
-            _k._gemm_dispatch(pre.qact, pre.scales, False, native_w, wscale, b, out, K, gate=g2, rows_per_gate=rows_per_gate, residual=r2)
+            _k._gemm_dispatch(pre.qact, pre.scales, False, weight, b, out, K, gate=g2, rows_per_gate=rows_per_gate, residual=r2)
         elif M:
             bf6 = _k._use_bf6(M, N, K)
             operand, scales = _k._quantize_for_gemm(x_2d, clip_ratio, act_code, bf6, None if pre is None else pre._args())
-            _k._gemm_dispatch(operand, scales, bf6, native_w, wscale, b, out, K, gate=g2, rows_per_gate=rows_per_gate, residual=r2)
+            _k._gemm_dispatch(operand, scales, bf6, weight, b, out, K, gate=g2, rows_per_gate=rows_per_gate, residual=r2)
     return out.view(*lead, N)
 
 
@@ -230,10 +235,10 @@ def qkv_projections_ln(attn, pre: LnInput):
     """Self-attention Q, K, V of ``pre`` through the cached concatenation Wq|Wk|Wv
     (the fused branch of ``get_qkv_projections``, attention.py:41-68 of the
     reference) with the LayerNorm fused into the one activation quantization."""
-    from .fused_qkv import _cat_cached
+    from .fused_qkv import _cat_prepared
 
-    w, s, b = _cat_cached(attn, ["to_q", "to_k", "to_v"], "qkv")
-    out = linear_ln_vdm_w4a4(pre, w, s, None, attn.to_q.kernel_clip_ratio, bias_half=b)
+    w, b = _cat_prepared(attn, ["to_q", "to_k", "to_v"], "qkv")
+    out = linear_ln_vdm_w4a4(pre, w, None, None, attn.to_q.kernel_clip_ratio, bias_half=b)
     n = attn.to_q.vdm_weight_packed.shape[0]
     return out.split(n, dim=-1)
 
@@ -241,8 +246,8 @@ def qkv_projections_ln(attn, pre: LnInput):
 def kv_projections(attn, encoder_hidden_states):
     """Cross-attention K, V through the cached concatenation Wk|Wv (attention.py:70-107 of the reference);
     ``encoder_hidden_states`` is the tensor or a ``QuantizedInput`` of it shared between blocks."""
-    from .fused_qkv import _cat_cached
+    from .fused_qkv import _cat_prepared
 
-    w, s, b = _cat_cached(attn, ["to_k", "to_v"], "kv")
-    kv = linear_fused(encoder_hidden_states, w, s, None, attn.to_k.kernel_clip_ratio, bias_half=b)
+    w, b = _cat_prepared(attn, ["to_k", "to_v"], "kv")
+    kv = linear_fused(encoder_hidden_states, w, None, None, attn.to_k.kernel_clip_ratio, bias_half=b)
     return kv.split(attn.to_k.vdm_weight_packed.shape[0], dim=-1)

@@ -9,9 +9,10 @@ self-attention), ``use_fused_qkv_kernel`` and ``qkv_kernel_backend``; optional
 
 Self-attention: ONE activation quantization and ONE GEMM against the cached
 row-concatenation Wq|Wk|Wv, split three ways.  Cross-attention: ``to_q`` on the
-tokens, one fused K|V GEMM on the encoder states.  The concatenated buffers are
-built on first use and cached on the module under the reference's attribute
-names (``_vdm_qkv_weight_packed`` ...).
+tokens, one fused K|V GEMM on the encoder states.  The concatenated weight is
+relaid once from the projections' own packed buffers into the form the kernels
+stream (no concatenated v1 copy is made); the concatenated bias is cached on
+the module under the reference's attribute name (``_vdm_qkv_bias_half`` ...).
 """
 from __future__ import annotations
 
@@ -20,13 +21,27 @@ from typing import List, Optional
 import torch
 
 
-def _cat_cached(attn, names: List[str], prefix: str):
-    """Concatenate the v1 buffers / biases of ``attn.<name>`` once and cache them."""
-    w_attr, s_attr, b_attr = f"_vdm_{prefix}_weight_packed", f"_vdm_{prefix}_weight_scale", f"_vdm_{prefix}_bias_half"
+def fused_parts(module):
+    """Names of the projections whose packed weights ``module`` uses as ONE concatenated weight: q|k|v of a
+    self-attention module and k|v of a cross-attention module once they are marked for the fused kernel path
+    (packed_checkpoint.py:167-188 of the reference sets the marks); nothing for any other module."""
+    if not (getattr(module, "use_fused_qkv_kernel", False) and getattr(module, "qkv_kernel_backend", None) == "vdm"):
+        return []
+    if not all(hasattr(module, n) and getattr(getattr(module, n), "vdm_weight_packed", None) is not None for n in ("to_q", "to_k", "to_v")):
+        return []
+    return [["to_q", "to_k", "to_v"]] if module.cross_attention_dim_head is None else [["to_k", "to_v"]]
+
+
+def _cat_prepared(attn, names: List[str], prefix: str):
+    """The concatenated weight of ``attn.<name>`` for the kernels and the concatenated fp16 bias (or None).  The
+    reference caches concatenated v1 buffers on the module (``_vdm_qkv_weight_packed`` ..., attention.py:44-54); the
+    kernels here never read a concatenated v1 buffer -- the operand is relaid from the projections' own buffers and
+    kept with them -- so only the bias keeps its cache attribute."""
+    from dsaquant_amd.kernels import vdm_w4a4 as k
+
+    b_attr = f"_vdm_{prefix}_bias_half"
     layers = [getattr(attn, n) for n in names]
-    if getattr(attn, w_attr, None) is None:
-        setattr(attn, w_attr, torch.cat([l.vdm_weight_packed for l in layers], dim=0).contiguous())
-        setattr(attn, s_attr, torch.cat([l.vdm_weight_scale_packed for l in layers], dim=0).contiguous())
+    weight = k._prepared([(l.vdm_weight_packed, l.vdm_weight_scale_packed) for l in layers])
     if getattr(attn, b_attr, None) is None:
         biases = [l._bias_half for l in layers]
         if any(b is not None for b in biases):
@@ -35,7 +50,15 @@ def _cat_cached(attn, names: List[str], prefix: str):
             setattr(attn, b_attr, torch.cat(filled, dim=0).contiguous())
         else:
             setattr(attn, b_attr, None)
-    return getattr(attn, w_attr), getattr(attn, s_attr), getattr(attn, b_attr)
+    return weight, getattr(attn, b_attr)
+
+
+def _project_cat(attn, names: List[str], prefix: str, x: torch.Tensor, clip_ratio: float):
+    from dsaquant_amd.kernels import vdm_w4a4 as k
+
+    weight, bias = _cat_prepared(attn, names, prefix)
+    out = k.linear_vdm_w4a4_prepared(x, weight, bias, clip_ratio)
+    return out.split(getattr(attn, names[0]).vdm_weight_packed.shape[0], dim=-1)
 
 
 def get_qkv_projections(attn, hidden_states: torch.Tensor, encoder_hidden_states: Optional[torch.Tensor]):
@@ -43,21 +66,10 @@ def get_qkv_projections(attn, hidden_states: torch.Tensor, encoder_hidden_states
         encoder_hidden_states = hidden_states
 
     if getattr(attn, "use_fused_qkv_kernel", False) and getattr(attn, "qkv_kernel_backend", None) == "vdm":
-        from dsaquant_amd.kernels.vdm_w4a4 import linear_vdm_w4a4, linear_vdm_w4a4_qkv
-
         if attn.cross_attention_dim_head is None:
-            w, s, b = _cat_cached(attn, ["to_q", "to_k", "to_v"], "qkv")
-            q, k, v = attn.to_q, attn.to_k, attn.to_v
-            return tuple(linear_vdm_w4a4_qkv(
-                hidden_states,
-                q.vdm_weight_packed, q.vdm_weight_scale_packed,
-                k.vdm_weight_packed, k.vdm_weight_scale_packed,
-                v.vdm_weight_packed, v.vdm_weight_scale_packed,
-                clip_ratio=q.kernel_clip_ratio, w_qkv_packed=w, w_qkv_scale=s, qkv_bias_half=b))
+            return tuple(_project_cat(attn, ["to_q", "to_k", "to_v"], "qkv", hidden_states, attn.to_q.kernel_clip_ratio))
         query = attn.to_q(hidden_states)
-        w, s, b = _cat_cached(attn, ["to_k", "to_v"], "kv")
-        kv = linear_vdm_w4a4(encoder_hidden_states, w, s, bias=None, clip_ratio=attn.to_k.kernel_clip_ratio, bias_half=b)
-        key, value = kv.split(attn.to_k.vdm_weight_packed.shape[0], dim=-1)
+        key, value = _project_cat(attn, ["to_k", "to_v"], "kv", encoder_hidden_states, attn.to_k.kernel_clip_ratio)
         return query, key, value
 
     if getattr(attn, "fused_projections", False):

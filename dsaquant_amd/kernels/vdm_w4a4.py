@@ -115,33 +115,185 @@ def k_padded(K: int) -> int:
     return int(_lib.load().vdmq_k_padded(K))
 
 
-# one-time v1 -> native relayout, cached per v1 tensor pair
-_NATIVE_CACHE: Dict[tuple, Tuple[torch.Tensor, torch.Tensor]] = {}
+# ------------------------------------------------- the weights in the form the kernels stream
+# A checkpoint's v1 buffers stay what the module holds (they are the state-dict contract).  The kernels want the
+# same integers either as native int4 rows (int8 matrix path) or as bf6 blocks (bf6 path), plus one fp16 scale per
+# channel.  A PreparedWeight makes those forms straight from the v1 buffers -- at load time through
+# prepare_weight() / prepare_model(), otherwise at the first call -- and keeps only the form that is used: a form
+# that was made ahead and never asked for is dropped as soon as the other one is.  It hangs on the v1 tensor
+# object itself (an attribute, so it lives exactly as long as that tensor and no address or version counter has
+# to be trusted to identify it); in-place writes to the v1 tensors are noticed where the tensor counts them.
+
+
+def _version_of(t: torch.Tensor):
+    # inference tensors do not count versions (reading ._version raises): they cannot be written in place either
+    return None if t.is_inference() else t._version
+
+
+class PreparedWeight:
+    """Operand forms of one packed weight, or of the row-concatenation of several (Wq|Wk|Wv): every 128-row block
+    of either form is self-contained, so the concatenation's forms are the parts' forms one after the other."""
+
+    def __init__(self, parts):
+        parts = [(q, s) for q, s in parts]
+        q0 = parts[0][0]
+        self.K = q0.shape[1] * 2
+        self.rows = [q.shape[0] for q, _ in parts]
+        self.N = sum(self.rows)
+        self.device = q0.device
+        for q, s in parts:
+            _check_device_tensor(q, "qweight", torch.uint8)
+            _check_device_tensor(s, "wscales", torch.float16)
+            _require(q.dim() == 2 and q.shape[1] * 2 == self.K and q.device == self.device, "the parts of a packed weight must agree in K and device")
+            _require(tuple(s.shape) == (q.shape[0], self.K // WARP_K), "wscales shape must be [N, K/64]")
+        self._parts = [(weakref.ref(q), weakref.ref(s)) for q, s in parts]
+        self._versions = [(_version_of(q), _version_of(s)) for q, s in parts]
+        self.native: Optional[torch.Tensor] = None
+        self.bf6: Optional[torch.Tensor] = None
+        self._used = {"native": False, "bf6": False}
+        lib = _load_ext()
+        with torch.cuda.device(self.device):
+            self.wscale = torch.empty((self.N,), dtype=torch.float16, device=self.device)
+            row = 0
+            for (q, s), n in zip(parts, self.rows):
+                _lib.check(lib.vdmq_wscale_v1_to_plain(s.data_ptr(), self.wscale[row:].data_ptr(), n, self.K, _stream(self.device)))
+                row += n
+
+    def matches(self, parts) -> bool:
+        if len(parts) != len(self._parts):
+            return False
+        for (rq, rs), (vq, vs), (q, s) in zip(self._parts, self._versions, parts):
+            if rq() is not q or rs() is not s or _version_of(q) != vq or _version_of(s) != vs:
+                return False
+        return True
+
+    def current(self) -> bool:
+        """The packed tensors still exist and have not been written since."""
+        parts = [(rq(), rs()) for rq, rs in self._parts]
+        return all(q is not None and s is not None for q, s in parts) and self.matches(parts)
+
+    def sources(self):
+        """The packed v1 tensors this weight was made from: ``[(qweight, wscales), ...]``."""
+        return self._sources()
+
+    def _sources(self):
+        parts = [(rq(), rs()) for rq, rs in self._parts]
+        if any(q is None for q, _ in parts):
+            raise _lib.VdmqError("the packed weight tensors of this prepared weight are gone")
+        return parts
+
+    def _build(self, form: str) -> torch.Tensor:
+        lib = _load_ext()
+        K = self.K
+        with torch.cuda.device(self.device):
+            s = _stream(self.device)
+            if form == "bf6":
+                out = torch.empty((int(lib.vdmq_bf6_bytes(self.N, K)),), dtype=torch.uint8, device=self.device)
+                row_bytes = int(lib.vdmq_bf6_bytes(32, K)) // 32
+                convert = lib.vdmq_weight_v1_to_bf6
+            else:
+                out = torch.empty((self.N, k_padded(K) // 2), dtype=torch.uint8, device=self.device)
+                row_bytes = k_padded(K) // 2
+                convert = lib.vdmq_weight_v1_to_native
+            flat, row = out.view(-1), 0
+            for (q, _), n in zip(self._sources(), self.rows):
+                _lib.check(convert(q.data_ptr(), flat[row * row_bytes:].data_ptr(), n, K, s))
+                row += n
+        return out
+
+    def operand(self, bf6: bool, eager: bool = False) -> torch.Tensor:
+        """The weights as bf6 blocks (``bf6``) or native int4 rows.  ``eager``: made ahead of use -- it does not count
+        as a use and drops nothing."""
+        form, other = ("bf6", "native") if bf6 else ("native", "bf6")
+        if getattr(self, form) is None:
+            setattr(self, form, self._build(form))
+        if not eager:
+            self._used[form] = True
+            if getattr(self, other) is not None and not self._used[other]:
+                setattr(self, other, None)  # made ahead for a call pattern that did not come
+        return getattr(self, form)
+
+    def extra_bytes(self) -> int:
+        return sum(t.numel() * t.element_size() for t in (self.native, self.bf6, self.wscale) if t is not None)
+
+
+_ATTR = "_vdmq_prepared"
+
+
+def _prepared(parts) -> PreparedWeight:
+    """The PreparedWeight of a packed weight given as ``[(qweight, wscales), ...]`` (one pair, or the pairs whose
+    rows are concatenated), kept on the first pair's qweight tensor."""
+    holder = parts[0][0]
+    kept = holder.__dict__.get(_ATTR)
+    if kept is not None:
+        for pw in kept:
+            if pw.matches(parts):
+                return pw
+        kept[:] = [pw for pw in kept if pw.current()]  # drop what was overwritten since
+    pw = PreparedWeight(parts)
+    holder.__dict__.setdefault(_ATTR, []).append(pw)
+    return pw
+
+
+def _prepared_weight(qweight: torch.Tensor, wscales: torch.Tensor) -> PreparedWeight:
+    if not (qweight.is_contiguous() and wscales.is_contiguous()):
+        # a fresh contiguous copy per call would be relaid per call: keep the copy with the tensor it came from
+        kept = qweight.__dict__.get("_vdmq_contiguous")
+        if kept is None or kept[0]() is not wscales or kept[1] != (_version_of(qweight), _version_of(wscales)):
+            kept = (weakref.ref(wscales), (_version_of(qweight), _version_of(wscales)), qweight.contiguous(), wscales.contiguous())
+            qweight.__dict__["_vdmq_contiguous"] = kept
+        qweight, wscales = kept[2], kept[3]
+    return _prepared([(qweight, wscales)])
+
+
+def prepare_weight(qweight: torch.Tensor, wscales: torch.Tensor, tokens: Optional[int] = None, path: Optional[str] = None) -> PreparedWeight:
+    """Relayout a packed weight now (load time, a known stream) instead of at its first call.  ``tokens``: the number
+    of rows its calls will have, which decides the matrix path under "auto" (default: a video-sized sequence)."""
+    pw = _prepared_weight(qweight, wscales)
+    pw.operand(_use_bf6(32768 if tokens is None else int(tokens), pw.N, pw.K, path=path), eager=True)
+    return pw
+
+
+def prepare_model(model, tokens: Optional[int] = None, path: Optional[str] = None) -> int:
+    """prepare_weight for every module of ``model`` that holds packed buffers and runs in kernel mode (the place the
+    reference attaches those buffers: packed_checkpoint.py:102-148, quant_linear.py:146-160).  Attention modules
+    marked for the fused QKV / KV path get the concatenated form instead of one per projection.  Returns the bytes
+    of HBM the prepared forms take beside the v1 buffers."""
+    from ..fused_qkv import fused_parts
+
+    done, total = set(), 0
+    for module in model.modules():
+        for names in fused_parts(module):
+            layers = [getattr(module, n) for n in names]
+            pw = _prepared([(l.vdm_weight_packed, l.vdm_weight_scale_packed) for l in layers])
+            pw.operand(_use_bf6(32768 if tokens is None else int(tokens), pw.N, pw.K, path=path), eager=True)
+            total += pw.extra_bytes()
+            done.update(id(l) for l in layers)
+    for module in model.modules():
+        if id(module) in done or not getattr(module, "use_vdm_kernel", False) or getattr(module, "vdm_weight_packed", None) is None:
+            continue
+        if not module.vdm_weight_packed.is_cuda:
+            continue
+        total += prepare_weight(module.vdm_weight_packed, module.vdm_weight_scale_packed, tokens, path).extra_bytes()
+    return total
+
+
+def release_prepared(qweight: torch.Tensor, concatenations: bool = False) -> None:
+    """Drop the prepared forms kept with ``qweight`` for itself (and, with ``concatenations``, for concatenations it
+    leads): a projection that is only ever used through its attention module's fused weight needs none of its own."""
+    kept = qweight.__dict__.get(_ATTR)
+    if kept is not None:
+        kept[:] = [pw for pw in kept if len(pw.rows) > 1 and not concatenations]
 
 
 def _native_weights(qweight: torch.Tensor, wscales: torch.Tensor) -> Tuple[torch.Tensor, torch.Tensor]:
-    key = (qweight.data_ptr(), wscales.data_ptr(), tuple(qweight.shape), qweight.device.index, qweight._version, wscales._version)
-    hit = _NATIVE_CACHE.get(key)
-    if hit is not None:
-        return hit
-    lib = _load_ext()
-    _check_device_tensor(qweight, "qweight", torch.uint8)
-    _check_device_tensor(wscales, "wscales", torch.float16)
-    N, K = qweight.shape[0], qweight.shape[1] * 2
-    with torch.cuda.device(qweight.device):
-        native = torch.empty((N, k_padded(K) // 2), dtype=torch.uint8, device=qweight.device)
-        plain = torch.empty((N,), dtype=torch.float16, device=qweight.device)
-        s = _stream(qweight.device)
-        _lib.check(lib.vdmq_weight_v1_to_native(qweight.data_ptr(), native.data_ptr(), N, K, s))
-        _lib.check(lib.vdmq_wscale_v1_to_plain(wscales.data_ptr(), plain.data_ptr(), N, K, s))
-    _NATIVE_CACHE[key] = (native, plain)
-    weakref.finalize(qweight, _NATIVE_CACHE.pop, key, None)
-    return native, plain
+    """(native int4 rows, plain fp16 channel scales) of a packed weight."""
+    pw = _prepared_weight(qweight, wscales)
+    return pw.operand(False), pw.wscale
 
 
 def clear_native_cache() -> None:
-    _NATIVE_CACHE.clear()
-    _BF6_CACHE.clear()
+    """Kept for callers of the earlier cache: prepared forms now live on the packed tensors and go with them."""
 
 
 # ------------------------------------------------- which matrix instructions run the GEMM
@@ -163,15 +315,15 @@ def matrix_path() -> str:
     return _MATRIX_PATH
 
 
-def _use_bf6(M: int, N: int, K: int, out_dtype: torch.dtype = torch.float16) -> bool:
-    if out_dtype != torch.float16 or _MATRIX_PATH == "int8" or M == 0:
+def _use_bf6(M: int, N: int, K: int, out_dtype: torch.dtype = torch.float16, path: Optional[str] = None) -> bool:
+    path = _MATRIX_PATH if path is None else path
+    if path == "bf6" and out_dtype != torch.float16:
+        raise _lib.VdmqError("the bf6 matrix path writes fp16 only; use matrix path 'int8' or 'auto' for a bf16 output")
+    if out_dtype != torch.float16 or path == "int8" or M == 0:
         return False
-    if _MATRIX_PATH == "bf6":
+    if path == "bf6":
         return True
     return bool(_load_ext().vdmq_bf6_pays(M, N, K))
-
-
-_BF6_CACHE: Dict[tuple, torch.Tensor] = {}
 
 
 def _to_bf6(native: torch.Tensor, rows: int, K: int) -> torch.Tensor:
@@ -180,18 +332,6 @@ def _to_bf6(native: torch.Tensor, rows: int, K: int) -> torch.Tensor:
     if rows:
         _lib.check(lib.vdmq_native_to_bf6(native.data_ptr(), rows, K, blocks.data_ptr(), _stream(native.device)))
     return blocks
-
-
-def _bf6_weights(native_w: torch.Tensor, K: int) -> torch.Tensor:
-    """bf6 blocks of a native weight tensor, converted once and kept as long as the native tensor lives."""
-    key = (native_w.data_ptr(), tuple(native_w.shape), native_w.device.index, K)
-    hit = _BF6_CACHE.get(key)
-    if hit is None:
-        with torch.cuda.device(native_w.device):
-            hit = _to_bf6(native_w, native_w.shape[0], K)
-        _BF6_CACHE[key] = hit
-        weakref.finalize(native_w, _BF6_CACHE.pop, key, None)
-    return hit
 
 
 def _quantize_for_gemm(x_2d: torch.Tensor, clip_ratio: float, act_code: int, bf6: bool, ln_args: Optional[tuple] = None):
@@ -219,7 +359,7 @@ def _quantize_for_gemm(x_2d: torch.Tensor, clip_ratio: float, act_code: int, bf6
     return op, scales
 
 
-def _gemm_dispatch(operand: torch.Tensor, scales: torch.Tensor, bf6: bool, native_w: torch.Tensor, wscale: torch.Tensor,
+def _gemm_dispatch(operand: torch.Tensor, scales: torch.Tensor, bf6: bool, weight: PreparedWeight,
                    bias: Optional[torch.Tensor], out: torch.Tensor, K: int, gate: Optional[torch.Tensor] = None, rows_per_gate: int = 1,
                    residual: Optional[torch.Tensor] = None) -> None:
     """GEMM + epilogue on a quantized activation (bf6 blocks if ``bf6`` else native rows) into ``out``.
@@ -230,13 +370,13 @@ def _gemm_dispatch(operand: torch.Tensor, scales: torch.Tensor, bf6: bool, nativ
     bias_p = None if bias is None else bias.data_ptr()
     gate_p, ldg = (None, 0) if gate is None else (gate.data_ptr(), gate.stride(0))
     res_p, ldr = (None, 0) if residual is None else (residual.data_ptr(), residual.stride(0))
+    w, wscale = weight.operand(bf6), weight.wscale
     if bf6:
-        wblocks = _bf6_weights(native_w, K)
-        _lib.check(lib.vdmq_gemm_w4a4_bf6_ex(operand.data_ptr(), scales.data_ptr(), wblocks.data_ptr(), wscale.data_ptr(), bias_p, gate_p, ldg,
+        _lib.check(lib.vdmq_gemm_w4a4_bf6_ex(operand.data_ptr(), scales.data_ptr(), w.data_ptr(), wscale.data_ptr(), bias_p, gate_p, ldg,
                                              rows_per_gate, res_p, ldr, out.data_ptr(), M, N, K, out.stride(0), s))
         return
     code = _lib.VDMQ_OUT_F16 if out.dtype == torch.float16 else _lib.VDMQ_OUT_BF16
-    _lib.check(lib.vdmq_gemm_w4a4_ex(operand.data_ptr(), scales.data_ptr(), native_w.data_ptr(), wscale.data_ptr(), bias_p, gate_p, ldg,
+    _lib.check(lib.vdmq_gemm_w4a4_ex(operand.data_ptr(), scales.data_ptr(), w.data_ptr(), wscale.data_ptr(), bias_p, gate_p, ldg,
                                      rows_per_gate, res_p, ldr, out.data_ptr(), code, M, N, K, out.stride(0), s))
 
 
@@ -267,10 +407,9 @@ def pack_weight_with_scale(weight: torch.Tensor, channel_scale: torch.Tensor):
         _lib.check(lib.vdmq_quantize_weight_native(weight_h.data_ptr(), scale_h.data_ptr(), native.data_ptr(), N, K, s))
         _lib.check(lib.vdmq_weight_native_to_v1(native.data_ptr(), qweight.data_ptr(), N, K, s))
         _lib.check(lib.vdmq_wscale_plain_to_v1(scale_h.data_ptr(), packed_scales.data_ptr(), N, K, s))
-    # the native form is already at hand: seed the cache so the first GEMM needs no relayout
-    key = (qweight.data_ptr(), packed_scales.data_ptr(), tuple(qweight.shape), dev.index, qweight._version, packed_scales._version)
-    _NATIVE_CACHE[key] = (native, scale_h.clone())
-    weakref.finalize(qweight, _NATIVE_CACHE.pop, key, None)
+    # the native form is already at hand: a first GEMM on the int8 path needs no relayout (an eager form: the bf6
+    # path, if that is what the calls take, drops it)
+    _prepared([(qweight, packed_scales)]).native = native
     return qweight, packed_scales, scale_h
 
 
@@ -299,13 +438,13 @@ def _act_code(act: Optional[str]) -> int:
     return _ACTIVATIONS[act]
 
 
-def _linear_2d(x_2d: torch.Tensor, native_w: torch.Tensor, wscale: torch.Tensor, bias: Optional[torch.Tensor], clip_ratio: float,
+def _linear_2d(x_2d: torch.Tensor, weight: PreparedWeight, bias: Optional[torch.Tensor], clip_ratio: float,
                out_dtype: torch.dtype = torch.float16, act: Optional[str] = None) -> torch.Tensor:
     _load_ext()  # raises when the library is missing
     M, K = x_2d.shape
-    N = native_w.shape[0]
+    N = weight.N
     dev = x_2d.device
-    _require(native_w.device == dev and wscale.device == dev, "weights and input must be on the same device")
+    _require(weight.device == dev, "weights and input must be on the same device")
     if bias is not None:
         _check_device_tensor(bias, "bias", torch.float16)
         _require(bias.dim() == 1, "bias must be [N]")
@@ -316,7 +455,7 @@ def _linear_2d(x_2d: torch.Tensor, native_w: torch.Tensor, wscale: torch.Tensor,
             return out
         bf6 = _use_bf6(M, N, K, out_dtype)
         operand, scales = _quantize_for_gemm(x_2d, clip_ratio, _act_code(act), bf6)
-        _gemm_dispatch(operand, scales, bf6, native_w, wscale, bias, out, K)
+        _gemm_dispatch(operand, scales, bf6, weight, bias, out, K)
     return out
 
 
@@ -335,12 +474,26 @@ def linear_vdm_w4a4(
     x_2d, orig_shape = _as_2d_half_contiguous(x)
     _check_linear_shapes(x_2d, qweight, wscales)
     _require(x_2d.is_cuda, "input must be a CUDA tensor")
-    native_w, wscale = _native_weights(qweight.contiguous(), wscales.contiguous())
-    b = bias_half if bias_half is not None else bias
-    if b is not None:
-        b = b.half().contiguous().view(-1)
-    out = _linear_2d(x_2d, native_w, wscale, b, clip_ratio)
-    return out.view(*orig_shape, -1)
+    return _linear_prepared(x_2d, _prepared_weight(qweight, wscales), bias_half if bias_half is not None else bias, clip_ratio).view(*orig_shape, -1)
+
+
+def linear_vdm_w4a4_prepared(x: torch.Tensor, weight: PreparedWeight, bias_half: Optional[torch.Tensor] = None,
+                             clip_ratio: float = 1.0) -> torch.Tensor:
+    """``linear_vdm_w4a4`` on a weight that is already in the kernels' form -- what the fused QKV / KV dispatch calls
+    with the concatenated weight of an attention module (no counterpart in the reference, which passes concatenated
+    v1 buffers to the same function)."""
+    _load_ext()
+    x_2d, orig_shape = _as_2d_half_contiguous(x)
+    if weight.K != x_2d.shape[1]:
+        raise ValueError("qweight shape must be [N, K/2]")
+    _require(x_2d.is_cuda, "input must be a CUDA tensor")
+    return _linear_prepared(x_2d, weight, bias_half, clip_ratio).view(*orig_shape, -1)
+
+
+def _linear_prepared(x_2d: torch.Tensor, weight: PreparedWeight, bias: Optional[torch.Tensor], clip_ratio: float) -> torch.Tensor:
+    if bias is not None:
+        bias = bias.half().contiguous().view(-1)
+    return _linear_2d(x_2d, weight, bias, clip_ratio)
 
 
 def quantize_activation_per_token(x: torch.Tensor, clip_ratio: float = 1.0):
@@ -412,7 +565,7 @@ def linear_prequantized(qact: torch.Tensor, ascales: torch.Tensor, qweight: torc
     _require(tuple(wscales.shape) == (N, K // WARP_K), "bad wscales shape")
     _require(M % BLOCK_M == 0, f"M must be a multiple of {BLOCK_M}")
     _require(N % BLOCK_N == 0, f"N must be a multiple of {BLOCK_N}")
-    native_w, wscale = _native_weights(qweight, wscales)
+    weight = _prepared_weight(qweight, wscales)
     dev = qact.device
     with torch.cuda.device(dev):
         s = _stream(dev)
@@ -423,7 +576,7 @@ def linear_prequantized(qact: torch.Tensor, ascales: torch.Tensor, qweight: torc
         scales = torch.empty((M,), dtype=torch.float16, device=dev)
         _lib.check(lib.vdmq_act_v1_to_native(qact.data_ptr(), ascales.data_ptr(), M, K, native.data_ptr(), scales.data_ptr(), s))
         bf6 = _use_bf6(M, N, K)
-        _gemm_dispatch(_to_bf6(native, M, K) if bf6 else native, scales, bf6, native_w, wscale, None, out, K)
+        _gemm_dispatch(_to_bf6(native, M, K) if bf6 else native, scales, bf6, weight, None, out, K)
     return out
 
 
@@ -466,27 +619,25 @@ def linear_vdm_w4a4_qkv(
     w_qkv_scale: Optional[torch.Tensor] = None,
     qkv_bias_half: Optional[torch.Tensor] = None,
 ):
-    """Fused QKV: one activation quantization and one GEMM against the
-    row-concatenated Wq|Wk|Wv; returns three views of one [..., 3N] tensor
-    (vdm_w4a4.py:259-298).  A row-concatenation of v1 buffers is itself a valid
-    v1 buffer because every 128-row block is self-contained."""
+    """Fused QKV: one activation quantization and one GEMM against the row-concatenated Wq|Wk|Wv; returns three
+    views of one [..., 3N] tensor.  Signature, argument handling (cached concatenation if given, zeros for missing
+    biases, ``split(n)``) and results are fixed by the reference's function of the same name (vdm_w4a4.py:259-298),
+    which this follows step by step.  Without the cached concatenation the reference concatenates the v1 buffers on
+    every call; here the three buffers are relaid once into one operand (every 128-row block of a v1 buffer is
+    self-contained, so the concatenation's operand is the parts' operands one after the other) and that is kept."""
     if w_qkv_packed is None or w_qkv_scale is None:
-        w_qkv_packed = torch.cat([q_weight_packed, k_weight_packed, v_weight_packed], dim=0).contiguous()
-        w_qkv_scale = torch.cat([q_weight_scale, k_weight_scale, v_weight_scale], dim=0).contiguous()
-    if qkv_bias_half is None:
-        n = q_weight_packed.shape[0]
-        has_bias = q_bias is not None or k_bias is not None or v_bias is not None
-        if has_bias:
-            device = w_qkv_packed.device
-
-            def zeros():
-                return torch.zeros(n, dtype=torch.float16, device=device)
-
-            qkv_bias_half = torch.cat([
-                q_bias.half().contiguous() if q_bias is not None else zeros(),
-                k_bias.half().contiguous() if k_bias is not None else zeros(),
-                v_bias.half().contiguous() if v_bias is not None else zeros(),
-            ], dim=0)
-    qkv = linear_vdm_w4a4(x, w_qkv_packed, w_qkv_scale, bias=None, clip_ratio=clip_ratio, bias_half=qkv_bias_half)
+        weight = _prepared([(q_weight_packed.contiguous(), q_weight_scale.contiguous()), (k_weight_packed.contiguous(), k_weight_scale.contiguous()),
+                            (v_weight_packed.contiguous(), v_weight_scale.contiguous())])
+    else:
+        weight = _prepared_weight(w_qkv_packed, w_qkv_scale)
     n = q_weight_packed.shape[0]
+    if qkv_bias_half is None and (q_bias is not None or k_bias is not None or v_bias is not None):
+        device = q_weight_packed.device
+        parts = [b.half().contiguous() if b is not None else torch.zeros(n, dtype=torch.float16, device=device) for b in (q_bias, k_bias, v_bias)]
+        qkv_bias_half = torch.cat(parts, dim=0)
+    _load_ext()
+    x_2d, orig_shape = _as_2d_half_contiguous(x)
+    _check_packed_weight(q_weight_packed, q_weight_scale, x_2d.shape[1])
+    _require(x_2d.is_cuda, "input must be a CUDA tensor")
+    qkv = _linear_prepared(x_2d, weight, qkv_bias_half, clip_ratio).view(*orig_shape, -1)
     return qkv.split(n, dim=-1)

@@ -115,9 +115,14 @@ class SharedContext:
         return q
 
 
+def _version_of(tensor: torch.Tensor):
+    # inference tensors keep no version counter (reading it raises) and cannot be written in place
+    return None if tensor.is_inference() else tensor._version
+
+
 def _weak_lookup(cache: dict, tensor: torch.Tensor):
     hit = cache.get(id(tensor))
-    if hit is not None and hit[0]() is tensor and hit[1] == tensor._version:
+    if hit is not None and hit[0]() is tensor and hit[1] == _version_of(tensor):
         return hit[2]
     return None
 
@@ -126,7 +131,7 @@ def _weak_store(cache: dict, tensor: torch.Tensor, value) -> None:
     import weakref
 
     key = id(tensor)
-    cache[key] = (weakref.ref(tensor, lambda _, d=cache, k=key: d.pop(k, None)), tensor._version, value)
+    cache[key] = (weakref.ref(tensor, lambda _, d=cache, k=key: d.pop(k, None)), _version_of(tensor), value)
 
 
 class Attention(nn.Module):
@@ -454,7 +459,7 @@ class KernelTimers:
 
 
 class time_w4a4_calls:
-    """Context manager: wraps ``linear_vdm_w4a4`` so that every W4A4 call is bracketed by events."""
+    """Context manager: wraps the W4A4 linear entry points so that every W4A4 call is bracketed by events."""
 
     def __init__(self, timers: KernelTimers):
         self.timers = timers
@@ -475,7 +480,8 @@ class time_w4a4_calls:
 
             return timed
 
-        self._saved = [(k, "linear_vdm_w4a4", k.linear_vdm_w4a4), (fused_ops, "linear_fused", fused_ops.linear_fused)]
+        self._saved = [(k, "linear_vdm_w4a4", k.linear_vdm_w4a4), (k, "linear_vdm_w4a4_prepared", k.linear_vdm_w4a4_prepared),
+                       (fused_ops, "linear_fused", fused_ops.linear_fused)]
         for mod, name, orig in self._saved:
             setattr(mod, name, wrap(orig))
         return self

@@ -235,6 +235,10 @@ int vdmq_linear_w4a4_bf6(const void *x, int64_t M, int64_t K, int64_t ldx, float
                          const void *bias, void *out, int64_t N, int64_t ldo, void *workspace, int64_t workspace_bytes,
                          vdmq_stream_t stream);
 int vdmq_native_to_bf6(const void *native, int64_t rows, int64_t K, void *blocks, vdmq_stream_t stream);
+/* A checkpoint's v1 weight buffer (u8 [N, K/2], weight_quantize_per_channel_kernel's order, vdm_w4a4_kernel.cu:518-551)
+ * straight to bf6 blocks: the one relayout a module needs when the bf6 path serves it, made once at load.
+ * Same bytes as vdmq_weight_v1_to_native followed by vdmq_native_to_bf6.  N % 128 == 0, K % 64 == 0. */
+int vdmq_weight_v1_to_bf6(const void *qweight_v1, void *wblocks, int64_t N, int64_t K, vdmq_stream_t stream);
 int vdmq_gemm_w4a4_bf6(const void *xblocks, const void *ascale, const void *wblocks, const void *wscale, const void *bias, void *out,
                        int64_t M, int64_t N, int64_t K, int64_t ldo, vdmq_stream_t stream);
 int vdmq_gemm_w4a4_bf6_ex(const void *xblocks, const void *ascale, const void *wblocks, const void *wscale, const void *bias,

@@ -30,6 +30,19 @@ def test_small_dit_structure_and_numerics():
     assert len(quant) == 10 * args.num_layers  # 300 at 30 layers, as the reference's build smoke test counts
     assert sum(isinstance(m, W.Attention) and m.use_fused_qkv_kernel for m in model.modules()) == 2 * args.num_layers
     assert all(m.use_vdm_kernel and m.weight is None for m in quant)
+    # the loader relaid every weight once: the fused q|k|v and k|v weights as one operand each, nothing for the
+    # projections they replace; every prepared weight holds exactly one form
+    prepared = []
+    for blk in model.blocks:
+        for attn, lead, fused in ((blk.attn1, "to_q", ("to_k", "to_v")), (blk.attn2, "to_k", ("to_v",))):
+            kept = getattr(attn, lead).vdm_weight_packed.__dict__["_vdmq_prepared"]
+            assert [len(p.rows) for p in kept] == [1 + len(fused)]
+            prepared += kept
+            assert all("_vdmq_prepared" not in getattr(attn, n).vdm_weight_packed.__dict__ or not getattr(attn, n).vdm_weight_packed.__dict__["_vdmq_prepared"] for n in fused)
+        for lay in (blk.attn1.to_out[0], blk.attn2.to_q, blk.attn2.to_out[0], blk.ffn.up, blk.ffn.down):
+            prepared += lay.vdm_weight_packed.__dict__["_vdmq_prepared"]
+    assert len(prepared) == 7 * args.num_layers
+    assert all((p.native is None) != (p.bf6 is None) for p in prepared)
 
     g = torch.Generator(device=dev).manual_seed(0)
     latent = torch.randn((1, 16, 3, 8, 12), generator=g, device=dev).half()  # 3*4*6 = 72 tokens
@@ -42,6 +55,10 @@ def test_small_dit_structure_and_numerics():
     timers.collect()
     assert y.shape == latent.shape and torch.isfinite(y).all()
     assert timers.counts() == {"w4a4": 7 * args.num_layers, "attention": 2 * args.num_layers}
+    # after a forward every weight still holds one form only -- the one its calls take (72 and 512 rows: native rows)
+    weights = sum(p.N * p.K for p in prepared)
+    assert all(p.native is not None and p.bf6 is None for p in prepared)
+    assert sum(p.extra_bytes() for p in prepared) <= 0.75 * weights
 
     # reference: the same forward with every W4A4 call replaced by fp32 arithmetic on the
     # dequantized operands (per-token int4 activations with clip 0.95, unpacked int4 weights)
@@ -63,13 +80,17 @@ def test_small_dit_structure_and_numerics():
             yy = yy + b.half()
         return yy.view(*x.shape[:-1], N)
 
-    orig = v.linear_vdm_w4a4
-    v.linear_vdm_w4a4 = ref_linear
+    def ref_prepared(x, weight, bias_half=None, clip_ratio=1.0):  # the fused QKV / KV calls: a concatenated weight
+        parts = weight.sources()
+        return ref_linear(x, torch.cat([q for q, _ in parts]), torch.cat([s for _, s in parts]), None, clip_ratio, bias_half)
+
+    orig = v.linear_vdm_w4a4, v.linear_vdm_w4a4_prepared
+    v.linear_vdm_w4a4, v.linear_vdm_w4a4_prepared = ref_linear, ref_prepared
     try:
         with torch.no_grad():
             y_ref = model(latent, t, ctx)
     finally:
-        v.linear_vdm_w4a4 = orig
+        v.linear_vdm_w4a4, v.linear_vdm_w4a4_prepared = orig
     err = (y.float() - y_ref.float()).abs().max().item()
     assert err <= 2e-2 * y_ref.float().abs().max().item() + 1e-3, err
 
@@ -140,6 +161,38 @@ def test_context_reuse_changes_nothing_but_the_work():
     assert all(torch.equal(o, p) for o, p in zip(outs, plain)) and torch.equal(outs[3], plain[0])
     L = args.num_layers
     assert counts == [7 * L, 7 * L, 6 * L, 7 * L]  # third forward: no K/V projection; a cloned context is a new tensor
+
+
+def test_first_call_after_load_can_be_captured():
+    """The loader has relaid the weights, so the first forward of a loaded layer may already run under HIP graph
+    capture: nothing is relaid inside the capture (the prepared form is the object the loader made), and replays with
+    new inputs, eager work and synchronisations between them, equal the eager results."""
+    from dsaquant_amd import wan_harness as W
+
+    dev = "cuda:0"
+    args = replace(W.WAN21_1P3B, num_layers=1, num_heads=2, ffn_dim=512, text_dim=128)
+    model = W.build_quantized(args, dev, seed=7)
+    layer, attn = model.blocks[0].ffn.up, model.blocks[0].attn1
+    made = layer.vdm_weight_packed.__dict__["_vdmq_prepared"][0]
+    form = made.native
+    assert form is not None
+    g = torch.Generator(device=dev).manual_seed(1)
+    x = torch.randn((1, 300, args.dim), generator=g, device=dev).half()
+    graph = torch.cuda.CUDAGraph()
+    print("capture of a loaded layer's first call", flush=True)
+    with torch.no_grad(), torch.cuda.graph(graph):
+        y = layer(x)
+        q, k, v = W.get_qkv_projections(attn, x, None)
+    assert layer.vdm_weight_packed.__dict__["_vdmq_prepared"] == [made] and made.native is form and made.bf6 is None
+    for it in range(3):
+        x.copy_(torch.randn((1, 300, args.dim), generator=g, device=dev).half() * (1 + it))
+        graph.replay()
+        torch.cuda.synchronize()
+        got = [t.clone() for t in (y, q, k, v)]
+        with torch.no_grad():
+            want = [layer(x), *W.get_qkv_projections(attn, x, None)]
+        torch.cuda.synchronize()
+        assert all(torch.equal(a, b) for a, b in zip(got, want)), it
 
 
 def test_patchify_roundtrip():

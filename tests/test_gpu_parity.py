@@ -188,12 +188,21 @@ def test_bf16_output_within_tolerance():
     v = vk()
     M, K, N = 300, 512, 256
     x, qw, ws, bias = O.synth_linear(M, K, N, seed=6)
-    native_w, wscale = v._native_weights(t16(O.np_pack_wgt_v1(qw)), t16(O.np_pack_wscales_v1(ws, K)))
-    y = v._linear_2d(t16(x), native_w, wscale, t16(bias), 1.0, out_dtype=torch.bfloat16)
+    qv1, sv1 = t16(O.np_pack_wgt_v1(qw)), t16(O.np_pack_wscales_v1(ws, K))  # (a prepared weight lives with its packed tensors)
+    weight = v._prepared_weight(qv1, sv1)
+    y = v._linear_2d(t16(x), weight, t16(bias), 1.0, out_dtype=torch.bfloat16)
     want, _, as_h, acc = O.np_linear(x, qw, ws, bias, 1.0)
     exact = acc.astype(np.float64) * as_h.astype(np.float64)[:, None] * ws.astype(np.float64)[None, :] + bias.astype(np.float64)
     err = np.abs(y.float().cpu().numpy().astype(np.float64) - exact)
     assert err.max() <= 2.0 ** -8 * np.abs(exact).max()
+    # the bf6 matrix path writes fp16 only: asked for by name with a bf16 output it says so instead of switching paths
+    old = v.matrix_path()
+    v.set_matrix_path("bf6")
+    try:
+        with pytest.raises(RuntimeError, match="fp16 only"):
+            v._linear_2d(t16(x), weight, t16(bias), 1.0, out_dtype=torch.bfloat16)
+    finally:
+        v.set_matrix_path(old)
 
 
 def test_shape_and_dtype_errors():
@@ -276,6 +285,66 @@ def test_quantize_activation_per_token_v1_and_prequantized():
     got = y.cpu().numpy()
     assert np.array_equal(got[:M].view(np.uint16), want.view(np.uint16))
     assert not got[M:].any()  # padded rows: zero activations, scale 1
+
+
+def test_prepared_weights_one_form_per_layer_made_from_the_v1_buffers():
+    """A packed weight is relaid straight from its v1 buffers into the form its calls use and only that form is kept:
+    bf6 blocks made ahead are dropped when the calls turn out to take the int8 path (and the other way round), a
+    non-contiguous qweight is not relaid per call, tensors made under inference_mode (no version counter) work, an
+    in-place write to the packed buffer is noticed, and the direct v1 -> bf6 relayout writes the bytes of the two-step one."""
+    from dsaquant_amd import _lib
+
+    v = vk()
+    lib = _lib.load()
+    M, K, N = 300, 448, 384
+    x, qw, ws, bias = O.synth_linear(M, K, N, seed=12)
+    want = O.np_linear(x, qw, ws, bias, 1.0)[0]
+    qv1, sv1 = t16(O.np_pack_wgt_v1(qw)), t16(O.np_pack_wscales_v1(ws, K))
+    pw = v.prepare_weight(qv1, sv1, path="bf6")  # made ahead for calls on the bf6 path
+    assert pw.bf6 is not None and pw.native is None
+    native = torch.empty((N, v.k_padded(K) // 2), dtype=torch.uint8, device=DEV)
+    two_step = torch.empty_like(pw.bf6)
+    _lib.check(lib.vdmq_weight_v1_to_native(qv1.data_ptr(), native.data_ptr(), N, K, None))
+    _lib.check(lib.vdmq_native_to_bf6(native.data_ptr(), N, K, two_step.data_ptr(), None))
+    assert torch.equal(pw.bf6, two_step)
+    y = v.linear_vdm_w4a4(t16(x), qv1, sv1, t16(bias))  # 300 rows: the int8 path under "auto"
+    assert np.array_equal(y.cpu().numpy().view(np.uint16), want.view(np.uint16))
+    assert v._prepared_weight(qv1, sv1) is pw and pw.native is not None and pw.bf6 is None
+    assert pw.extra_bytes() == N * v.k_padded(K) // 2 + 2 * N
+    old = v.matrix_path()
+    v.set_matrix_path("bf6")
+    try:
+        y = v.linear_vdm_w4a4(t16(x), qv1, sv1, t16(bias))
+        assert np.array_equal(y.cpu().numpy().view(np.uint16), want.view(np.uint16))
+        assert pw.native is not None and pw.bf6 is not None  # both have been used: both stay
+    finally:
+        v.set_matrix_path(old)
+    # non-contiguous packed buffers (a strided view): one contiguous copy and one relayout, kept with the view
+    wide = torch.zeros((N, K), dtype=torch.uint8, device=DEV)
+    wide[:, : K // 2] = qv1
+    view = wide[:, : K // 2]
+    assert not view.is_contiguous()
+    y1 = v.linear_vdm_w4a4(t16(x), view, sv1, t16(bias))
+    first = v._prepared_weight(view, sv1)
+    y2 = v.linear_vdm_w4a4(t16(x), view, sv1, t16(bias))
+    assert v._prepared_weight(view, sv1) is first and torch.equal(y1, y2)
+    assert np.array_equal(y1.cpu().numpy().view(np.uint16), want.view(np.uint16))
+    # an in-place write is a new weight
+    qw2 = qw.copy()
+    qw2[0] = -qw2[0].clip(-7, 7)
+    qv1.copy_(t16(O.np_pack_wgt_v1(qw2)))
+    y = v.linear_vdm_w4a4(t16(x), qv1, sv1, t16(bias))
+    assert v._prepared_weight(qv1, sv1) is not pw
+    assert np.array_equal(y.cpu().numpy().view(np.uint16), O.np_linear(x, qw2, ws, bias, 1.0)[0].view(np.uint16))
+    # tensors created under inference_mode keep no version counter
+    with torch.inference_mode():
+        qi, si = t16(O.np_pack_wgt_v1(qw)), t16(O.np_pack_wscales_v1(ws, K))
+        assert qi.is_inference()
+        for _ in range(2):
+            y = v.linear_vdm_w4a4(t16(x), qi, si, t16(bias))
+        q3, k3, v3 = v.linear_vdm_w4a4_qkv(t16(x), qi, si, qi, si, qi, si, t16(bias), None, None)
+        assert torch.equal(q3, y) and torch.equal(k3, v3)
+    assert np.array_equal(y.cpu().numpy().view(np.uint16), want.view(np.uint16))
 
 
 # --------------------------------------------------------------- fused QKV

@@ -444,6 +444,26 @@ def test_loader_errors_read_as_the_reference_loader_errors():
         assert [type(info.value).__name__, str(info.value)] == want["errors"][name], name
 
 
+def test_cache_keys_work_for_tensors_made_under_inference_mode():
+    """Inference tensors keep no version counter (reading ``_version`` raises); the caches that watch for in-place
+    writes must not read it on them."""
+    from dsaquant_amd import wan_harness
+    from dsaquant_amd.kernels import vdm_w4a4 as v
+
+    with torch.inference_mode():
+        t = torch.zeros(4)
+    with pytest.raises(RuntimeError):
+        t._version
+    assert v._version_of(t) is None and wan_harness._version_of(t) is None
+    cache = {}
+    wan_harness._weak_store(cache, t, "kept")
+    assert wan_harness._weak_lookup(cache, t) == "kept"
+    u = torch.zeros(4)
+    wan_harness._weak_store(cache, u, "kept too")
+    u.add_(1)  # an ordinary tensor written in place is a miss
+    assert wan_harness._weak_lookup(cache, u) is None
+
+
 def test_library_says_where_the_fp6_path_pays():
     """vdmq_bf6_pays is a pure function of the sizes (no GPU work): the BASELINE shapes and the measured crossovers."""
     from dsaquant_amd import _lib
