@@ -22,6 +22,16 @@ timed region.  Prints ONE JSON line.
              launch duration, against the 8 TB/s HBM3E peak
   cpu_baseline  the torch QuantLinear floating-point path (oracle/quantlinear_torch.py,
              a restatement of the reference's CPU-runnable path) on config 0
+
+Beside the headline fields the line carries, all measured in the same run:
+  int8_path     the same workload with the GEMM forced onto the int8 matrix instructions (gemm_w4a4_kernel), with its
+                own roofline object against the 5.0 POP/s INT8 peak
+  workloads     whole-step TOPS of the other block workloads (Wan-2.1 1.3B at 480p, Wan-2.2 5B) on the path the
+                library picks, with the per-linear figures
+  mfma_ceiling  what the two MFMA instructions sustain in a loop with nothing else (vdmq_mfma_probe) on all-zero
+                operands, on int4-valued operands and on operands with the workload's statistics: the published peaks
+                assume the top clock, which the part does not hold under matrix load
+--ubench prints only that probe (longer runs), for counter collection with rocprofv3.
 """
 from __future__ import annotations
 
@@ -38,18 +48,20 @@ sys.path.insert(0, str(ROOT))
 
 INT8_PEAK_TOPS = 5000.0  # MI355X dense INT8 MFMA, published
 FP6_PEAK_TOPS = 10100.0  # MI355X dense FP6 MFMA, published
-# HBM bytes per launch of the dominant kernels on the default workload, from rocprofv3 --pmc FETCH_SIZE and
-# WRITE_SIZE runs of this program (mean over the four launches of a step; the summary with the scaling by
-# the copy kernel's readings is profiles/gemm_w4a4_kernel+quantize_rows_kernel.wan14b_720p_block.md for the int8
-# path and profiles/gemm_bf6_persistent_kernel+quantize_rows_kernel.wan14b_720p_block.md for the bf6 path)
-# gemm: (FETCH_SIZE 1377438 KiB x 2.0 + WRITE_SIZE 1455495 KiB x 1.0) x 1024; the reads are requests leaving L2
-# (Infinity Cache or HBM), 9x the operand bytes because every XCD fetches most of its super-tile's slabs once.
-# quant: (FETCH_SIZE 538736 KiB x 2.0 + WRITE_SIZE 269920 KiB x 1.0) x 1024 = 1.0005 x the algorithmic bytes.
-# bf6 path, same method: gemm (FETCH_SIZE 2692746 KiB x 2.0 + WRITE_SIZE 1456313 KiB x 1.0) x 1024 (6-bit operands and
-# little slab re-use between super-tiles: 12x the operand bytes); quant (538745 x 2.0 + 404284 x 1.0) x 1024 = 1.0002 x
-# the algorithmic bytes.
-MEASURED_TRAFFIC = {("wan14b_720p_block", "int8"): {"gemm": 4311418572, "quant": 1379729408},
-                    ("wan14b_720p_block", "bf6"): {"gemm": 7006008524, "quant": 1517336576}}
+# Bytes that left the XCDs' L2 caches per launch of the dominant kernels on the default workload (mean over the four
+# launches of a step).  NOT measured by this program: hardware counters need the profiler.  The figures are copied
+# from the rocprofv3 --pmc FETCH_SIZE / WRITE_SIZE summaries named below (each reading scaled by what the same counter
+# shows for the library's plain copy kernel of known size in the same run) and belong to the library build those
+# files name; the line says so ("traffic_source").  Requests that leave an L2 are served by the 256 MB Infinity Cache
+# or by HBM -- no counter available here separates the two -- so for the GEMM, whose operands fit that cache, this is
+# an upper bound of its HBM bytes; for the quantizer (a stream far larger than the cache) it is the HBM traffic.
+TRAFFIC_FROM_PROFILES = {
+    ("wan14b_720p_block", "int8"): {"gemm": 4311418572, "quant": 1379729408,
+                                    "source": "profiles/gemm_w4a4_kernel+quantize_rows_kernel.wan14b_720p_block.md"},
+    ("wan14b_720p_block", "bf6"): {"gemm": 7006008524, "quant": 1517336576,
+                                   "source": "profiles/gemm_bf6_persistent_kernel+quantize_rows_kernel.wan14b_720p_block.md"},
+}
+TRAFFIC_UNIT = "bytes leaving L2 per launch (Infinity Cache or HBM), mean of the step's four launches; from the profile named in traffic_source, not from this run"
 HBM_PEAK_GBS = 8000.0    # MI355X HBM3E, published
 
 # (name, K, N) at M tokens
@@ -114,6 +126,187 @@ def cpu_baseline(torch, budget_s=16.0):
                   + ", ".join(f"{k}={v:.4f} ({reps[k]} reps)" for k, v in out.items()),
     }
 
+class Workload:
+    """The linears of one block with inputs, packed weights and outputs resident on the device."""
+
+    def __init__(self, torch, lib, v, name, path, dev):
+        from dsaquant_amd import _lib
+
+        self.torch, self.lib, self._lib, self.name, self.dev = torch, lib, _lib, name, dev
+        wl = WORKLOADS[name]
+        self.M = M = wl["M"]
+        self.stream = torch.cuda.current_stream(dev)
+        s = self.stream.cuda_stream
+        self.layers = []
+        for i, (lname, K, N) in enumerate(wl["linears"]):
+            x, wq, ws, bias = synth_inputs(torch, M, K, N, seed=i, dev=dev)
+            assert v.k_padded(K) == K
+            bf6 = v._use_bf6(M, N, K, path=path)
+            if bf6:  # operands of the bf6 path: 6-bit blocks (weights converted once, as a loaded module holds them)
+                wblocks = torch.empty(int(lib.vdmq_bf6_bytes(N, K)), dtype=torch.uint8, device=dev)
+                _lib.check(lib.vdmq_native_to_bf6(wq.data_ptr(), N, K, wblocks.data_ptr(), s))
+                wq = wblocks
+                qact = torch.empty(int(lib.vdmq_bf6_bytes(M, K)), dtype=torch.uint8, device=dev)
+            else:
+                qact = torch.empty((M, K // 2), dtype=torch.uint8, device=dev)
+            self.layers.append(dict(name=lname, K=K, N=N, x=x, wq=wq, ws=ws, bias=bias, bf6=bf6, qact=qact,
+                                    scale=torch.empty((M,), dtype=torch.float16, device=dev),
+                                    out=torch.empty((M, N), dtype=torch.float16, device=dev)))
+        torch.cuda.synchronize()
+
+    def step(self, events=None):
+        lib, _lib, M, s = self.lib, self._lib, self.M, self.stream.cuda_stream
+        for li, L in enumerate(self.layers):
+            if events is not None:
+                events[li][0].record(self.stream)
+            if L["bf6"]:
+                _lib.check(lib.vdmq_quantize_act_bf6(L["x"].data_ptr(), M, L["K"], L["K"], 1.0, 0, L["qact"].data_ptr(), L["scale"].data_ptr(), s))
+            else:
+                _lib.check(lib.vdmq_quantize_act(L["x"].data_ptr(), M, L["K"], L["K"], 1.0, L["qact"].data_ptr(), L["scale"].data_ptr(), s))
+            if events is not None:
+                events[li][1].record(self.stream)
+            if L["bf6"]:
+                _lib.check(lib.vdmq_gemm_w4a4_bf6(L["qact"].data_ptr(), L["scale"].data_ptr(), L["wq"].data_ptr(), L["ws"].data_ptr(),
+                                                  L["bias"].data_ptr(), L["out"].data_ptr(), M, L["N"], L["K"], L["N"], s))
+            else:
+                _lib.check(lib.vdmq_gemm_w4a4(L["qact"].data_ptr(), L["scale"].data_ptr(), L["wq"].data_ptr(), L["ws"].data_ptr(),
+                                              L["bias"].data_ptr(), L["out"].data_ptr(), _lib.VDMQ_OUT_F16, M, L["N"], L["K"], L["N"], s))
+            if events is not None:
+                events[li][2].record(self.stream)
+            if events is not None and "kernel" not in L:
+                L["kernel"] = {1: "gemm_w4a4_kernel", 2: "gemm_bf6_kernel", 3: "gemm_bf6_persistent_kernel"}[_lib.last_gemm_launch().kernel]
+
+    def measure(self, steps, warmup):
+        """W untimed steps, then exactly K timed steps between synchronisations; per-launch times from HIP events
+        recorded on the stream the kernels run on."""
+        torch, M = self.torch, self.M
+        for _ in range(warmup):
+            self.step()
+        torch.cuda.synchronize()
+        evs = [[[torch.cuda.Event(enable_timing=True) for _ in range(3)] for _ in self.layers] for _ in range(steps)]
+        torch.cuda.synchronize()
+        t0 = time.perf_counter()
+        for k in range(steps):
+            self.step(evs[k])
+        torch.cuda.synchronize()
+        wall = time.perf_counter() - t0
+        ms_per_step = wall * 1e3 / steps
+        total_ops = sum(2.0 * M * L["N"] * L["K"] for L in self.layers)
+        per_layer, gemm_ms, quant_ms = {}, 0.0, 0.0
+        for li, L in enumerate(self.layers):
+            q_ms = statistics.mean(evs[k][li][0].elapsed_time(evs[k][li][1]) for k in range(steps))
+            g_ms = statistics.mean(evs[k][li][1].elapsed_time(evs[k][li][2]) for k in range(steps))
+            gemm_ms += g_ms
+            quant_ms += q_ms
+            per_layer[L["name"]] = {
+                "K": L["K"], "N": L["N"], "gemm_ms": round(g_ms, 4), "gemm_tops": round(2.0 * M * L["N"] * L["K"] / g_ms / 1e9, 1),
+                "quant_ms": round(q_ms, 4), "quant_gbs": round(quant_bytes(M, L["K"], L["bf6"]) / q_ms / 1e6, 1),
+                "quant_gbs_int4_bytes": round(quant_bytes(M, L["K"]) / q_ms / 1e6, 1),
+                "matrix_path": "bf6" if L["bf6"] else "int8", "kernel": L["kernel"],
+            }
+        n = len(self.layers)
+        paths = sorted({"bf6" if L["bf6"] else "int8" for L in self.layers})
+        kernels = sorted({L["kernel"] for L in self.layers})
+        path = paths[0] if len(paths) == 1 else "mixed"
+        # a step that mixes both kinds of launches is priced against the higher peak
+        peak = INT8_PEAK_TOPS if path == "int8" else FP6_PEAK_TOPS
+        gemm_tops = total_ops / gemm_ms / 1e9
+        block_bytes = sum(quant_bytes(M, L["K"], L["bf6"]) for L in self.layers)
+        int4_bytes = sum(quant_bytes(M, L["K"]) for L in self.layers)
+        traffic = TRAFFIC_FROM_PROFILES.get((self.name, path), {})
+        return {
+            "path": path, "ms_per_step": ms_per_step, "step_tops": total_ops / (ms_per_step * 1e-3) / 1e12, "total_ops": total_ops,
+            "roofline": {"bound": "mfma", "achieved": round(gemm_tops, 1), "peak": peak, "unit": "TOP/s", "frac": round(gemm_tops / peak, 4),
+                         "frac_of_int8_peak": round(gemm_tops / INT8_PEAK_TOPS, 4), "traffic": traffic.get("gemm"),
+                         "traffic_unit": TRAFFIC_UNIT, "traffic_source": traffic.get("source"), "kernel": " + ".join(kernels),
+                         "algorithmic_ops_per_launch": total_ops / n, "avg_launch_ms": round(gemm_ms / n, 4)},
+            "quantizer": {"bound": "hbm", "achieved": round(block_bytes / quant_ms / 1e6, 1), "peak": HBM_PEAK_GBS, "unit": "GB/s",
+                          "frac": round(block_bytes / quant_ms / 1e6 / HBM_PEAK_GBS, 4),
+                          "bytes_counted": "what the kernel moves: 2K in, 3K/4 (bf6 blocks) or K/2 (int4 rows) out, 2 per scale",
+                          "achieved_int4_bytes": round(int4_bytes / quant_ms / 1e6, 1),
+                          "frac_int4_bytes": round(int4_bytes / quant_ms / 1e6 / HBM_PEAK_GBS, 4),
+                          "int4_bytes_counted": "2MK + MK/2 + 2M per launch whatever the output form: the path's algorithmic bytes",
+                          "traffic": traffic.get("quant"), "traffic_unit": TRAFFIC_UNIT, "traffic_source": traffic.get("source"),
+                          "kernel": "quantize_rows_kernel", "algorithmic_bytes_per_launch": block_bytes / n,
+                          "avg_launch_ms": round(quant_ms / n, 4)},
+            "per_linear": per_layer,
+        }
+
+
+BF6_CODES = [0x00, 0x0C, 0x10, 0x12, 0x14, 0x15, 0x16, 0x17, 0x18]  # E3M2 codes of |q| = 0..8; the sign is bit 5
+
+
+def probe_operands(np, kind, data, rng):
+    """Register images for vdmq_mfma_probe: [8 waves][12 operands][64 lanes] x 32 bytes.  ``data``: "zeros"; "int4"
+    = both sides uniform in [-8, 7]; "workload" = weight side uniform in [-7, 7], token side with the statistics of
+    the benchmark activations (N(0,1) with 1 % of the channels x 20, per-token scale absmax / 7: mostly 0 and +-1);
+    "bytes" (int8 only) = uniformly random bytes."""
+    per = 32 if kind == "bf6" else 16  # int4 values one lane holds per operand: a 192-bit string of codes / 16 bytes
+    shape = (8, 12, 64, per)
+    if data == "zeros":
+        q = np.zeros(shape, np.int64)
+    elif data == "int4":
+        q = rng.integers(-8, 8, shape)
+    elif data == "workload":
+        q = rng.integers(-7, 8, shape)
+        K = 5120
+        x = rng.standard_normal((8 * 8 * 64, K)).astype(np.float32)
+        x[:, rng.permutation(K)[: -(-K // 100)]] *= 20.0
+        scale = np.abs(x).max(axis=1, keepdims=True) / 7.0
+        qx = np.clip(np.rint(x / scale), -8, 7).astype(np.int64)  # one token row per lane; the lane takes `per` consecutive k
+        start = rng.integers(0, K - per, 8 * 8 * 64)
+        tok = np.stack([qx[i, st:st + per] for i, st in enumerate(start)]).reshape(8, 8, 64, per)
+        for side, o in enumerate((2, 3, 4, 5, 8, 9, 10, 11)):  # the token-side operands
+            q[:, o] = tok[:, side]
+    elif data == "bytes" and kind == "int8":
+        q = None
+    else:
+        raise ValueError(data)
+    img = np.zeros((8, 12, 64, 32), np.uint8)
+    if kind == "int8":
+        img[..., :16] = rng.integers(0, 256, shape, dtype=np.uint8) if q is None else ((q & 0xF) << 4).astype(np.uint8)  # bytes 16 * q
+    else:
+        codes = np.asarray(BF6_CODES, np.uint8)[np.abs(q)] | np.where(q < 0, 0x20, 0).astype(np.uint8)
+        bits = (codes[..., None] >> np.arange(6, dtype=np.uint8)) & 1  # code e at bits [6e, 6e + 6)
+        img[..., :24] = np.packbits(bits.reshape(*shape[:3], 192), axis=-1, bitorder="little")
+    return img
+
+
+def mfma_ceiling(torch, lib, dev, ms_target=30.0, repeats=3):
+    """TOP/s of the MFMA-only loop per instruction and operand data, HIP events around each launch."""
+    import ctypes
+
+    import numpy as np
+
+    from dsaquant_amd import _lib
+
+    stream = torch.cuda.current_stream(dev)
+    cus = torch.cuda.get_device_properties(dev).multi_processor_count
+    out = torch.empty(cus * 512, dtype=torch.int32, device=dev)
+    rng = np.random.default_rng(0)
+    res = {"workgroups": cus, "waves_per_workgroup": 8, "mfma_per_wave_and_iteration": 16}
+    for kind, code, datas in (("int8", 0, ("zeros", "int4", "workload", "bytes")), ("bf6", 1, ("zeros", "int4", "workload"))):
+        res[kind] = {}
+        for data in datas:
+            ops = ctypes.c_double()
+            operands = torch.from_numpy(probe_operands(np, kind, data, rng)).to(dev)
+            assert operands.numel() == lib.vdmq_mfma_probe_operand_bytes()
+
+            def launch(iters):
+                a, b = torch.cuda.Event(enable_timing=True), torch.cuda.Event(enable_timing=True)
+                a.record(stream)
+                _lib.check(lib.vdmq_mfma_probe(code, operands.data_ptr(), iters, cus, out.data_ptr(), ctypes.byref(ops), stream.cuda_stream))
+                b.record(stream)
+                torch.cuda.synchronize()
+                return a.elapsed_time(b)
+
+            iters = 2000
+            ms = launch(iters)
+            iters = max(2000, int(iters * ms_target / max(ms, 1e-3)))
+            times = [launch(iters) for _ in range(repeats)]
+            res[kind][data] = {"tops": round(ops.value / (statistics.median(times) * 1e-3) / 1e12, 1), "ms": round(statistics.median(times), 3)}
+    return res
+
 
 def main():
     ap = argparse.ArgumentParser()
@@ -124,6 +317,8 @@ def main():
     ap.add_argument("--matrix-path", default="auto", choices=["auto", "int8", "bf6"],
                     help="matrix instructions of the GEMM: auto = what the library picks for the shape")
     ap.add_argument("--no-cpu-baseline", action="store_true")
+    ap.add_argument("--no-extras", action="store_true", help="skip the int8-path run, the other workloads and the MFMA probe")
+    ap.add_argument("--ubench", action="store_true", help="only the MFMA-only probe, 200 ms per case (for counter collection)")
     ap.add_argument("--calibrate-copy", action="store_true",
                     help="also run the library's plain 1 GiB copy kernel three times first, so that a rocprofv3 --pmc FETCH_SIZE / WRITE_SIZE "
                          "run holds a copy kernel of known size to scale the counters by")
@@ -141,8 +336,11 @@ def main():
     lib = _lib.load()
     dev = torch.device("cuda:0")
     torch.cuda.set_device(dev)
-    wl = WORKLOADS[args.workload]
-    M = wl["M"]
+
+    if args.ubench:
+        print(json.dumps({"metric": "MFMA-only loop, TOP/s", "unit": "TOP/s", "peaks": {"int8": INT8_PEAK_TOPS, "bf6": FP6_PEAK_TOPS},
+                          "mfma_ceiling": mfma_ceiling(torch, lib, dev, ms_target=200.0, repeats=3)}))
+        return
 
     if args.calibrate_copy:
         # the library's plain 128-bit copy kernel: reads 1 GiB, writes 1 GiB
@@ -153,104 +351,48 @@ def main():
         torch.cuda.synchronize()
         del src, dst
 
-    v.set_matrix_path(args.matrix_path)
-    stream = torch.cuda.current_stream(dev)
-    s = stream.cuda_stream
-    layers = []
-    for i, (name, K, N) in enumerate(wl["linears"]):
-        x, wq, ws, bias = synth_inputs(torch, M, K, N, seed=i, dev=dev)
-        Kp = v.k_padded(K)
-        assert Kp == K
-        bf6 = v._use_bf6(M, N, K)
-        if bf6:  # operands of the bf6 path: 6-bit blocks (weights converted once, like a module's cache does)
-            wblocks = torch.empty(int(lib.vdmq_bf6_bytes(N, K)), dtype=torch.uint8, device=dev)
-            _lib.check(lib.vdmq_native_to_bf6(wq.data_ptr(), N, K, wblocks.data_ptr(), s))
-            wq = wblocks
-            qact = torch.empty(int(lib.vdmq_bf6_bytes(M, K)), dtype=torch.uint8, device=dev)
-        else:
-            qact = torch.empty((M, Kp // 2), dtype=torch.uint8, device=dev)
-        layers.append(dict(name=name, K=K, N=N, x=x, wq=wq, ws=ws, bias=bias, bf6=bf6, qact=qact,
-                           scale=torch.empty((M,), dtype=torch.float16, device=dev),
-                           out=torch.empty((M, N), dtype=torch.float16, device=dev)))
-    torch.cuda.synchronize()
-
-    def run_step(events=None):
-        for li, L in enumerate(layers):
-            if events is not None:
-                events[li][0].record(stream)
-            if L["bf6"]:
-                _lib.check(lib.vdmq_quantize_act_bf6(L["x"].data_ptr(), M, L["K"], L["K"], 1.0, 0, L["qact"].data_ptr(), L["scale"].data_ptr(), s))
-            else:
-                _lib.check(lib.vdmq_quantize_act(L["x"].data_ptr(), M, L["K"], L["K"], 1.0, L["qact"].data_ptr(), L["scale"].data_ptr(), s))
-            if events is not None:
-                events[li][1].record(stream)
-            if L["bf6"]:
-                _lib.check(lib.vdmq_gemm_w4a4_bf6(L["qact"].data_ptr(), L["scale"].data_ptr(), L["wq"].data_ptr(), L["ws"].data_ptr(),
-                                                  L["bias"].data_ptr(), L["out"].data_ptr(), M, L["N"], L["K"], L["N"], s))
-            else:
-                _lib.check(lib.vdmq_gemm_w4a4(L["qact"].data_ptr(), L["scale"].data_ptr(), L["wq"].data_ptr(), L["ws"].data_ptr(),
-                                              L["bias"].data_ptr(), L["out"].data_ptr(), _lib.VDMQ_OUT_F16, M, L["N"], L["K"], L["N"], s))
-            if events is not None:
-                events[li][2].record(stream)
-
-    for _ in range(args.warmup):
-        run_step()
-    torch.cuda.synchronize()
-
-    evs = [[[torch.cuda.Event(enable_timing=True) for _ in range(3)] for _ in layers] for _ in range(args.steps)]
-    torch.cuda.synchronize()
-    t0 = time.perf_counter()
-    for k in range(args.steps):
-        run_step(evs[k])
-    torch.cuda.synchronize()
-    wall = time.perf_counter() - t0
-
-    ms_per_step = wall * 1e3 / args.steps
-    total_ops = sum(2.0 * M * L["N"] * L["K"] for L in layers)
-    per_layer = {}
-    gemm_ms_sum = quant_ms_sum = 0.0
-    for li, L in enumerate(layers):
-        q_ms = statistics.mean(evs[k][li][0].elapsed_time(evs[k][li][1]) for k in range(args.steps))
-        g_ms = statistics.mean(evs[k][li][1].elapsed_time(evs[k][li][2]) for k in range(args.steps))
-        gemm_ms_sum += g_ms
-        quant_ms_sum += q_ms
-        per_layer[L["name"]] = {
-            "K": L["K"], "N": L["N"], "gemm_ms": round(g_ms, 4), "gemm_tops": round(2.0 * M * L["N"] * L["K"] / g_ms / 1e9, 1),
-            "quant_ms": round(q_ms, 4), "quant_gbs": round(quant_bytes(M, L["K"], L["bf6"]) / q_ms / 1e6, 1),
-            "matrix_path": "bf6" if L["bf6"] else "int8",
-        }
-    gemm_tops = total_ops / gemm_ms_sum / 1e9
-    quant_gbs = sum(quant_bytes(M, L["K"], L["bf6"]) for L in layers) / quant_ms_sum / 1e6
-    paths = sorted({"bf6" if L["bf6"] else "int8" for L in layers})
-    path = paths[0] if len(paths) == 1 else "mixed"
-    # a step that mixes both kinds of launches is priced against the higher peak
-    peak = INT8_PEAK_TOPS if path == "int8" else FP6_PEAK_TOPS
-    gemm_kernel = {"int8": "gemm_w4a4_kernel", "bf6": "gemm_bf6_persistent_kernel"}.get(path, "gemm_w4a4_kernel + gemm_bf6_persistent_kernel")
-    traffic = MEASURED_TRAFFIC.get((args.workload, path), {})
-    value = total_ops / (ms_per_step * 1e-3) / 1e12
-
+    wl = WORKLOADS[args.workload]
+    main_wl = Workload(torch, lib, v, args.workload, args.matrix_path, dev)
+    r = main_wl.measure(args.steps, args.warmup)
+    path = r["path"]
     result = {
         "metric": "W4A4 GEMM TOPS (% INT8-MFMA peak) at Wan-14B 720p shapes; A4-quant GB/s",
-        "value": round(value, 1), "unit": "TOPS", "n_gpus": 1, "steps": args.steps, "warmup": args.warmup,
-        "ms_per_step": round(ms_per_step, 4), "higher_is_better": True, "scaling": "weak", "vs_baseline": None,
+        "value": round(r["step_tops"], 1), "unit": "TOPS", "n_gpus": 1, "steps": args.steps, "warmup": args.warmup,
+        "ms_per_step": round(r["ms_per_step"], 4), "higher_is_better": True, "scaling": "weak", "vs_baseline": None,
         "dtype": ("int4 x int4 -> int32 (int8 MFMA), fp16 in/out" if path == "int8" else
                   "int4 x int4 as exact E3M2 floats -> fp32 accumulator holding the exact integer (FP6 MFMA), fp16 in/out"),
         "data": "synthetic", "matrix_path": path,
-        "config": {"workload": f"{args.workload}: M={M} tokens, linears " + ", ".join(f"{n} {k}->{o}" for n, k, o in wl["linears"])
+        "config": {"workload": f"{args.workload}: M={wl['M']} tokens, linears " + ", ".join(f"{n} {k}->{o}" for n, k, o in wl["linears"])
                                + "; each = A4 quantizer + W4A4 GEMM + scale/bias epilogue, clip 1.0"},
-        "roofline": {"bound": "mfma", "achieved": round(gemm_tops, 1), "peak": peak, "unit": "TOP/s",
-                     "frac": round(gemm_tops / peak, 4), "frac_of_int8_peak": round(gemm_tops / INT8_PEAK_TOPS, 4),
-                     "traffic": traffic.get("gemm"),
-                     "traffic_unit": "HBM bytes per launch (mean of the step's four launches)", "kernel": gemm_kernel,
-                     "algorithmic_ops_per_launch": total_ops / len(layers),
-                     "avg_launch_ms": round(gemm_ms_sum / len(layers), 4)},
-        "quantizer": {"bound": "hbm", "achieved": round(quant_gbs, 1), "peak": HBM_PEAK_GBS, "unit": "GB/s",
-                      "frac": round(quant_gbs / HBM_PEAK_GBS, 4), "traffic": traffic.get("quant"),
-                      "traffic_unit": "HBM bytes per launch (mean of the step's four launches)", "kernel": "quantize_rows_kernel",
-                      "algorithmic_bytes_per_launch": sum(quant_bytes(M, L["K"], L["bf6"]) for L in layers) / len(layers),
-                      "avg_launch_ms": round(quant_ms_sum / len(layers), 4)},
-        "per_linear": per_layer,
+        "roofline": r["roofline"], "quantizer": r["quantizer"], "per_linear": r["per_linear"],
     }
+    del main_wl
+    torch.cuda.empty_cache()
+    if not args.no_extras:
+        extra_steps, extra_warmup = max(3, args.steps // 4), 2
+        if path != "int8":  # the instruction the path was specified on: the same workload on the int8 matrix path
+            w8 = Workload(torch, lib, v, args.workload, "int8", dev)
+            r8 = w8.measure(extra_steps, extra_warmup)
+            result["int8_path"] = {"steps": extra_steps, "warmup": extra_warmup, "step_tops": round(r8["step_tops"], 1),
+                                   "ms_per_step": round(r8["ms_per_step"], 4), "roofline": r8["roofline"], "quantizer": r8["quantizer"],
+                                   "per_linear": r8["per_linear"]}
+            del w8
+            torch.cuda.empty_cache()
+        result["workloads"] = {}
+        for other in sorted(WORKLOADS):
+            if other == args.workload:
+                continue
+            wo = Workload(torch, lib, v, other, args.matrix_path, dev)
+            ro = wo.measure(extra_steps, extra_warmup)
+            result["workloads"][other] = {"M": WORKLOADS[other]["M"], "steps": extra_steps, "warmup": extra_warmup,
+                                          "step_tops": round(ro["step_tops"], 1), "ms_per_step": round(ro["ms_per_step"], 4),
+                                          "gemm_tops": ro["roofline"]["achieved"], "gemm_frac": ro["roofline"]["frac"],
+                                          "gemm_frac_of_int8_peak": ro["roofline"]["frac_of_int8_peak"],
+                                          "quant_gbs": ro["quantizer"]["achieved"], "quant_gbs_int4_bytes": ro["quantizer"]["achieved_int4_bytes"],
+                                          "per_linear": ro["per_linear"]}
+            del wo
+            torch.cuda.empty_cache()
+        result["mfma_ceiling"] = mfma_ceiling(torch, lib, dev)
     if not args.no_cpu_baseline:
         result["cpu_baseline"] = cpu_baseline(torch)
     print(json.dumps(result))

@@ -521,4 +521,16 @@ int vdmq_quantize_weight_native(const void *w, const void *scale_h, void *wq_nat
                                        static_cast<uint8_t *>(wq_native), as_stream(stream));
 }
 
+int64_t vdmq_mfma_probe_operand_bytes(void) { return mfma_probe_operand_bytes(); }
+
+int vdmq_mfma_probe(int kind, const void *operands, int64_t iters, int64_t workgroups, void *out, double *ops, vdmq_stream_t stream) {
+    if (kind != VDMQ_PROBE_INT8 && kind != VDMQ_PROBE_BF6) return fail(VDMQ_EINVAL, "unknown probe kind %d", kind);
+    if (iters <= 0 || iters > (1 << 30) || workgroups <= 0 || workgroups > (1 << 20))
+        return fail(VDMQ_ESHAPE, "iters and workgroups must be positive (got %lld, %lld)", (long long)iters, (long long)workgroups);
+    if (ops == nullptr) return fail(VDMQ_EINVAL, "ops is null");
+    VDMQ_TRY(check_ptr(operands, "operands"));
+    VDMQ_TRY(check_ptr(out, "out"));
+    return launch_mfma_probe(kind, operands, static_cast<int>(iters), static_cast<int>(workgroups), out, ops, as_stream(stream));
+}
+
 }  // extern "C"

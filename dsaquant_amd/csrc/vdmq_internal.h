@@ -66,4 +66,8 @@ int launch_gemm_bf6(const uint8_t *xblocks, const __half *ascale, const uint8_t 
                     __half *out, int32_t *acc_out, int64_t M, int64_t N, int64_t K, int64_t ldo, const GemmTail &tail,
                     hipStream_t stream);
 
+// matrix-pipe ceiling probe (vdmq_probe.hip)
+int64_t mfma_probe_operand_bytes();
+int launch_mfma_probe(int kind, const void *operands, int iters, int workgroups, void *out, double *ops, hipStream_t stream);
+
 }  // namespace vdmq

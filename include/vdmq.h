@@ -286,6 +286,20 @@ int vdmq_quantize_weight_native(const void *w, const void *scale_h, void *wq_nat
  * traffic counters are collected so that their readings can be scaled. */
 int vdmq_copy_u128(const void *src, void *dst, int64_t bytes, vdmq_stream_t stream);
 
+/* Matrix-pipe ceiling probe (no counterpart in the reference): the MFMA instruction of the int8 path
+ * (VDMQ_PROBE_INT8: v_mfma_i32_32x32x32_i8) or of the bf6 path (VDMQ_PROBE_BF6: v_mfma_f32_32x32x64_f8f6f4 on
+ * E3M2 operands) issued back to back -- 16 per loop iteration and wave onto 8 accumulator tiles, the GEMM kernels'
+ * wave tile -- by `workgroups` workgroups of eight waves, with no memory or LDS access in the loop.  `operands`
+ * holds the register contents: vdmq_mfma_probe_operand_bytes() bytes, [wave 0..7][operand 0..11][lane 0..63] x 32
+ * bytes (int8 reads the first 16 of each, bf6 the first 24; operands 0-1 and 6-7 are the weight side, 2-5 and 8-11
+ * the token side of the two operand sets).  `out` receives workgroups * 512 ints (a checksum that keeps the loop
+ * alive); *ops the operations one launch performs (2 per multiply-accumulate).  Timed by the caller: what it sustains
+ * on given operand data is the ceiling the GEMM kernels' rates are read against. */
+#define VDMQ_PROBE_INT8 0
+#define VDMQ_PROBE_BF6 1
+int64_t vdmq_mfma_probe_operand_bytes(void);
+int vdmq_mfma_probe(int kind, const void *operands, int64_t iters, int64_t workgroups, void *out, double *ops, vdmq_stream_t stream);
+
 #ifdef __cplusplus
 }
 #endif
