@@ -45,6 +45,8 @@ SIGNATURES = {
     "vdmq_gemm_w4a4": (_int, [_p, _p, _p, _p, _p, _p, _int, _i64, _i64, _i64, _i64, _p]),
     "vdmq_gemm_w4a4_ex": (_int, [_p, _p, _p, _p, _p, _p, _i64, _i64, _p, _i64, _p, _int, _i64, _i64, _i64, _i64, _p]),
     "vdmq_gemm_w4a4_acc": (_int, [_p, _p, _p, _i64, _i64, _i64, _p]),
+    "vdmq_gemm_w4a4_split": (_int, [_p, _p, _p, _p, _p, _p, _i64, _i64, _i64, _i64, _i64, _i64, _p]),
+    "vdmq_gemm_w4a4_bf6_split": (_int, [_p, _p, _p, _p, _p, _p, _i64, _i64, _i64, _i64, _i64, _i64, _p]),
     "vdmq_last_gemm_launch": (_int, [ctypes.POINTER(GemmLaunchInfo)]),
     "vdmq_workspace_bytes": (_i64, [_i64, _i64]),
     "vdmq_linear_w4a4": (_int, [_p, _i64, _i64, _i64, _f32, _p, _p, _p, _p, _int, _i64, _i64, _p, _i64, _p]),

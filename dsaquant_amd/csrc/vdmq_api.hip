@@ -224,6 +224,16 @@ static GemmTail make_tail(const void *gate, int64_t ldg, int64_t rows_per_gate, 
     return tail;
 }
 
+// Output split of vdmq_gemm_w4a4_split: checks, and the columns a row of `out` has to hold
+static int check_split(GemmTail &tail, int64_t N, int64_t split_cols, int64_t part_stride) {
+    if (split_cols <= 0 || split_cols % 64 != 0 || N % split_cols != 0)
+        return fail(VDMQ_ESHAPE, "split_cols must be a positive multiple of 64 that divides N (got %lld, N = %lld)", (long long)split_cols, (long long)N);
+    if (part_stride < 0 || part_stride % 8 != 0) return fail(VDMQ_ESHAPE, "part_stride must be a non-negative multiple of 8 (got %lld)", (long long)part_stride);
+    tail.split_cols = static_cast<int>(split_cols);
+    tail.part_stride = part_stride;
+    return VDMQ_OK;
+}
+
 static int gemm_checked(const void *qact, const void *ascale, const void *wq, const void *wscale, const void *bias, void *out,
                         int out_dtype, int32_t *acc, int64_t M, int64_t N, int64_t K, int64_t ldo, const GemmTail &tail,
                         vdmq_stream_t stream) {
@@ -239,10 +249,10 @@ static int gemm_checked(const void *qact, const void *ascale, const void *wq, co
         VDMQ_TRY(check_ptr(out, "out"));
         if (bias != nullptr) VDMQ_TRY(check_ptr(bias, "bias"));
         if (out_dtype != VDMQ_OUT_F16 && out_dtype != VDMQ_OUT_BF16) return fail(VDMQ_EINVAL, "unknown out_dtype %d", out_dtype);
-        if (ldo < N || ldo % 8 != 0 || ldo > kMaxLdo)
-            return fail(VDMQ_ESHAPE, "ldo must be >= N, a multiple of 8 and at most %lld (got %lld)", (long long)kMaxLdo, (long long)ldo);
-        if (tail.gate != nullptr || tail.residual != nullptr) {
-            if (out_dtype != VDMQ_OUT_F16) return fail(VDMQ_EINVAL, "gate and residual need an fp16 output");
+        if (ldo < (tail.split_cols ? tail.split_cols : N) || ldo % 8 != 0 || ldo > kMaxLdo)
+            return fail(VDMQ_ESHAPE, "ldo must be >= the columns of a row, a multiple of 8 and at most %lld (got %lld)", (long long)kMaxLdo, (long long)ldo);
+        if (tail.gate != nullptr || tail.residual != nullptr || tail.split_cols != 0) {
+            if (out_dtype != VDMQ_OUT_F16) return fail(VDMQ_EINVAL, "gate, residual and a split output need an fp16 output");
             VDMQ_TRY(check_tail(tail, N));
         }
     } else {
@@ -263,6 +273,13 @@ int vdmq_gemm_w4a4_ex(const void *qact, const void *ascale, const void *wq, cons
                       int64_t N, int64_t K, int64_t ldo, vdmq_stream_t stream) {
     return gemm_checked(qact, ascale, wq, wscale, bias, out, out_dtype, nullptr, M, N, K, ldo, make_tail(gate, ldg, rows_per_gate, residual, ldr),
                         stream);
+}
+
+int vdmq_gemm_w4a4_split(const void *qact, const void *ascale, const void *wq, const void *wscale, const void *bias, void *out, int64_t M,
+                         int64_t N, int64_t K, int64_t ldo, int64_t split_cols, int64_t part_stride, vdmq_stream_t stream) {
+    GemmTail tail;
+    VDMQ_TRY(check_split(tail, N, split_cols, part_stride));
+    return gemm_checked(qact, ascale, wq, wscale, bias, out, VDMQ_OUT_F16, nullptr, M, N, K, ldo, tail, stream);
 }
 
 int vdmq_gemm_w4a4_acc(const void *qact, const void *wq, int32_t *acc, int64_t M, int64_t N, int64_t K, vdmq_stream_t stream) {
@@ -376,8 +393,8 @@ static int gemm_bf6_checked(const void *xblocks, const void *ascale, const void 
         VDMQ_TRY(check_ptr(wscale, "wscale"));
         VDMQ_TRY(check_ptr(out, "out"));
         if (bias != nullptr) VDMQ_TRY(check_ptr(bias, "bias"));
-        if (ldo < N || ldo % 8 != 0 || ldo > kMaxLdo)
-            return fail(VDMQ_ESHAPE, "ldo must be >= N, a multiple of 8 and at most %lld (got %lld)", (long long)kMaxLdo, (long long)ldo);
+        if (ldo < (tail.split_cols ? tail.split_cols : N) || ldo % 8 != 0 || ldo > kMaxLdo)
+            return fail(VDMQ_ESHAPE, "ldo must be >= the columns of a row, a multiple of 8 and at most %lld (got %lld)", (long long)kMaxLdo, (long long)ldo);
         VDMQ_TRY(check_tail(tail, N));
     } else {
         VDMQ_TRY(check_ptr(acc, "acc"));
@@ -397,6 +414,13 @@ int vdmq_gemm_w4a4_bf6_ex(const void *xblocks, const void *ascale, const void *w
                           int64_t N, int64_t K, int64_t ldo, vdmq_stream_t stream) {
     return gemm_bf6_checked(xblocks, ascale, wblocks, wscale, bias, out, nullptr, M, N, K, ldo,
                             make_tail(gate, ldg, rows_per_gate, residual, ldr), stream);
+}
+
+int vdmq_gemm_w4a4_bf6_split(const void *xblocks, const void *ascale, const void *wblocks, const void *wscale, const void *bias, void *out,
+                             int64_t M, int64_t N, int64_t K, int64_t ldo, int64_t split_cols, int64_t part_stride, vdmq_stream_t stream) {
+    GemmTail tail;
+    VDMQ_TRY(check_split(tail, N, split_cols, part_stride));
+    return gemm_bf6_checked(xblocks, ascale, wblocks, wscale, bias, out, nullptr, M, N, K, ldo, tail, stream);
 }
 
 int vdmq_gemm_w4a4_bf6_acc(const void *xblocks, const void *wblocks, int32_t *acc, int64_t M, int64_t N, int64_t K,

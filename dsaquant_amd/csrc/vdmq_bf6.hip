@@ -145,8 +145,10 @@ __device__ __forceinline__ void bf6_epilogue(const v16f (&acc)[Cfg::NI][Cfg::MI]
     // vector offset only (a scalar offset is added after it), so the row goes into the vector offset: one addition
     // per store where a 64-bit address takes a multiplication and several additions.
     const int wave_rows = min(M - m0, MI * 32);
-    const __amdgpu_buffer_rsrc_t out_rsrc =
-        __builtin_amdgcn_make_buffer_rsrc(out + static_cast<int64_t>(m0) * ldo + n0, 0, wave_rows * static_cast<int>(ldo) * 2, 0x00020000);
+    const int part = tail.split_cols != 0 ? n0 / tail.split_cols : 0; /* the wave's 64 columns lie inside one part */
+    const __amdgpu_buffer_rsrc_t out_rsrc = __builtin_amdgcn_make_buffer_rsrc(
+        out + part * tail.part_stride + static_cast<int64_t>(m0) * ldo + (n0 - part * tail.split_cols), 0, wave_rows * static_cast<int>(ldo) * 2,
+        0x00020000);
     const int out_voff = ((lane / PR) * static_cast<int>(ldo) + (lane % PR) * 8) * 2;
     // Row of the gate vectors for output row m = m / rows_per_gate, without a division per element: one vector per
     // token is the row itself, and with at least as many rows per vector as the wave owns the wave's rows meet at

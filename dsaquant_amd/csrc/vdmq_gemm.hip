@@ -98,6 +98,7 @@ struct GemmCfg {
     static constexpr int kPiecesPerRow = kWaveN / 8; /* 16-byte pieces of one strip row */
     static_assert(kStagingBytes * kWaves <= kStageBytes * STAGES_, "epilogue staging reuses the stage ring");
     static_assert(kWaveN <= 64, "one lane per column fetches the channel scale and the bias");
+    static_assert(kWaveN == 64, "an output split by blocks of 64 columns keeps a wave's stores inside one part");
     static_assert(kRowBlocks % kWaves == 0, "row blocks must divide evenly over the waves");
     static_assert(BN % kDmaRows == 0 && kWaveM % 32 == 0 && kWaveN % 32 == 0, "tile shape");
     static_assert(kLoads * (STAGES - 1) < 64, "vmcnt is a 6-bit counter");
@@ -397,8 +398,10 @@ __global__ __launch_bounds__(Cfg::kThreads, Cfg::kOccupancy * Cfg::kWaves / 4) v
         // offset: one addition per store where a 64-bit address takes a multiplication and several additions.
         const int wave_rows = min(max(M - (m0 + wm0), 0), Cfg::kWaveM);
         if (n0 + wn0 >= N || wave_rows == 0) return; /* the same for the whole wave */
+        const int part = tail.split_cols != 0 ? (n0 + wn0) / tail.split_cols : 0; /* the wave's columns lie inside one part */
         const __amdgpu_buffer_rsrc_t out_rsrc = __builtin_amdgcn_make_buffer_rsrc(
-            static_cast<__half *>(out) + static_cast<int64_t>(m0 + wm0) * ldo + n0 + wn0, 0, wave_rows * static_cast<int>(ldo) * 2, 0x00020000);
+            static_cast<__half *>(out) + part * tail.part_stride + static_cast<int64_t>(m0 + wm0) * ldo + (n0 + wn0 - part * tail.split_cols), 0,
+            wave_rows * static_cast<int>(ldo) * 2, 0x00020000);
         const int out_voff = ((lane / PR) * static_cast<int>(ldo) + (lane % PR) * 8) * 2;
         // Row of the gate vectors for output row m = m / rows_per_gate, without a division per element: one vector per
         // token is the row itself, and with at least as many rows per vector as the wave owns the wave's rows meet at

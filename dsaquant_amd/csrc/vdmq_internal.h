@@ -41,6 +41,11 @@ struct GemmTail {
     int rows_per_gate = 1;
     const __half *residual = nullptr; /* fp16 [M, N], row stride ldr */
     int64_t ldr = 0;
+    // Output split by column blocks (0 = none): element (m, n) goes to out[(n / split_cols) * part_stride + m * ldo +
+    // n % split_cols]; split_cols is a multiple of 64, the width of a wave's corner of a tile, so a wave's stores
+    // stay inside one part.  Gate and residual keep their [*, N] addressing.
+    int split_cols = 0;
+    int64_t part_stride = 0;
 };
 
 int launch_gemm(const uint8_t *qact, const __half *ascale, const uint8_t *wq, const __half *wscale, const __half *bias,

@@ -160,6 +160,7 @@ def linear_fused(
     act: Optional[str] = None,
     residual: Optional[torch.Tensor] = None,
     gate: Optional[torch.Tensor] = None,
+    split_cols: Optional[int] = None,
 ) -> torch.Tensor:
     """``residual + linear_vdm_w4a4(act(x), ...) * gate`` in two kernels.
 
@@ -170,7 +171,8 @@ def linear_fused(
     GEMM epilogue as the two fp16 tensor operations of the reference's
     ``hidden_states + attn_output * gate`` (dit_block.py:102, :107, :112); either may
     be omitted.  ``qweight`` may be a ``PreparedWeight`` (then ``wscales`` is ignored): the concatenated weight of a
-    fused projection.  Returns a new tensor; nothing is updated in place."""
+    fused projection.  ``split_cols``: the output columns as N / split_cols contiguous tensors, stacked in front
+    (``[N / split_cols, ..., split_cols]``; without gate and residual).  Returns a new tensor; nothing is updated in place."""
     _k._load_ext()  # raises when the library is missing
     if isinstance(x, LnInput):
         if act is not None:
@@ -220,15 +222,20 @@ def linear_fused(
             raise ValueError(f"residual must have shape {tuple(lead) + (N,)}, got {tuple(residual.shape)}")
         r2 = residual.reshape(-1, N).half().contiguous()
         _k._check_device_tensor(r2, "residual", torch.float16)
+    if split_cols is not None:
+        if gate is not None or residual is not None:
+            raise ValueError("a split output takes neither gate nor residual")
+        if split_cols <= 0 or split_cols % 64 != 0 or N % split_cols != 0:
+            raise ValueError(f"split_cols must be a positive multiple of 64 that divides N={N} (got {split_cols})")
     with torch.cuda.device(dev):
-        out = torch.empty((M, N), dtype=torch.float16, device=dev)
+        out = torch.empty((M, N) if split_cols is None else (N // split_cols, M, split_cols), dtype=torch.float16, device=dev)
         if M and isinstance(pre, QuantizedInput):
             _k._gemm_dispatch(pre.qact, pre.scales, False, weight, b, out, K, gate=g2, rows_per_gate=rows_per_gate, residual=r2)
         elif M:
             bf6 = _k._use_bf6(M, N, K)
             operand, scales = _k._quantize_for_gemm(x_2d, clip_ratio, act_code, bf6, None if pre is None else pre._args())
             _k._gemm_dispatch(operand, scales, bf6, weight, b, out, K, gate=g2, rows_per_gate=rows_per_gate, residual=r2)
-    return out.view(*lead, N)
+    return out.view(*lead, N) if split_cols is None else out.view(N // split_cols, *lead, split_cols)
 
 
 def qkv_projections_ln(attn, pre: LnInput):
@@ -238,9 +245,10 @@ def qkv_projections_ln(attn, pre: LnInput):
     from .fused_qkv import _cat_prepared
 
     w, b = _cat_prepared(attn, ["to_q", "to_k", "to_v"], "qkv")
-    out = linear_ln_vdm_w4a4(pre, w, None, None, attn.to_q.kernel_clip_ratio, bias_half=b)
     n = attn.to_q.vdm_weight_packed.shape[0]
-    return out.split(n, dim=-1)
+    if getattr(attn, "qkv_contiguous_outputs", True):
+        return linear_fused(pre, w, None, None, attn.to_q.kernel_clip_ratio, bias_half=b, split_cols=n).unbind(0)
+    return linear_ln_vdm_w4a4(pre, w, None, None, attn.to_q.kernel_clip_ratio, bias_half=b).split(n, dim=-1)
 
 
 def kv_projections(attn, encoder_hidden_states):
@@ -249,5 +257,7 @@ def kv_projections(attn, encoder_hidden_states):
     from .fused_qkv import _cat_prepared
 
     w, b = _cat_prepared(attn, ["to_k", "to_v"], "kv")
-    kv = linear_fused(encoder_hidden_states, w, None, None, attn.to_k.kernel_clip_ratio, bias_half=b)
-    return kv.split(attn.to_k.vdm_weight_packed.shape[0], dim=-1)
+    n = attn.to_k.vdm_weight_packed.shape[0]
+    if getattr(attn, "qkv_contiguous_outputs", True):
+        return linear_fused(encoder_hidden_states, w, None, None, attn.to_k.kernel_clip_ratio, bias_half=b, split_cols=n).unbind(0)
+    return linear_fused(encoder_hidden_states, w, None, None, attn.to_k.kernel_clip_ratio, bias_half=b).split(n, dim=-1)

@@ -57,8 +57,12 @@ def _project_cat(attn, names: List[str], prefix: str, x: torch.Tensor, clip_rati
     from dsaquant_amd.kernels import vdm_w4a4 as k
 
     weight, bias = _cat_prepared(attn, names, prefix)
-    out = k.linear_vdm_w4a4_prepared(x, weight, bias, clip_ratio)
-    return out.split(getattr(attn, names[0]).vdm_weight_packed.shape[0], dim=-1)
+    n = getattr(attn, names[0]).vdm_weight_packed.shape[0]
+    if getattr(attn, "qkv_contiguous_outputs", True):
+        # each projection's output as its own contiguous tensor, written in place by the GEMM epilogue: the values of
+        # the reference's strided views (vdm_w4a4.py:297-298) without the strides
+        return k.linear_vdm_w4a4_prepared(x, weight, bias, clip_ratio, split_cols=n).unbind(0)
+    return k.linear_vdm_w4a4_prepared(x, weight, bias, clip_ratio).split(n, dim=-1)
 
 
 def get_qkv_projections(attn, hidden_states: torch.Tensor, encoder_hidden_states: Optional[torch.Tensor]):

@@ -362,12 +362,20 @@ def _quantize_for_gemm(x_2d: torch.Tensor, clip_ratio: float, act_code: int, bf6
 def _gemm_dispatch(operand: torch.Tensor, scales: torch.Tensor, bf6: bool, weight: PreparedWeight,
                    bias: Optional[torch.Tensor], out: torch.Tensor, K: int, gate: Optional[torch.Tensor] = None, rows_per_gate: int = 1,
                    residual: Optional[torch.Tensor] = None) -> None:
-    """GEMM + epilogue on a quantized activation (bf6 blocks if ``bf6`` else native rows) into ``out``.
+    """GEMM + epilogue on a quantized activation (bf6 blocks if ``bf6`` else native rows) into ``out`` [M, N], or,
+    for an ``out`` of shape [N / cols, M, cols], into N / cols separate matrices (vdmq_gemm_w4a4_split).
     Must run under ``torch.cuda.device(out.device)``."""
     lib = _load_ext()
-    M, N = out.shape
     s = _stream(out.device)
     bias_p = None if bias is None else bias.data_ptr()
+    if out.dim() == 3:
+        _require(gate is None and residual is None and out.dtype == torch.float16, "a split output takes neither gate nor residual and is fp16")
+        parts, M, cols = out.shape
+        fn = lib.vdmq_gemm_w4a4_bf6_split if bf6 else lib.vdmq_gemm_w4a4_split
+        _lib.check(fn(operand.data_ptr(), scales.data_ptr(), weight.operand(bf6).data_ptr(), weight.wscale.data_ptr(), bias_p, out.data_ptr(),
+                      M, parts * cols, K, out.stride(1), cols, out.stride(0), s))
+        return
+    M, N = out.shape
     gate_p, ldg = (None, 0) if gate is None else (gate.data_ptr(), gate.stride(0))
     res_p, ldr = (None, 0) if residual is None else (residual.data_ptr(), residual.stride(0))
     w, wscale = weight.operand(bf6), weight.wscale
@@ -439,7 +447,8 @@ def _act_code(act: Optional[str]) -> int:
 
 
 def _linear_2d(x_2d: torch.Tensor, weight: PreparedWeight, bias: Optional[torch.Tensor], clip_ratio: float,
-               out_dtype: torch.dtype = torch.float16, act: Optional[str] = None) -> torch.Tensor:
+               out_dtype: torch.dtype = torch.float16, act: Optional[str] = None, split_cols: Optional[int] = None) -> torch.Tensor:
+    """[M, N], or [N / split_cols, M, split_cols] with ``split_cols`` (each part a contiguous matrix)."""
     _load_ext()  # raises when the library is missing
     M, K = x_2d.shape
     N = weight.N
@@ -449,8 +458,11 @@ def _linear_2d(x_2d: torch.Tensor, weight: PreparedWeight, bias: Optional[torch.
         _check_device_tensor(bias, "bias", torch.float16)
         _require(bias.dim() == 1, "bias must be [N]")
         _require(bias.numel() == N, "bias length must equal N")
+    if split_cols is not None and (split_cols <= 0 or split_cols % 64 != 0 or N % split_cols != 0):
+        raise ValueError(f"split_cols must be a positive multiple of 64 that divides N={N} (got {split_cols})")
     with torch.cuda.device(dev):
-        out = torch.empty((M, N), dtype=out_dtype, device=dev)
+        shape = (M, N) if split_cols is None else (N // split_cols, M, split_cols)
+        out = torch.empty(shape, dtype=out_dtype, device=dev)
         if M == 0:
             return out
         bf6 = _use_bf6(M, N, K, out_dtype)
@@ -478,22 +490,26 @@ def linear_vdm_w4a4(
 
 
 def linear_vdm_w4a4_prepared(x: torch.Tensor, weight: PreparedWeight, bias_half: Optional[torch.Tensor] = None,
-                             clip_ratio: float = 1.0) -> torch.Tensor:
+                             clip_ratio: float = 1.0, split_cols: Optional[int] = None) -> torch.Tensor:
     """``linear_vdm_w4a4`` on a weight that is already in the kernels' form -- what the fused QKV / KV dispatch calls
     with the concatenated weight of an attention module (no counterpart in the reference, which passes concatenated
-    v1 buffers to the same function)."""
+    v1 buffers to the same function).  ``split_cols``: the N output columns are written as N / split_cols separate
+    contiguous tensors, returned stacked as ``[N / split_cols, ..., split_cols]`` -- the bits of
+    ``out.split(split_cols, -1)``, without the strided views (the GEMM epilogue writes them in place)."""
     _load_ext()
     x_2d, orig_shape = _as_2d_half_contiguous(x)
     if weight.K != x_2d.shape[1]:
         raise ValueError("qweight shape must be [N, K/2]")
     _require(x_2d.is_cuda, "input must be a CUDA tensor")
-    return _linear_prepared(x_2d, weight, bias_half, clip_ratio).view(*orig_shape, -1)
+    out = _linear_prepared(x_2d, weight, bias_half, clip_ratio, split_cols)
+    return out.view(*orig_shape, -1) if split_cols is None else out.view(out.shape[0], *orig_shape, split_cols)
 
 
-def _linear_prepared(x_2d: torch.Tensor, weight: PreparedWeight, bias: Optional[torch.Tensor], clip_ratio: float) -> torch.Tensor:
+def _linear_prepared(x_2d: torch.Tensor, weight: PreparedWeight, bias: Optional[torch.Tensor], clip_ratio: float,
+                     split_cols: Optional[int] = None) -> torch.Tensor:
     if bias is not None:
         bias = bias.half().contiguous().view(-1)
-    return _linear_2d(x_2d, weight, bias, clip_ratio)
+    return _linear_2d(x_2d, weight, bias, clip_ratio, split_cols=split_cols)
 
 
 def quantize_activation_per_token(x: torch.Tensor, clip_ratio: float = 1.0):
@@ -618,13 +634,16 @@ def linear_vdm_w4a4_qkv(
     w_qkv_packed: Optional[torch.Tensor] = None,
     w_qkv_scale: Optional[torch.Tensor] = None,
     qkv_bias_half: Optional[torch.Tensor] = None,
+    contiguous_outputs: bool = False,
 ):
     """Fused QKV: one activation quantization and one GEMM against the row-concatenated Wq|Wk|Wv; returns three
     views of one [..., 3N] tensor.  Signature, argument handling (cached concatenation if given, zeros for missing
     biases, ``split(n)``) and results are fixed by the reference's function of the same name (vdm_w4a4.py:259-298),
     which this follows step by step.  Without the cached concatenation the reference concatenates the v1 buffers on
     every call; here the three buffers are relaid once into one operand (every 128-row block of a v1 buffer is
-    self-contained, so the concatenation's operand is the parts' operands one after the other) and that is kept."""
+    self-contained, so the concatenation's operand is the parts' operands one after the other) and that is kept.
+    ``contiguous_outputs`` (not in the reference): q, k and v are written by the GEMM epilogue as three contiguous
+    tensors instead of strided views of one -- the same bits."""
     if w_qkv_packed is None or w_qkv_scale is None:
         weight = _prepared([(q_weight_packed.contiguous(), q_weight_scale.contiguous()), (k_weight_packed.contiguous(), k_weight_scale.contiguous()),
                             (v_weight_packed.contiguous(), v_weight_scale.contiguous())])
@@ -639,5 +658,7 @@ def linear_vdm_w4a4_qkv(
     x_2d, orig_shape = _as_2d_half_contiguous(x)
     _check_packed_weight(q_weight_packed, q_weight_scale, x_2d.shape[1])
     _require(x_2d.is_cuda, "input must be a CUDA tensor")
+    if contiguous_outputs:
+        return _linear_prepared(x_2d, weight, qkv_bias_half, clip_ratio, split_cols=n).view(3, *orig_shape, n).unbind(0)
     qkv = _linear_prepared(x_2d, weight, qkv_bias_half, clip_ratio).view(*orig_shape, -1)
     return qkv.split(n, dim=-1)

@@ -139,6 +139,18 @@ int vdmq_gemm_w4a4_ex(const void *qact, const void *ascale, const void *wq, cons
                       int64_t ldg, int64_t rows_per_gate, const void *residual, int64_t ldr, void *out, int out_dtype, int64_t M,
                       int64_t N, int64_t K, int64_t ldo, vdmq_stream_t stream);
 
+/* vdmq_gemm_w4a4 (fp16 output) writing its N columns as N / split_cols separate matrices: element (m, n) goes to
+ *   out[(n / split_cols) * part_stride + m * ldo + n % split_cols]        (fp16 elements)
+ * -- the same values vdmq_gemm_w4a4 writes to out[m * ldo + n].  For the fused QKV projection (N = 3 * dim, the
+ * reference splits one [M, 3 * dim] result into strided views and unflattens them per head,
+ * vdm_infer/kernels/vdm_w4a4.py:297-298, vdm_infer/models/wan_vdm/modules/attention.py:165-172):
+ *   split_cols = dim, ldo = dim, part_stride = M * dim        q, k, v as three contiguous [M, dim] matrices
+ *   split_cols = head_dim, ldo = head_dim, part_stride = M * head_dim
+ *                                                           head-major: [3 * heads][M][head_dim]
+ * split_cols is a multiple of 64 that divides N; ldo >= split_cols, ldo and part_stride multiples of 8. */
+int vdmq_gemm_w4a4_split(const void *qact, const void *ascale, const void *wq, const void *wscale, const void *bias, void *out, int64_t M,
+                         int64_t N, int64_t K, int64_t ldo, int64_t split_cols, int64_t part_stride, vdmq_stream_t stream);
+
 /* Same GEMM, but writes the raw int32 accumulators acc [M, N] (row stride N)
  * instead of the scaled output: the checker's view of the value the reference
  * holds in `ipsum` before finalize_int_accum (vdm_w4a4_kernel.cu:650, :684). */
@@ -244,6 +256,9 @@ int vdmq_gemm_w4a4_bf6(const void *xblocks, const void *ascale, const void *wblo
 int vdmq_gemm_w4a4_bf6_ex(const void *xblocks, const void *ascale, const void *wblocks, const void *wscale, const void *bias,
                           const void *gate, int64_t ldg, int64_t rows_per_gate, const void *residual, int64_t ldr, void *out, int64_t M,
                           int64_t N, int64_t K, int64_t ldo, vdmq_stream_t stream); /* with vdmq_gemm_w4a4_ex's tail */
+int vdmq_gemm_w4a4_bf6_split(const void *xblocks, const void *ascale, const void *wblocks, const void *wscale, const void *bias, void *out,
+                             int64_t M, int64_t N, int64_t K, int64_t ldo, int64_t split_cols, int64_t part_stride,
+                             vdmq_stream_t stream); /* vdmq_gemm_w4a4_split on bf6 operands */
 int vdmq_gemm_w4a4_bf6_acc(const void *xblocks, const void *wblocks, int32_t *acc, int64_t M, int64_t N, int64_t K,
                            vdmq_stream_t stream);
 

@@ -80,9 +80,10 @@ def test_small_dit_structure_and_numerics():
             yy = yy + b.half()
         return yy.view(*x.shape[:-1], N)
 
-    def ref_prepared(x, weight, bias_half=None, clip_ratio=1.0):  # the fused QKV / KV calls: a concatenated weight
+    def ref_prepared(x, weight, bias_half=None, clip_ratio=1.0, split_cols=None):  # the fused QKV / KV calls: a concatenated weight
         parts = weight.sources()
-        return ref_linear(x, torch.cat([q for q, _ in parts]), torch.cat([s for _, s in parts]), None, clip_ratio, bias_half)
+        out = ref_linear(x, torch.cat([q for q, _ in parts]), torch.cat([s for _, s in parts]), None, clip_ratio, bias_half)
+        return out if split_cols is None else torch.stack(out.split(split_cols, dim=-1))
 
     orig = v.linear_vdm_w4a4, v.linear_vdm_w4a4_prepared
     v.linear_vdm_w4a4, v.linear_vdm_w4a4_prepared = ref_linear, ref_prepared

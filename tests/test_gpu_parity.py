@@ -373,6 +373,56 @@ def test_fused_qkv_is_bitwise_three_separate_calls():
     assert torch.equal(q2, sep[0]) and torch.equal(k2, sep[1]) and torch.equal(v2, sep[2])
 
 
+@pytest.mark.parametrize("M,K,n", [(1000, 1536, 1536), (8200, 512, 1536), (3000, 256, 128)])
+def test_split_outputs_are_the_bits_of_the_strided_views(each_matrix_path, M, K, n):
+    """Fused QKV with q, k, v written as three contiguous tensors by the GEMM epilogue, and head-major
+    ([3 * heads, M, 128]): the same bits as splitting the one [M, 3n] result (vdm_w4a4.py:297-298, attention.py:165-172
+    of the reference); raw C-ABI call with a part stride larger than a part; the Python entries; bad splits refused."""
+    from dsaquant_amd import _lib, fused_ops
+
+    v = vk()
+    lib = _lib.load()
+    x = O.synth_linear(M, K, 128, seed=n)[0]
+    parts = [O.synth_linear(1, K, n, seed=50 + i) for i in range(3)]
+    W = [t16(O.np_pack_wgt_v1(p[1])) for p in parts]
+    S = [t16(O.np_pack_wscales_v1(p[2], K)) for p in parts]
+    B = [t16(p[3]) for p in parts]
+    xt = t16(x)
+    print(f"split outputs M={M} K={K} n={n} path={each_matrix_path}", flush=True)
+    q0, k0, v0 = v.linear_vdm_w4a4_qkv(xt, W[0], S[0], W[1], S[1], W[2], S[2], B[0], B[1], B[2], clip_ratio=0.95)
+    assert not q0.is_contiguous()
+    q1, k1, v1 = v.linear_vdm_w4a4_qkv(xt, W[0], S[0], W[1], S[1], W[2], S[2], B[0], B[1], B[2], clip_ratio=0.95, contiguous_outputs=True)
+    assert all(t.is_contiguous() and t.shape == (M, n) for t in (q1, k1, v1))
+    assert torch.equal(q1, q0) and torch.equal(k1, k0) and torch.equal(v1, v0)
+    want = O.np_linear(x[:64], parts[1][1], parts[1][2], parts[1][3], 0.95)[0]
+    assert np.array_equal(k1[:64].cpu().numpy().view(np.uint16), want.view(np.uint16))
+    # head-major through the prepared-weight entry: [3 * heads, M, 128]
+    weight = v._prepared([(W[i], S[i]) for i in range(3)])
+    heads = v.linear_vdm_w4a4_prepared(xt, weight, torch.cat(B), 0.95, split_cols=128)
+    assert heads.shape == (3 * n // 128, M, 128) and heads.is_contiguous()
+    assert torch.equal(heads.permute(1, 0, 2).reshape(M, 3 * n), torch.cat([q0, k0, v0], dim=1))
+    # LayerNorm input + split, against LayerNorm input without
+    rng = np.random.default_rng(1)
+    a, b = t16((0.2 * rng.standard_normal((1, K))).astype(np.float16)), t16((0.3 * rng.standard_normal((1, K))).astype(np.float16))
+    whole = fused_ops.linear_fused(fused_ops.LnInput(xt, a, b, 1e-6), weight, None, None, 0.95, bias_half=torch.cat(B))
+    three = fused_ops.linear_fused(fused_ops.LnInput(xt, a, b, 1e-6), weight, None, None, 0.95, bias_half=torch.cat(B), split_cols=n)
+    assert torch.equal(three.permute(1, 0, 2).reshape(M, 3 * n), whole)
+    # raw C ABI on the int8 path: parts one row further apart than they are long, the gap untouched
+    qn, sc = v.quantize_activation_native(xt, 0.95)
+    out = torch.full((3, M + 1, n), -3.0, dtype=torch.float16, device=DEV)
+    _lib.check(lib.vdmq_gemm_w4a4_split(qn.data_ptr(), sc.data_ptr(), weight.operand(False).data_ptr(), weight.wscale.data_ptr(),
+                                        torch.cat(B).data_ptr(), out.data_ptr(), M, 3 * n, K, n, n, (M + 1) * n, torch.cuda.current_stream().cuda_stream))
+    torch.cuda.synchronize()
+    v.set_matrix_path("int8")
+    ref = v.linear_vdm_w4a4_qkv(xt, W[0], S[0], W[1], S[1], W[2], S[2], B[0], B[1], B[2], clip_ratio=0.95)
+    assert all(torch.equal(out[i, :M], ref[i]) for i in range(3)) and (out[:, M] == -3.0).all()
+    fake = out.data_ptr()
+    assert lib.vdmq_gemm_w4a4_split(fake, fake, fake, fake, None, fake, M, 3 * n, K, n, n + 32, M * n, None) == -2  # not a multiple of 64
+    assert lib.vdmq_gemm_w4a4_split(fake, fake, fake, fake, None, fake, M, 3 * n, K, 64, n, M * n, None) == -2      # rows shorter than a part
+    with pytest.raises(ValueError):
+        v.linear_vdm_w4a4_prepared(xt, weight, None, 0.95, split_cols=96)
+
+
 # ------------------------------------------------- GELU fused into the quantizer
 
 def gpu_gelu_table():
