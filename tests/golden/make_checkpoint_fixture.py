@@ -23,26 +23,8 @@ import torch.nn as nn
 
 ROOT = Path(__file__).resolve().parents[2]
 HERE = Path(__file__).resolve().parent
-QPARAMS = {"w": {"bit": 4, "sym": True}, "act": {"bit": 4, "sym": True}}
-
-
-def build_toy(quant_linear_cls, seed: int = 0) -> nn.Module:
-    """One plain linear, one norm and two QuantLinear layers (with and without bias); the tests build the same
-    model from this repository's QuantLinear."""
-    torch.manual_seed(seed)
-
-    class Toy(nn.Module):
-        def __init__(self):
-            super().__init__()
-            self.pre = nn.Linear(8, 64)
-            self.norm = nn.LayerNorm(64)
-            self.q1 = quant_linear_cls(nn.Linear(64, 128, bias=True), {"w": "lsq", "act": "dynamic"}, QPARAMS)
-            self.q2 = quant_linear_cls(nn.Linear(128, 128, bias=False), {"w": "lsq", "act": "dynamic"}, QPARAMS)
-
-        def forward(self, x):
-            return self.q2(self.q1(self.norm(self.pre(x))))
-
-    return Toy()
+sys.path.insert(0, str(ROOT))
+from tests.toy_model import build_toy  # noqa: E402  (the tests build the same model from this repository's QuantLinear)
 
 
 def load_by_path(name: str, path: Path):

@@ -1049,19 +1049,16 @@ def test_reference_written_checkpoint_runs_through_the_kernels(tag):
     """The checkpoint the reference's own save_packed_checkpoint wrote (tests/golden/make_checkpoint_fixture.py), loaded
     with the kernel required: both QuantLinear layers give the oracle's fp16 bits for the integers and scales the
     file holds, at the module's clip ratio of 0.95 (quant_linear.py:121, :163-172)."""
-    import importlib.util
     from pathlib import Path
 
     from dsaquant_amd.checkpoints import packed_checkpoint as pc
     from dsaquant_amd.quantization.quant_linear import QuantLinear
+    from tests.toy_model import build_toy
 
     vk()
     golden = Path(__file__).parent / "golden"
-    spec = importlib.util.spec_from_file_location("_make_checkpoint_fixture", golden / "make_checkpoint_fixture.py")
-    gen = importlib.util.module_from_spec(spec)
-    spec.loader.exec_module(gen)
     ckpt = pc.load_quant_checkpoint(str(golden / f"reference_written_packed_{tag}.pt"), dcp_loader=None)
-    model = gen.build_toy(QuantLinear, seed=3)
+    model = build_toy(QuantLinear, seed=3)
     missing, unexpected = pc.load_packed_quantized_model(model, ckpt, quant_linear_cls=QuantLinear, dtype=torch.float16,
                                                         device=torch.device("cuda:0"))
     assert missing == [] and unexpected == []
