@@ -92,6 +92,14 @@ def rope_frequencies(head_dim: int, f: int, h: int, w: int, device) -> torch.Ten
     return freqs.reshape(f * h * w, 1, -1).to(torch.complex64).to(device)
 
 
+def timestep_embedding(freq_dim: int, timestep: torch.Tensor) -> torch.Tensor:
+    """[B] -> [B, freq_dim] in float64: cos of the freq_dim/2 angles t * 10000^(-i / (freq_dim/2)) first, then their
+    sin (modules/embedding.py:7-10)."""
+    half = freq_dim // 2
+    ang = torch.outer(timestep.double(), torch.pow(10000.0, -torch.arange(half, dtype=torch.float64, device=timestep.device) / half))
+    return torch.cat([torch.cos(ang), torch.sin(ang)], dim=1)
+
+
 def apply_rope(x: torch.Tensor, freqs: torch.Tensor) -> torch.Tensor:
     """x [B, L, H, D]; consecutive channel pairs are rotated (fp32 complex arithmetic)."""
     xc = torch.view_as_complex(x.float().reshape(*x.shape[:-1], -1, 2))
@@ -310,10 +318,12 @@ class WanDiT(nn.Module):
         return x.permute(0, 2, 4, 6, 1, 3, 5, 7).reshape(1, (f // p1) * (h // p2) * (w // p3), c * p1 * p2 * p3)
 
     def unpatchify(self, tokens: torch.Tensor, f: int, h: int, w: int) -> torch.Tensor:
+        """[1, L, 4*C] -> [1, C, F, H, W]: the head's output of a token is patch-position major, channel minor
+        ('1 l (n c) -> 1 (l n) c' with n = 4, modules/model.py:353), unlike the channel-major input patches."""
         p1, p2, p3 = self.args.patch_size
         c = self.args.in_channels
-        x = tokens.reshape(1, f // p1, h // p2, w // p3, c, p1, p2, p3)
-        return x.permute(0, 4, 1, 5, 2, 6, 3, 7).reshape(1, c, f, h, w)
+        x = tokens.reshape(1, f // p1, h // p2, w // p3, p1, p2, p3, c)
+        return x.permute(0, 7, 1, 4, 2, 5, 3, 6).reshape(1, c, f, h, w)
 
     # reuse_context: embed each context tensor once (the prompt's cond / uncond embeddings are the same tensors in
     # every denoise step), keep the blocks' cross-attention K/V per embedded context, and quantize a context that
@@ -336,9 +346,7 @@ class WanDiT(nn.Module):
         _, _, f, h, w = latent.shape
         freqs = rope_frequencies(a.head_dim, f // a.patch_size[0], h // a.patch_size[1], w // a.patch_size[2], latent.device)
         x = self.patch_embedding_mlp(self.patchify(latent))
-        half = a.freq_dim // 2
-        ang = torch.outer(timestep.double(), torch.pow(10000.0, -torch.arange(half, dtype=torch.float64, device=latent.device) / half))
-        temb = self.time_embedder(torch.cat([torch.cos(ang), torch.sin(ang)], dim=1).to(x.dtype))
+        temb = self.time_embedder(timestep_embedding(a.freq_dim, timestep).to(x.dtype))
         tproj = self.time_proj(F.silu(temb)).unflatten(1, (6, -1))
         ctx = self._embedded_context(context)
         for blk in self.blocks:

@@ -194,16 +194,3 @@ def test_first_call_after_load_can_be_captured():
             want = [layer(x), *W.get_qkv_projections(attn, x, None)]
         torch.cuda.synchronize()
         assert all(torch.equal(a, b) for a, b in zip(got, want)), it
-
-
-def test_patchify_roundtrip():
-    from dsaquant_amd import wan_harness as W
-
-    with torch.device("meta"):
-        m = W.WanDiT(replace(W.WAN21_1P3B, num_layers=1))
-    x = torch.arange(16 * 3 * 8 * 12, dtype=torch.float32).reshape(1, 16, 3, 8, 12)
-    tok = m.patchify(x)
-    assert tok.shape == (1, 3 * 4 * 6, 64)
-    assert torch.equal(m.unpatchify(tok, 3, 8, 12), x)
-    # token 0 holds channel-major 2x2 patches: element [c, dh, dw] at index c*4 + dh*2 + dw
-    assert tok[0, 0, 5].item() == x[0, 1, 0, 0, 1].item()
