@@ -386,11 +386,15 @@ __global__ __launch_bounds__(Cfg::kWaves * 64, (Cfg::kWaves * Cfg::kOcc + 3) / 4
         if (tile_m >= tmap.tiles_m || tile_n >= tmap.tiles_n) tile_m = -1;
         return true;
     };
-    auto next_tile = [&](int &seq, int &tile_m, int &tile_n) -> bool { /* advances seq to the next existing tile */
+    // Advances seq to the next existing tile; `skipped` counts the super-tiles passed on the way in which this place
+    // has no tile (a ragged edge).
+    auto next_tile = [&](int &seq, int &tile_m, int &tile_n, int &skipped) -> bool {
+        skipped = 0;
         for (;;) {
             ++seq;
             if (!locate(seq, tile_m, tile_n)) return false;
             if (tile_m >= 0) return true;
+            ++skipped;
         }
     };
     uint32_t lane_off[kLoads];
@@ -455,8 +459,8 @@ __global__ __launch_bounds__(Cfg::kWaves * 64, (Cfg::kWaves * Cfg::kOcc + 3) / 4
                 acc[ni][mi] = __builtin_amdgcn_mfma_scale_f32_32x32x64_f8f6f4(wf[ni], xf[mi], acc[ni][mi], 3, 3, 0, 0, 0, 0);
     };
 
-    int seq = -1, tile_m = -1, tile_n = 0;
-    if (!next_tile(seq, tile_m, tile_n)) return;
+    int seq = -1, tile_m = -1, tile_n = 0, skipped = 0;
+    if (!next_tile(seq, tile_m, tile_n, skipped)) return;
     __amdgpu_buffer_rsrc_t src[kLoads];
     sources(src, tile_m, tile_n);
     bool k_reverse = tmap.contig && (seq & 1) != 0;
@@ -475,6 +479,7 @@ __global__ __launch_bounds__(Cfg::kWaves * 64, (Cfg::kWaves * Cfg::kOcc + 3) / 4
     int cur = 0; /* ring slot of the tile's K step under work */
     v8i wfa[NI], xfa[MI], wfb[NI], xfb[MI];
     for (;;) {
+        const uint64_t tile_started = wall_clock64(); /* 100 MHz */
 #pragma unroll
         for (int ni = 0; ni < NI; ++ni)
 #pragma unroll
@@ -508,25 +513,31 @@ __global__ __launch_bounds__(Cfg::kWaves * 64, (Cfg::kWaves * Cfg::kOcc + 3) / 4
         for (; kt < ksteps; ++kt) k_step(kt, std::false_type{});
 
         // ---- the next tile: its first two K steps go into slots 1 and 2 now (every wave is past the last barrier of
-        // the K loop, behind which nothing reads the ring any more); slot 0 holds the epilogue's staging
+        // the K loop, behind which nothing reads the ring any more); slot 0 holds the epilogue's staging.  Not so when
+        // this place has no tile in the super-tile(s) that follow: a workgroup that went straight on would from then
+        // on run a tile ahead of the rest of its XCD -- on another super-tile, whose operand slabs it would pull through
+        // L2 alone (measured on N = 13824, 54 tile columns: half again as many bytes from beyond L2).  It sits those
+        // super-tiles out, a tile's time each, and starts its next tile when the XCD's other workgroups do.
         const int m0 = tile_m * BM, n0 = tile_n * BN;
         int next_m = -1, next_n = 0;
-        const bool more = next_tile(seq, next_m, next_n);
+        const bool more = next_tile(seq, next_m, next_n, skipped);
+        const bool prefetch = more && skipped == 0;
         Side next_side = {};
         bool next_reverse = false;
-        if (more) {
+        auto request_next = [&]() __attribute__((always_inline)) {
             sources(src, next_m, next_n);
             next_reverse = tmap.contig && (seq & 1) != 0;
             next_side = side_fetch(next_m, next_n);
             issue(src, next_reverse, 0, 1);
             if (ksteps > 1) issue(src, next_reverse, 1, 2);
-        }
+        };
+        if (prefetch) request_next();
 
         // ---- fp16 epilogue of this tile.  The prefetched steps have to be in LDS, for every wave, before the next tile
         // reads them.  Loads and stores share one counter, so the wave waits for its loads before its first store --
         // by then they have had the first strip's conversion to arrive -- and the barrier below publishes them.
         auto prefetch_landed = [&] {
-            if (more) __builtin_amdgcn_s_waitcnt(waitcnt_imm(0, 15));
+            if (prefetch) __builtin_amdgcn_s_waitcnt(waitcnt_imm(0, 15));
         };
         if (n0 + wn0 < N && m0 + wm0 < M) /* the same for the whole wave */
             bf6_epilogue<Cfg, STREAM_OUT, TAIL>(acc, side, lds + wave * Cfg::kStagingBytes, lane, m0 + wm0, n0 + wn0, out, ldo, M, N, tail,
@@ -534,6 +545,12 @@ __global__ __launch_bounds__(Cfg::kWaves * 64, (Cfg::kWaves * Cfg::kOcc + 3) / 4
         else
             prefetch_landed();
         if (!more) break;
+        if (!prefetch) {
+            const uint64_t now = wall_clock64(), until = now + static_cast<uint64_t>(skipped) * (now - tile_started);
+            while (wall_clock64() < until) __builtin_amdgcn_s_sleep(32);
+            request_next();
+            __builtin_amdgcn_s_waitcnt(waitcnt_imm(0, 15));
+        }
         __builtin_amdgcn_s_waitcnt(waitcnt_imm(63, 0)); /* the staging reads of this wave are done */
         lds_barrier();
         side_publish(next_side);
