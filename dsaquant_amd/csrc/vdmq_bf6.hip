@@ -78,7 +78,6 @@ struct Bf6Cfg {
     static_assert(kLdsBytes * kOcc <= 160 * 1024, "the CU's LDS holds OCC workgroups");
 };
 using Bf6Big = Bf6Cfg<256, 256, 2, 4, 3, 1>;
-constexpr int kValuPerMfma = 3; /* address arithmetic and operand assembly spread between the MFMAs */
 
 struct Bf6TileMap {
     int tiles_m, tiles_n, super_n, total_super;
@@ -105,20 +104,93 @@ struct Bf6TileMap {
     return r;
 }
 
-template <int NDS, int NVMEM, int I = 0>
-__device__ __forceinline__ void schedule_region() {
-    if constexpr (I < 8) { /* the 4 x 2 MFMAs of a k-block */
-        __builtin_amdgcn_sched_group_barrier(0x008, 1, 0); /* MFMA */
-        if constexpr (2 * I < NDS) __builtin_amdgcn_sched_group_barrier(0x100, 2, 0); /* DS reads */
-        if constexpr (I < NVMEM) __builtin_amdgcn_sched_group_barrier(0x020, 1, 0); /* direct-to-LDS load */
-        __builtin_amdgcn_sched_group_barrier(0x002, kValuPerMfma, 0); /* VALU */
-        schedule_region<NDS, NVMEM, I + 1>();
-    } else {
-        __builtin_amdgcn_sched_barrier(0);
-    }
-}
-
 #if defined(__HIP_DEVICE_COMPILE__) /* (the host pass does not know the buffer builtins) */
+// The K loop of one tile, shared by the two kernels.
+//
+// One K step = two k-blocks of eight MFMAs each (the wave's 2 x 4 MFMA tiles).  Fragment f of a k-block (0: weight
+// rows 0-31, 1...4: the four token row-blocks, 5: weight rows 32-63 -- the order in which the MFMAs first need them)
+// is read from LDS behind the f-th MFMA of the k-block before it.  The six global -> LDS loads of a stage go out
+// three per k-block, behind every other MFMA: loads 3...5 of stage kt + 2 in the first k-block of step kt, loads
+// 0...2 of stage kt + 3 in its second one, each into a ring slot whose last reader has passed a barrier.  That way
+// the CU's eight waves hand the texture path one load every few cycles; issued together, 48 at a time, they queue
+// up in front of it, and a wave that cannot issue its load cannot issue the MFMAs behind it either (all six behind
+// the k-block's last MFMAs: 6.5 % slower on the 14B shapes).  Direct-to-LDS loads and LDS reads keep their program
+// order -- the compiler sees one LDS and orders every such pair -- so the order written here, pinned per MFMA by
+// sched_barrier, is the order of the instruction stream; scheduling hints alone cannot move a load in front of an
+// LDS read that precedes it in the source.
+//
+// On entry stages 0, 1 and 2 of the tile are requested (0 and 1 landed and published), `cur` is the ring slot of
+// stage 0 and wfa / xfa hold its first k-block's fragments.  `ksteps` K steps are worked; stage t lies at K step
+// ksteps - 1 - t of the operands if `k_reverse`, else at t.
+template <class Cfg>
+struct Bf6KLoop {
+    static constexpr int NI = Cfg::NI, MI = Cfg::MI, S = Cfg::S, kLoads = Cfg::kLoads, kWaves = Cfg::kWaves, BN = Cfg::BN;
+    static_assert(NI == 2 && MI == 4 && kLoads == 6 && S == 3, "the schedule is written for this shape");
+    uint8_t *lds;
+    const __amdgpu_buffer_rsrc_t (&src)[kLoads];
+    const uint32_t (&lane_off)[kLoads];
+    int wave, wn, wm;
+    uint32_t la, lb;
+    int ksteps;
+    bool k_reverse;
+
+    __device__ __forceinline__ v8i frag_at(const uint8_t *stage, int f, int kb) const {
+        const int rb = f == 0 ? wn * NI : (f == NI + MI - 1 ? wn * NI + 1 : BN / 32 + wm * MI + f - 1);
+        return ld_frag(stage + (rb * 2 + kb) * kBlkBytes, la, lb);
+    }
+    static __device__ __forceinline__ void put(v8i (&wf)[NI], v8i (&xf)[MI], int f, const v8i &v) {
+        if (f == 0) wf[0] = v;
+        else if (f == NI + MI - 1) wf[1] = v;
+        else xf[f - 1] = v;
+    }
+    __device__ __forceinline__ void load_one(int i, int stage_no, int slot) const {
+        const int kpos = k_reverse ? ksteps - 1 - stage_no : stage_no;
+        __builtin_amdgcn_raw_ptr_buffer_load_lds(src[i], VDMQ_LDS_PTR(lds + slot * Cfg::kStageBytes + (i * kWaves + wave) * 1024), 16, lane_off[i],
+                                                 kpos * (KS / 64) * kBf6PanelKb, 0, 0);
+    }
+    // LOAD_B / LOAD_A: this step issues the second half of stage kt + 2 / the first half of stage kt + 3; READ_NEXT: a
+    // step follows; YOUNGER: stage kt + 2 exists, i.e. six loads may stay in flight across the barrier (-1: look at kt)
+    template <bool LOAD_B, bool LOAD_A, bool READ_NEXT, int YOUNGER>
+    __device__ __forceinline__ void step(int kt, int &cur, v16f (&acc)[NI][MI], v8i (&wfa)[NI], v8i (&xfa)[MI], v8i (&wfb)[NI],
+                                         v8i (&xfb)[MI]) const {
+        const uint8_t *stage = lds + cur * Cfg::kStageBytes;
+        const int nxt = cur + 1 == S ? 0 : cur + 1, prv = cur == 0 ? S - 1 : cur - 1;
+#pragma unroll
+        for (int i = 0; i < NI * MI; ++i) {
+            acc[i / MI][i % MI] = __builtin_amdgcn_mfma_scale_f32_32x32x64_f8f6f4(wfa[i / MI], xfa[i % MI], acc[i / MI][i % MI], 3, 3, 0, 0, 0, 0); /* bf6 x bf6, no scaling */
+            if (i < NI + MI) put(wfb, xfb, i, frag_at(stage, i, 1));
+            if (LOAD_B && (i & 1) && i / 2 < kLoads / 2) load_one(kLoads / 2 + i / 2, kt + 2, prv);
+            __builtin_amdgcn_sched_barrier(0);
+        }
+        // one barrier per step: behind it stage kt + 1 is complete for every wave (the stage after it may still be on
+        // its way: six loads), and nobody reads slot `cur` any more
+        if (YOUNGER > 0 || (YOUNGER < 0 && kt + 2 < ksteps))
+            __builtin_amdgcn_s_waitcnt(waitcnt_imm(kLoads, 0));
+        else
+            __builtin_amdgcn_s_waitcnt(waitcnt_imm(0, 0));
+        lds_barrier();
+#pragma unroll
+        for (int i = 0; i < NI * MI; ++i) {
+            acc[i / MI][i % MI] = __builtin_amdgcn_mfma_scale_f32_32x32x64_f8f6f4(wfb[i / MI], xfb[i % MI], acc[i / MI][i % MI], 3, 3, 0, 0, 0, 0);
+            if (READ_NEXT && i < NI + MI) put(wfa, xfa, i, frag_at(lds + nxt * Cfg::kStageBytes, i, 0));
+            if (LOAD_A && (i & 1) && i / 2 < kLoads / 2) load_one(i / 2, kt + 3, cur);
+            __builtin_amdgcn_sched_barrier(0);
+        }
+        cur = nxt;
+    }
+    __device__ __forceinline__ void run(int &cur, v16f (&acc)[NI][MI], v8i (&wfa)[NI], v8i (&xfa)[MI], v8i (&wfb)[NI], v8i (&xfb)[MI]) const {
+        int kt = 0;
+        if (ksteps > S) {
+            step<false, true, true, 1>(0, cur, acc, wfa, xfa, wfb, xfb);
+            for (kt = 1; kt + S < ksteps; ++kt) step<true, true, true, 1>(kt, cur, acc, wfa, xfa, wfb, xfb);
+            step<true, false, true, 1>(kt, cur, acc, wfa, xfa, wfb, xfb);
+            ++kt;
+        }
+        for (; kt + 1 < ksteps; ++kt) step<false, false, true, -1>(kt, cur, acc, wfa, xfa, wfb, xfb);
+        step<false, false, false, 0>(kt, cur, acc, wfa, xfa, wfb, xfb);
+    }
+};
+
 // fp16 epilogue of one wave's 128 x 64 corner of a tile, as in the int8 kernel:
 // out = fp16(float(acc) * (float(as) * float(ws))) (+ bias in fp16) [then residual + y * gate]; one 32-row strip at
 // a time is transposed through the wave's staging area so that rows leave as whole 128-byte lines.  `side` holds the
@@ -268,13 +340,6 @@ __global__ __launch_bounds__(Cfg::kWaves * 64, (Cfg::kWaves * Cfg::kOcc + 3) / 4
             for (int r = 0; r < 16; ++r) acc[ni][mi][r] = 0.f;
     // weight rows are the A operand, token rows the B operand: accumulator register r of a 32 x 32
     // tile holds n = 8 * (r / 4) + 4 * (lane / 32) + r % 4, m = lane % 32
-    auto mma = [&](const v8i (&wf)[NI], const v8i (&xf)[MI]) __attribute__((always_inline)) {
-#pragma unroll
-        for (int ni = 0; ni < NI; ++ni)
-#pragma unroll
-            for (int mi = 0; mi < MI; ++mi)
-                acc[ni][mi] = __builtin_amdgcn_mfma_scale_f32_32x32x64_f8f6f4(wf[ni], xf[mi], acc[ni][mi], 3, 3, 0, 0, 0, 0); /* bf6 x bf6, no scaling */
-    };
     const int ksteps = kblocks / (KS / 64);
     const int m0 = tile_m * BM, n0 = tile_n * BN, wm0 = wm * MI * 32, wn0 = wn * NI * 32;
     uint8_t *side = lds + Cfg::kRingBytes + wave * kSideBytes;
@@ -304,31 +369,8 @@ __global__ __launch_bounds__(Cfg::kWaves * 64, (Cfg::kWaves * Cfg::kOcc + 3) / 4
     v8i wfa[NI], xfa[MI], wfb[NI], xfb[MI];
     read(wfa, xfa, lds, 0);
     int cur = 0;
-    // one stage = two k-blocks; the ring is published by one barrier per stage, placed before the second k-block's MFMAs
-    auto k_step = [&](int kt, auto steady_tag) __attribute__((always_inline)) {
-        constexpr bool STEADY = decltype(steady_tag)::value;
-        const uint8_t *stage = lds + cur * kStageBytes;
-        const int nxt = cur + 1 == S ? 0 : cur + 1;
-        read(wfb, xfb, stage, 1);
-        mma(wfa, xfa);
-        schedule_region<2 * (NI + MI), 0>();
-        if (STEADY)
-            __builtin_amdgcn_s_waitcnt(waitcnt_imm(kLoads * (S - 2), 0));
-        else
-            __builtin_amdgcn_s_waitcnt(waitcnt_imm(0, 0));
-        lds_barrier();
-        if (STEADY || kt + 1 < ksteps) read(wfa, xfa, lds + nxt * kStageBytes, 0);
-        if (STEADY) issue(kt + S, cur);
-        mma(wfb, xfb);
-        if (STEADY)
-            schedule_region<2 * (NI + MI), kLoads>();
-        else
-            schedule_region<2 * (NI + MI), 0>();
-        cur = nxt;
-    };
-    int kt = 0;
-    for (; kt + S < ksteps; ++kt) k_step(kt, std::true_type{});
-    for (; kt < ksteps; ++kt) k_step(kt, std::false_type{});
+    const Bf6KLoop<Cfg> k_loop{lds, src, lane_off, wave, wn, wm, la, lb, ksteps, k_reverse};
+    k_loop.run(cur, acc, wfa, xfa, wfb, xfb);
 
     const int l32 = lane & 31, lh = lane >> 5;
     if (ACC_OUT) {
@@ -451,13 +493,6 @@ __global__ __launch_bounds__(Cfg::kWaves * 64, (Cfg::kWaves * Cfg::kOcc + 3) / 4
         for (int mi = 0; mi < MI; ++mi) xf[mi] = ld_frag(stage + ((BN / 32 + wm * MI + mi) * 2 + kb) * kBlkBytes, la, lb);
     };
     v16f acc[NI][MI];
-    auto mma = [&](const v8i (&wf)[NI], const v8i (&xf)[MI]) __attribute__((always_inline)) {
-#pragma unroll
-        for (int ni = 0; ni < NI; ++ni)
-#pragma unroll
-            for (int mi = 0; mi < MI; ++mi)
-                acc[ni][mi] = __builtin_amdgcn_mfma_scale_f32_32x32x64_f8f6f4(wf[ni], xf[mi], acc[ni][mi], 3, 3, 0, 0, 0, 0);
-    };
 
     int seq = -1, tile_m = -1, tile_n = 0, skipped = 0;
     if (!next_tile(seq, tile_m, tile_n, skipped)) return;
@@ -487,30 +522,8 @@ __global__ __launch_bounds__(Cfg::kWaves * 64, (Cfg::kWaves * Cfg::kOcc + 3) / 4
 #pragma unroll
                 for (int r = 0; r < 16; ++r) acc[ni][mi][r] = 0.f;
         read(wfa, xfa, lds + cur * kStageBytes, 0);
-        auto k_step = [&](int kt, auto steady_tag) __attribute__((always_inline)) {
-            constexpr bool STEADY = decltype(steady_tag)::value;
-            const uint8_t *stage = lds + cur * kStageBytes;
-            const int nxt = cur + 1 == S ? 0 : cur + 1;
-            read(wfb, xfb, stage, 1);
-            mma(wfa, xfa);
-            schedule_region<2 * (NI + MI), 0>();
-            if (STEADY)
-                __builtin_amdgcn_s_waitcnt(waitcnt_imm(kLoads * (S - 2), 0));
-            else
-                __builtin_amdgcn_s_waitcnt(waitcnt_imm(0, 0));
-            lds_barrier();
-            if (STEADY || kt + 1 < ksteps) read(wfa, xfa, lds + nxt * kStageBytes, 0);
-            if (STEADY) issue(src, k_reverse, kt + S, cur);
-            mma(wfb, xfb);
-            if (STEADY)
-                schedule_region<2 * (NI + MI), kLoads>();
-            else
-                schedule_region<2 * (NI + MI), 0>();
-            cur = nxt;
-        };
-        int kt = 0;
-        for (; kt + S < ksteps; ++kt) k_step(kt, std::true_type{});
-        for (; kt < ksteps; ++kt) k_step(kt, std::false_type{});
+        const Bf6KLoop<Cfg> k_loop{lds, src, lane_off, wave, wn, wm, la, lb, ksteps, k_reverse};
+        k_loop.run(cur, acc, wfa, xfa, wfb, xfb);
 
         // ---- the next tile: its first two K steps go into slots 1 and 2 now (every wave is past the last barrier of
         // the K loop, behind which nothing reads the ring any more); slot 0 holds the epilogue's staging.  Not so when
