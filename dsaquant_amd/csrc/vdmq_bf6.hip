@@ -110,7 +110,7 @@ struct Bf6TileMap {
 // One K step = two k-blocks of eight MFMAs each (the wave's 2 x 4 MFMA tiles).  Fragment f of a k-block (0: weight
 // rows 0-31, 1...4: the four token row-blocks, 5: weight rows 32-63 -- the order in which the MFMAs first need them)
 // is read from LDS behind the f-th MFMA of the k-block before it.  The six global -> LDS loads of a stage go out
-// three per k-block, behind every other MFMA: loads 3...5 of stage kt + 2 in the first k-block of step kt, loads
+// three per k-block, behind every other MFMA (kLoadSlots*): loads 3...5 of stage kt + 2 in the first k-block of step kt, loads
 // 0...2 of stage kt + 3 in its second one, each into a ring slot whose last reader has passed a barrier.  That way
 // the CU's eight waves hand the texture path one load every few cycles; issued together, 48 at a time, they queue
 // up in front of it, and a wave that cannot issue its load cannot issue the MFMAs behind it either (all six behind
@@ -126,6 +126,10 @@ template <class Cfg>
 struct Bf6KLoop {
     static constexpr int NI = Cfg::NI, MI = Cfg::MI, S = Cfg::S, kLoads = Cfg::kLoads, kWaves = Cfg::kWaves, BN = Cfg::BN;
     static_assert(NI == 2 && MI == 4 && kLoads == 6 && S == 3, "the schedule is written for this shape");
+    // MFMAs of a k-block (bit i = behind the i-th) that are followed by a load: behind the 2nd, 4th and 6th in the first
+    // k-block, the 3rd, 5th and 7th in the second.  Measured against other triples: a load behind a k-block's first
+    // MFMA (right after the barrier, or the loop's head) costs 2 %, the rest lie within 1 %.
+    static constexpr unsigned kLoadSlotsB = 0x2A, kLoadSlotsA = 0x54;
     uint8_t *lds;
     const __amdgpu_buffer_rsrc_t (&src)[kLoads];
     const uint32_t (&lane_off)[kLoads];
@@ -149,7 +153,8 @@ struct Bf6KLoop {
                                                  kpos * (KS / 64) * kBf6PanelKb, 0, 0);
     }
     // LOAD_B / LOAD_A: this step issues the second half of stage kt + 2 / the first half of stage kt + 3; READ_NEXT: a
-    // step follows; YOUNGER: stage kt + 2 exists, i.e. six loads may stay in flight across the barrier (-1: look at kt)
+    // step follows; YOUNGER: stage kt + 2 exists, i.e. six loads may stay in flight across the barrier (-1: look at kt;
+    // 2: stage kt + 1 is known to have landed, no wait for loads at all)
     template <bool LOAD_B, bool LOAD_A, bool READ_NEXT, int YOUNGER>
     __device__ __forceinline__ void step(int kt, int &cur, v16f (&acc)[NI][MI], v8i (&wfa)[NI], v8i (&xfa)[MI], v8i (&wfb)[NI],
                                          v8i (&xfb)[MI]) const {
@@ -159,12 +164,14 @@ struct Bf6KLoop {
         for (int i = 0; i < NI * MI; ++i) {
             acc[i / MI][i % MI] = __builtin_amdgcn_mfma_scale_f32_32x32x64_f8f6f4(wfa[i / MI], xfa[i % MI], acc[i / MI][i % MI], 3, 3, 0, 0, 0, 0); /* bf6 x bf6, no scaling */
             if (i < NI + MI) put(wfb, xfb, i, frag_at(stage, i, 1));
-            if (LOAD_B && (i & 1) && i / 2 < kLoads / 2) load_one(kLoads / 2 + i / 2, kt + 2, prv);
+            if (LOAD_B && ((kLoadSlotsB >> i) & 1)) load_one(kLoads / 2 + __builtin_popcount(kLoadSlotsB & ((1 << i) - 1)), kt + 2, prv);
             __builtin_amdgcn_sched_barrier(0);
         }
         // one barrier per step: behind it stage kt + 1 is complete for every wave (the stage after it may still be on
         // its way: six loads), and nobody reads slot `cur` any more
-        if (YOUNGER > 0 || (YOUNGER < 0 && kt + 2 < ksteps))
+        if (YOUNGER == 2)
+            __builtin_amdgcn_s_waitcnt(waitcnt_imm(63, 0));
+        else if (YOUNGER > 0 || (YOUNGER < 0 && kt + 2 < ksteps))
             __builtin_amdgcn_s_waitcnt(waitcnt_imm(kLoads, 0));
         else
             __builtin_amdgcn_s_waitcnt(waitcnt_imm(0, 0));
@@ -173,15 +180,20 @@ struct Bf6KLoop {
         for (int i = 0; i < NI * MI; ++i) {
             acc[i / MI][i % MI] = __builtin_amdgcn_mfma_scale_f32_32x32x64_f8f6f4(wfb[i / MI], xfb[i % MI], acc[i / MI][i % MI], 3, 3, 0, 0, 0, 0);
             if (READ_NEXT && i < NI + MI) put(wfa, xfa, i, frag_at(lds + nxt * Cfg::kStageBytes, i, 0));
-            if (LOAD_A && (i & 1) && i / 2 < kLoads / 2) load_one(i / 2, kt + 3, cur);
+            if (LOAD_A && ((kLoadSlotsA >> i) & 1)) load_one(__builtin_popcount(kLoadSlotsA & ((1 << i) - 1)), kt + 3, cur);
             __builtin_amdgcn_sched_barrier(0);
         }
         cur = nxt;
     }
+    // TWO_LANDED: stage 1 has landed too (the kernel that walks tiles requests a tile's first stages under the epilogue
+    // of the tile before and waits for them there).  Step 0 then waits for no load: the one counter that tracks
+    // loads also tracks the output stores issued in between, and waiting for "all but the last six" would wait
+    // for every one of those.
+    template <bool TWO_LANDED>
     __device__ __forceinline__ void run(int &cur, v16f (&acc)[NI][MI], v8i (&wfa)[NI], v8i (&xfa)[MI], v8i (&wfb)[NI], v8i (&xfb)[MI]) const {
         int kt = 0;
         if (ksteps > S) {
-            step<false, true, true, 1>(0, cur, acc, wfa, xfa, wfb, xfb);
+            step<false, true, true, TWO_LANDED ? 2 : 1>(0, cur, acc, wfa, xfa, wfb, xfb);
             for (kt = 1; kt + S < ksteps; ++kt) step<true, true, true, 1>(kt, cur, acc, wfa, xfa, wfb, xfb);
             step<true, false, true, 1>(kt, cur, acc, wfa, xfa, wfb, xfb);
             ++kt;
@@ -370,7 +382,7 @@ __global__ __launch_bounds__(Cfg::kWaves * 64, (Cfg::kWaves * Cfg::kOcc + 3) / 4
     read(wfa, xfa, lds, 0);
     int cur = 0;
     const Bf6KLoop<Cfg> k_loop{lds, src, lane_off, wave, wn, wm, la, lb, ksteps, k_reverse};
-    k_loop.run(cur, acc, wfa, xfa, wfb, xfb);
+    k_loop.template run<false>(cur, acc, wfa, xfa, wfb, xfb);
 
     const int l32 = lane & 31, lh = lane >> 5;
     if (ACC_OUT) {
@@ -504,8 +516,8 @@ __global__ __launch_bounds__(Cfg::kWaves * 64, (Cfg::kWaves * Cfg::kOcc + 3) / 4
 #pragma unroll
         for (int s = 0; s < S; ++s)
             if (s < ksteps) issue(src, k_reverse, s, s);
-        if (ksteps >= S)
-            __builtin_amdgcn_s_waitcnt(waitcnt_imm(kLoads * (S - 1), 15));
+        if (ksteps >= S) /* stages 0 and 1, as for every later tile (Bf6KLoop::run<true>) */
+            __builtin_amdgcn_s_waitcnt(waitcnt_imm(kLoads * (S - 2), 15));
         else
             __builtin_amdgcn_s_waitcnt(waitcnt_imm(0, 15));
         lds_barrier();
@@ -523,7 +535,7 @@ __global__ __launch_bounds__(Cfg::kWaves * 64, (Cfg::kWaves * Cfg::kOcc + 3) / 4
                 for (int r = 0; r < 16; ++r) acc[ni][mi][r] = 0.f;
         read(wfa, xfa, lds + cur * kStageBytes, 0);
         const Bf6KLoop<Cfg> k_loop{lds, src, lane_off, wave, wn, wm, la, lb, ksteps, k_reverse};
-        k_loop.run(cur, acc, wfa, xfa, wfb, xfb);
+        k_loop.template run<false>(cur, acc, wfa, xfa, wfb, xfb);
 
         // ---- the next tile: its first two K steps go into slots 1 and 2 now (every wave is past the last barrier of
         // the K loop, behind which nothing reads the ring any more); slot 0 holds the epilogue's staging.  Not so when
