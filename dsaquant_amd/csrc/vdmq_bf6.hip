@@ -751,16 +751,17 @@ int launch_bf6_cfg(const uint8_t *xblocks, const __half *ascale, const uint8_t *
     // sequence -- where the hardware dispatcher would refill a CU as soon as it is free: it pays when no XCD has many
     // partly empty super-tiles (a ragged last row of super-tiles spread over an XCD's run costs whole rounds:
     // measured -16 % on M = 27280, N = 14336, where that takes a third more rounds), i.e. when its rounds are within 15 % of
-    // the busiest XCD's tiles / places (M = 32760, N = 4608: 10 rounds for 9, still +4 %).
+    // the busiest XCD's tiles / places (M = 32760, N = 4608: 10 rounds for 9, still +4 %).  Every fp16 output mode has
+    // it (with the gated residual tail: 249 registers, +3...4 % on the 14B and 5B output projections).
     const int64_t all_tiles = static_cast<int64_t>(tm.tiles_m) * tm.tiles_n;
     const int64_t busiest = tm.contig || best_load == 0 ? ceil_div(all_tiles, kXcds) : best_load;
-    const bool persistent = which < 2 && /* with the gated residual tail it needs more registers than there are: 10 % slower */
-                             static_cast<int64_t>(rounds) * 100 <= ceil_div(busiest, per) * 115;
+    const bool persistent = which != 2 && static_cast<int64_t>(rounds) * 100 <= ceil_div(busiest, per) * 115;
     if (persistent) {
         using PKernel = void (*)(const uint8_t *, const uint8_t *, const __half *, const __half *, const __half *, __half *, int, int, int,
                                  int64_t, Bf6TileMap, GemmTail);
-        const PKernel pk[2] = {gemm_bf6_persistent_kernel<Cfg, 0>, gemm_bf6_persistent_kernel<Cfg, 1>};
-        static bool pattr[kMaxDevices][2] = {};
+        const PKernel pk[5] = {gemm_bf6_persistent_kernel<Cfg, 0>, gemm_bf6_persistent_kernel<Cfg, 1>, nullptr, gemm_bf6_persistent_kernel<Cfg, 3>,
+                               gemm_bf6_persistent_kernel<Cfg, 4>};
+        static bool pattr[kMaxDevices][5] = {};
         if (!pattr[dev][which]) {
             hipError_t e = hipFuncSetAttribute(reinterpret_cast<const void *>(pk[which]), hipFuncAttributeMaxDynamicSharedMemorySize,
                                                Cfg::kLdsBytes);
