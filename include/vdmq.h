@@ -232,9 +232,10 @@ int vdmq_linear_w4a4_noalloc(const void *x, int64_t M, int64_t K, int64_t ldx, f
  * instead of native rows: same scales, same integers; K <= 16384. */
 int64_t vdmq_bf6_bytes(int64_t rows, int64_t K);
 /* 1 when the bf6 path is the faster one for an fp16 linear of this size (quantizer + GEMM, measured on MI355X), 0
- * otherwise: its kernel has one tile shape, 256 x 256, so it wants at least 512 output tiles, or 128 when K >= 4096
- * lets the K loop outweigh a tile's prologue and epilogue.  A host that keeps both weight forms asks this per call;
- * the results are the same bits either way.  No counterpart in the reference (it has one matrix path). */
+ * otherwise: its kernel has one tile shape, 256 x 256, so it wants at least 512 output tiles -- or, when K >= 3072
+ * lets the K loop outweigh a tile's prologue and epilogue, N >= 5120 or at least 96 tiles.  A host that keeps both
+ * weight forms asks this per call; the results are the same bits either way.  No counterpart in the reference (it
+ * has one matrix path). */
 int vdmq_bf6_pays(int64_t M, int64_t N, int64_t K);
 int vdmq_quantize_act_bf6(const void *x, int64_t M, int64_t K, int64_t ldx, float clip, int act, void *xblocks, void *scale_h,
                           vdmq_stream_t stream);

@@ -473,6 +473,8 @@ def test_library_says_where_the_fp6_path_pays():
     assert pays(75600, 15360, 5120) and pays(75600, 5120, 13824) and pays(32760, 1536, 1536) and pays(27280, 3072, 14336)
     assert pays(2048, 5120, 5120)            # 160 tiles, long K
     assert not pays(4096, 4608, 1536)        # config 0: 288 tiles, short K
-    assert not pays(4096, 1536, 8960)        # 96 tiles
-    assert not pays(512, 10240, 5120)        # the skinny cross-attention K/V case: 80 tiles
+    assert pays(4096, 1536, 8960)            # 96 tiles, long K
+    assert not pays(2048, 1536, 8960)        # 48 tiles, narrow N
+    assert pays(512, 10240, 5120)            # the skinny cross-attention K/V case of the 14B model: wide N, long K
+    assert not pays(512, 3072, 1536)         # the same of the 1.3B model
     assert not pays(0, 128, 64) and not pays(-1, 128, 64)
