@@ -93,17 +93,19 @@ def test_full_size_linear(cfg, name, M, K, N, calls, expect, path):
         torch.cuda.empty_cache()
 
 
-def test_persistent_bf6_kernel_with_one_two_and_three_k_steps():
+def test_persistent_bf6_kernel_with_one_to_six_k_steps():
     """The bf6 kernel that walks tiles prefetches the next tile's first two K steps under the epilogue and has
-    branches for K of one, two and three steps (K = 64/128, 256, 384): 65 x 16 tiles, four per workgroup and more,
-    accumulators against the int8 path and, for a slice, the integer product on the CPU."""
+    branches for K of one, two and three steps (K = 64/128, 256, 384); its K loop issues a stage's loads in two halves
+    and runs through its step variants in a fixed order that four, five and six steps (K = 512, 640, 768) exercise from
+    the first to the last: 65 x 16 tiles, four per workgroup and more, outputs against the int8 path and, for a slice,
+    the oracle."""
     from dsaquant_amd import _lib
     from dsaquant_amd.kernels import vdm_w4a4 as v
 
     assert v.is_available(), v.load_error()
     rng = np.random.default_rng(5)
     M, N = 16400, 4096
-    for K in (64, 128, 256, 384):
+    for K in (64, 128, 256, 384, 512, 640, 768):
         qw = rng.integers(-8, 8, (N, K), dtype=np.int8)
         x = O.synth_linear(M, K, 128, seed=K)[0]
         _, _, ws, bias = O.synth_linear(1, 64, N, seed=K + 1)
