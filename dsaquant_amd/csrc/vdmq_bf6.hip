@@ -755,7 +755,11 @@ int launch_bf6_cfg(const uint8_t *xblocks, const __half *ascale, const uint8_t *
     // it (with the gated residual tail: 249 registers, +3...4 % on the 14B and 5B output projections).
     const int64_t all_tiles = static_cast<int64_t>(tm.tiles_m) * tm.tiles_n;
     const int64_t busiest = tm.contig || best_load == 0 ? ceil_div(all_tiles, kXcds) : best_load;
-    const bool persistent = which != 2 && static_cast<int64_t>(rounds) * 100 <= ceil_div(busiest, per) * 115;
+    // (one workgroup per CU position: only where the device has as many CUs as the kernel has positions; elsewhere the
+    // hardware dispatcher places the one-tile workgroups)
+    static int cu_count[kMaxDevices] = {};
+    if (cu_count[dev] == 0 && hipDeviceGetAttribute(&cu_count[dev], hipDeviceAttributeMultiprocessorCount, dev) != hipSuccess) cu_count[dev] = -1;
+    const bool persistent = which != 2 && cu_count[dev] == kXcds * per && static_cast<int64_t>(rounds) * 100 <= ceil_div(busiest, per) * 115;
     if (persistent) {
         using PKernel = void (*)(const uint8_t *, const uint8_t *, const __half *, const __half *, const __half *, __half *, int, int, int,
                                  int64_t, Bf6TileMap, GemmTail);
