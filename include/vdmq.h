@@ -171,7 +171,7 @@ typedef struct vdmq_gemm_launch_info {
     int tile_m, tile_n;         /* output tile of one workgroup: token rows x channels */
     int group_m, group_n;       /* super-tile, in tiles */
     int contiguous_runs;        /* 1: each XCD walks one contiguous run of super-tiles, K direction alternating */
-    int split_k_tiles;          /* tiles of the last, partly filled round whose K range was split over idle CUs */
+    int split_k_tiles;          /* always 0: no launch splits the K range of its tiles (kept for the layout of the struct) */
     int64_t workgroups;         /* grid size */
 } vdmq_gemm_launch_info;
 int vdmq_last_gemm_launch(vdmq_gemm_launch_info *info);
