@@ -234,7 +234,11 @@ struct Bf6Scratch { /* LDS of one workgroup */
 // row has gone to the transpose buffer and its registers are free: a workgroup that walks several
 // row groups loads the next row's chunk there, so those loads overlap the rest of this row's
 // conversion.  `phase` counts the groups this workgroup has staged (it picks the staging copy).
-constexpr bool bf6_walks(int nch) { return nch >= 17; } /* rows longer than 8192: one workgroup per CU, which walks row groups */
+// Which row lengths take the walking form (a resident grid whose workgroups take row groups in turn, the next group's
+// loads in flight under this group's conversion): rows longer than 8192, which leave room for one workgroup per CU
+// only, and rows of at most 2048, whose groups are too little work for a workgroup of their own (K = 512...1536:
+// +8...17 % at 32760 and 75600 rows; K = 3072: +2.5 % / -4 %; K = 4096: -6 %).
+constexpr bool bf6_walks(int nch) { return nch >= 17 || nch <= 4; }
 struct NoRefill {
     __device__ __forceinline__ void operator()(int) const {}
 };
