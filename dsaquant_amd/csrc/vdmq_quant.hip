@@ -215,6 +215,7 @@ __device__ __forceinline__ void quantize_held_row(const u32x4 (&v)[NCH], int lan
 // so the conversion is exact -- into the string.  Rows of the last row-block beyond M stay unwritten
 // (the GEMM never stores them); K is padded to 128 with zeros.
 typedef _Float16 f16x32 __attribute__((ext_vector_type(32)));
+typedef float f32x16 __attribute__((ext_vector_type(16)));
 typedef unsigned int u32x6 __attribute__((ext_vector_type(6)));
 typedef unsigned int u32x2 __attribute__((ext_vector_type(2)));
 constexpr int kBf6Rows = 8;                      /* rows (= waves) per workgroup of the bf6 quantizers */
@@ -245,7 +246,7 @@ struct NoRefill {
 template <int NCH, class Refill>
 __device__ __forceinline__ void quantize_held_row_bf6(u32x4 (&v)[NCH], int lane, int wave, int64_t row0, bool valid, int M, int Kb,
                                                       float clip, uint8_t *__restrict__ blocks, __half *__restrict__ scale_h,
-                                                      Bf6Scratch &lds, int &phase, Refill &&refill) {
+                                                      bool stream_out, Bf6Scratch &lds, int &phase, Refill &&refill) {
     uint32_t m2 = 0;
 #pragma unroll
     for (int c = 0; c < NCH; ++c) m2 = absmax_bits(v[c], m2);
@@ -290,19 +291,25 @@ __device__ __forceinline__ void quantize_held_row_bf6(u32x4 (&v)[NCH], int lane,
         u32x4 tr[4];
 #pragma unroll
         for (int u = 0; u < 4; ++u) tr[u] = *reinterpret_cast<const u32x4 *>(tbuf + lane * 64 + u * 16 + (lane >> 2) * 16);
-        f16x32 q; /* this lane's 32 consecutive k: 2048 g + 32 lane ... */
+        // this lane's 32 consecutive k, 2048 g + 32 lane ..., become one 192-bit string
+        u32x6 str;
         if (fast_u) {
+            // the conversion from fp32 takes the even elements from one operand and the odd ones from the other:
+            // the low and high halves of the words as they lie
+            f32x16 even, odd;
 #pragma unroll
             for (int u = 0; u < 4; ++u) {
                 const uint32_t w[4] = {tr[u].x, tr[u].y, tr[u].z, tr[u].w};
 #pragma unroll
                 for (int i = 0; i < 4; ++i) {
                     const f16x2 h = __builtin_bit_cast(f16x2, w[i]);
-                    q[u * 8 + i * 2] = static_cast<_Float16>(__builtin_rintf(__builtin_amdgcn_fmed3f(__builtin_fmaf(static_cast<float>(h[0]), rscale, 0.0f), -8.0f, 7.0f)));
-                    q[u * 8 + i * 2 + 1] = static_cast<_Float16>(__builtin_rintf(__builtin_amdgcn_fmed3f(__builtin_fmaf(static_cast<float>(h[1]), rscale, 0.0f), -8.0f, 7.0f)));
+                    even[u * 4 + i] = __builtin_rintf(__builtin_amdgcn_fmed3f(__builtin_fmaf(static_cast<float>(h[0]), rscale, 0.0f), -8.0f, 7.0f));
+                    odd[u * 4 + i] = __builtin_rintf(__builtin_amdgcn_fmed3f(__builtin_fmaf(static_cast<float>(h[1]), rscale, 0.0f), -8.0f, 7.0f));
                 }
             }
+            str = __builtin_amdgcn_cvt_scalef32_2xpk16_bf6_f32(even, odd, 1.0f);
         } else {
+            f16x32 q;
 #pragma unroll
             for (int u = 0; u < 4; ++u) {
                 const uint32_t w[4] = {tr[u].x, tr[u].y, tr[u].z, tr[u].w};
@@ -316,8 +323,8 @@ __device__ __forceinline__ void quantize_held_row_bf6(u32x4 (&v)[NCH], int lane,
                     }
                 }
             }
+            str = __builtin_amdgcn_cvt_scalef32_pk32_bf6_f16(q, 1.0f);
         }
-        const u32x6 str = __builtin_amdgcn_cvt_scalef32_pk32_bf6_f16(q, 1.0f);
         // per-lane stores would scatter 16-byte pieces over 64 cache lines per instruction (measured: 2x
         // slower than the HBM-bound int4 quantizer): collect the workgroup's strings in LDS instead -- its
         // eight rows are one panel, whose 128-byte and 64-byte runs of one k-block are adjacent in memory
@@ -329,10 +336,20 @@ __device__ __forceinline__ void quantize_held_row_bf6(u32x4 (&v)[NCH], int lane,
         const int k0 = 2048 * g + 32 * sidx;
         if (k0 < Kb && grow < M) {
             const int kb = k0 >> 6, h = (k0 >> 5) & 1;
-            *reinterpret_cast<u32x4 *>(blocks + bf6_piece(grow, kb, h, false, kblocks)) =
-                *reinterpret_cast<const u32x4 *>(lds.part_a[copy][srow] + sidx * 16);
-            *reinterpret_cast<u32x2 *>(blocks + bf6_piece(grow, kb, h, true, kblocks)) =
-                *reinterpret_cast<const u32x2 *>(lds.part_b[copy][srow] + sidx * 8);
+            const u32x4 part_a = *reinterpret_cast<const u32x4 *>(lds.part_a[copy][srow] + sidx * 16);
+            const u32x2 part_b = *reinterpret_cast<const u32x2 *>(lds.part_b[copy][srow] + sidx * 8);
+            u32x4 *dst_a = reinterpret_cast<u32x4 *>(blocks + bf6_piece(grow, kb, h, false, kblocks));
+            u32x2 *dst_b = reinterpret_cast<u32x2 *>(blocks + bf6_piece(grow, kb, h, true, kblocks));
+            if (stream_out) { /* the same for every thread of the launch */
+                // (the empty statements keep the compiler from merging the two branches into plain stores)
+                asm volatile("" ::: "memory");
+                __builtin_nontemporal_store(part_a, dst_a);
+                __builtin_nontemporal_store(part_b, dst_b);
+                asm volatile("" ::: "memory");
+            } else {
+                *dst_a = part_a;
+                *dst_b = part_b;
+            }
         }
     }
 }
@@ -348,7 +365,7 @@ __device__ __forceinline__ void quantize_held_row_bf6(u32x4 (&v)[NCH], int lane,
 template <int NCH, bool STREAM_OUT, int ACT, int FMT>
 __global__ __launch_bounds__((FMT == 1 ? kBf6Rows : kRowsPerBlock) * kWaveSize) void quantize_rows_kernel(
     const __half *__restrict__ x, int64_t ldx, int M, int K, int Kp, float clip, uint8_t *__restrict__ qact,
-    __half *__restrict__ scale_h) {
+    __half *__restrict__ scale_h, int stream_bf6) {
     constexpr int ROWS = FMT == 1 ? kBf6Rows : kRowsPerBlock;
     const int lane = threadIdx.x & (kWaveSize - 1), wave = threadIdx.x >> 6;
     if constexpr (FMT == 1) {
@@ -378,7 +395,7 @@ __global__ __launch_bounds__((FMT == 1 ? kBf6Rows : kRowsPerBlock) * kWaveSize) 
             }
             const int64_t row0 = static_cast<int64_t>(group) * ROWS;
             const u32x4 *next = row_ptr(more ? group + gridDim.x : group);
-            quantize_held_row_bf6<NCH>(v, lane, wave, row0, row0 + wave < M, M, Kp, clip, qact, scale_h, scratch, phase,
+            quantize_held_row_bf6<NCH>(v, lane, wave, row0, row0 + wave < M, M, Kp, clip, qact, scale_h, stream_bf6 != 0, scratch, phase,
                                        [&](int c) {
                                            if constexpr (bf6_walks(NCH))
                                                if (more) v[c] = load(next, c);
@@ -436,7 +453,7 @@ template <int NCH, int LNMODE, bool EMIT_H, int FMT>
 __global__ __launch_bounds__((FMT == 1 ? kBf6Rows : kRowsPerBlock) * kWaveSize) void ln_quantize_rows_kernel(
     const __half *__restrict__ x, int64_t ldx, int M, int K, int Kp, float eps, const __half *__restrict__ va,
     const __half *__restrict__ vb, int64_t ldv, int rows_per_vec, float clip, uint8_t *__restrict__ qact,
-    __half *__restrict__ scale_h, __half *__restrict__ h_out, int64_t ldh) {
+    __half *__restrict__ scale_h, __half *__restrict__ h_out, int64_t ldh, int stream_bf6) {
     constexpr int ROWS = FMT == 1 ? kBf6Rows : kRowsPerBlock;
     const int lane = threadIdx.x & (kWaveSize - 1), wave = threadIdx.x >> 6;
     const int64_t row0 = static_cast<int64_t>(blockIdx.x) * ROWS;
@@ -532,7 +549,7 @@ __global__ __launch_bounds__((FMT == 1 ? kBf6Rows : kRowsPerBlock) * kWaveSize) 
     if (FMT == 1) {
         __shared__ __attribute__((aligned(16))) Bf6Scratch scratch;
         int phase = 0;
-        quantize_held_row_bf6<NCH>(v, lane, wave, row0, valid, M, Kp, clip, qact, scale_h, scratch, phase, NoRefill{});
+        quantize_held_row_bf6<NCH>(v, lane, wave, row0, valid, M, Kp, clip, qact, scale_h, stream_bf6 != 0, scratch, phase, NoRefill{});
     } else {
         quantize_held_row<NCH, false>(v, lane, row, Kp, clip, qact, scale_h);
     }
@@ -589,6 +606,12 @@ __global__ __launch_bounds__(256) void quantize_given_scale_kernel(const __half 
 }
 
 constexpr int64_t kStreamOutBytes = int64_t(224) << 20; /* outputs larger than this bypass the caches */
+// The same for the bf6 blocks, judged by the quantizer and the GEMM that reads its output together: streamed stores
+// cost the GEMM the part of its operand that plain stores leave in the Infinity Cache (38 MB and 63 MB of blocks:
+// the pair 3 % and 2 % slower), and spare it the wait for the dirty lines of a large one (220 MB, 290 MB, 780 MB:
+// the pair 3 %, 0.7 % and 0.7 % faster).
+constexpr int64_t kStreamOutBytesBf6 = int64_t(128) << 20;
+int stream_bf6(int64_t M, int64_t K) { return bf6_bytes(M, K) > kStreamOutBytesBf6 ? 1 : 0; }
 
 // Workgroups of `kernel` the current device runs at once (CUs x workgroups per CU), or -1.  The answer is
 // kept per device in `cache` (one array per kernel, zero-initialised): the occupancy query costs tens of
@@ -620,14 +643,14 @@ int launch_reg(const __half *x, int64_t M, int64_t K, int64_t ldx, float clip, i
         if (resident <= 0) return fail(VDMQ_ELAUNCH, "quantize_rows_kernel: the occupancy query for the current device failed");
         hipLaunchKernelGGL((quantize_rows_kernel<NCH, false, ACT, 1>), dim3(static_cast<unsigned>(!bf6_walks(NCH) || groups < resident ? groups : resident)),
                            dim3(kBf6Rows * kWaveSize), 0, s, x, ldx, static_cast<int>(M), static_cast<int>(K),
-                           static_cast<int>(bf6_kblocks(K) * 64), clip, qact, scale_h);
+                           static_cast<int>(bf6_kblocks(K) * 64), clip, qact, scale_h, stream_bf6(M, K));
     }
     else if (M * (k_padded(K) / 2) > kStreamOutBytes)
         hipLaunchKernelGGL((quantize_rows_kernel<NCH, true, ACT, 0>), grid, block, 0, s, x, ldx, static_cast<int>(M), static_cast<int>(K),
-                           static_cast<int>(k_padded(K)), clip, qact, scale_h);
+                           static_cast<int>(k_padded(K)), clip, qact, scale_h, 0);
     else
         hipLaunchKernelGGL((quantize_rows_kernel<NCH, false, ACT, 0>), grid, block, 0, s, x, ldx, static_cast<int>(M), static_cast<int>(K),
-                           static_cast<int>(k_padded(K)), clip, qact, scale_h);
+                           static_cast<int>(k_padded(K)), clip, qact, scale_h, 0);
     return check_launch("quantize_rows_kernel");
 }
 
@@ -666,14 +689,15 @@ int launch_ln_reg(const __half *x, int64_t M, int64_t K, int64_t ldx, float eps,
     const dim3 grid(static_cast<unsigned>(ceil_div(M, kRowsPerBlock))), block(kRowsPerBlock * kWaveSize);
     if (h_out != nullptr)
         hipLaunchKernelGGL((ln_quantize_rows_kernel<NCH, LNMODE, true, 0>), grid, block, 0, s, x, ldx, static_cast<int>(M), static_cast<int>(K),
-                           static_cast<int>(k_padded(K)), eps, va, vb, ldv, static_cast<int>(rows_per_vec), clip, qact, scale_h, h_out, ldh);
+                           static_cast<int>(k_padded(K)), eps, va, vb, ldv, static_cast<int>(rows_per_vec), clip, qact, scale_h, h_out, ldh, 0);
     else if (fmt == 1)
         hipLaunchKernelGGL((ln_quantize_rows_kernel<NCH, LNMODE, false, 1>), dim3(static_cast<unsigned>(ceil_div(M, kBf6Rows))),
                            dim3(kBf6Rows * kWaveSize), 0, s, x, ldx, static_cast<int>(M), static_cast<int>(K),
-                           static_cast<int>(bf6_kblocks(K) * 64), eps, va, vb, ldv, static_cast<int>(rows_per_vec), clip, qact, scale_h, h_out, ldh);
+                           static_cast<int>(bf6_kblocks(K) * 64), eps, va, vb, ldv, static_cast<int>(rows_per_vec), clip, qact, scale_h, h_out, ldh,
+                           stream_bf6(M, K));
     else
         hipLaunchKernelGGL((ln_quantize_rows_kernel<NCH, LNMODE, false, 0>), grid, block, 0, s, x, ldx, static_cast<int>(M), static_cast<int>(K),
-                           static_cast<int>(k_padded(K)), eps, va, vb, ldv, static_cast<int>(rows_per_vec), clip, qact, scale_h, h_out, ldh);
+                           static_cast<int>(k_padded(K)), eps, va, vb, ldv, static_cast<int>(rows_per_vec), clip, qact, scale_h, h_out, ldh, 0);
     return check_launch("ln_quantize_rows_kernel");
 }
 
