@@ -156,15 +156,17 @@ class Workload:
 
     def step(self, events=None):
         lib, _lib, M, s = self.lib, self._lib, self.M, self.stream.cuda_stream
+        # events[2 * li] .. [2 * li + 1] bracket layer li's quantizer, [2 * li + 1] .. [2 * li + 2] its GEMM: a GEMM's
+        # end is the next quantizer's start (an event record costs the stream 2...3 us)
+        if events is not None:
+            events[0].record(self.stream)
         for li, L in enumerate(self.layers):
-            if events is not None:
-                events[li][0].record(self.stream)
             if L["bf6"]:
                 _lib.check(lib.vdmq_quantize_act_bf6(L["x"].data_ptr(), M, L["K"], L["K"], 1.0, 0, L["qact"].data_ptr(), L["scale"].data_ptr(), s))
             else:
                 _lib.check(lib.vdmq_quantize_act(L["x"].data_ptr(), M, L["K"], L["K"], 1.0, L["qact"].data_ptr(), L["scale"].data_ptr(), s))
             if events is not None:
-                events[li][1].record(self.stream)
+                events[2 * li + 1].record(self.stream)
             if L["bf6"]:
                 _lib.check(lib.vdmq_gemm_w4a4_bf6(L["qact"].data_ptr(), L["scale"].data_ptr(), L["wq"].data_ptr(), L["ws"].data_ptr(),
                                                   L["bias"].data_ptr(), L["out"].data_ptr(), M, L["N"], L["K"], L["N"], s))
@@ -172,7 +174,7 @@ class Workload:
                 _lib.check(lib.vdmq_gemm_w4a4(L["qact"].data_ptr(), L["scale"].data_ptr(), L["wq"].data_ptr(), L["ws"].data_ptr(),
                                               L["bias"].data_ptr(), L["out"].data_ptr(), _lib.VDMQ_OUT_F16, M, L["N"], L["K"], L["N"], s))
             if events is not None:
-                events[li][2].record(self.stream)
+                events[2 * li + 2].record(self.stream)
             if events is not None and "kernel" not in L:
                 L["kernel"] = {1: "gemm_w4a4_kernel", 2: "gemm_bf6_kernel", 3: "gemm_bf6_persistent_kernel"}[_lib.last_gemm_launch().kernel]
 
@@ -183,7 +185,7 @@ class Workload:
         for _ in range(warmup):
             self.step()
         torch.cuda.synchronize()
-        evs = [[[torch.cuda.Event(enable_timing=True) for _ in range(3)] for _ in self.layers] for _ in range(steps)]
+        evs = [[torch.cuda.Event(enable_timing=True) for _ in range(2 * len(self.layers) + 1)] for _ in range(steps)]
         torch.cuda.synchronize()
         t0 = time.perf_counter()
         for k in range(steps):
@@ -194,8 +196,8 @@ class Workload:
         total_ops = sum(2.0 * M * L["N"] * L["K"] for L in self.layers)
         per_layer, gemm_ms, quant_ms = {}, 0.0, 0.0
         for li, L in enumerate(self.layers):
-            q_ms = statistics.mean(evs[k][li][0].elapsed_time(evs[k][li][1]) for k in range(steps))
-            g_ms = statistics.mean(evs[k][li][1].elapsed_time(evs[k][li][2]) for k in range(steps))
+            q_ms = statistics.mean(evs[k][2 * li].elapsed_time(evs[k][2 * li + 1]) for k in range(steps))
+            g_ms = statistics.mean(evs[k][2 * li + 1].elapsed_time(evs[k][2 * li + 2]) for k in range(steps))
             gemm_ms += g_ms
             quant_ms += q_ms
             per_layer[L["name"]] = {
