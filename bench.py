@@ -56,9 +56,9 @@ FP6_PEAK_TOPS = 10100.0  # MI355X dense FP6 MFMA, published
 # or by HBM -- no counter available here separates the two -- so for the GEMM, whose operands fit that cache, this is
 # an upper bound of its HBM bytes; for the quantizer (a stream far larger than the cache) it is the HBM traffic.
 TRAFFIC_FROM_PROFILES = {
-    ("wan14b_720p_block", "int8"): {"gemm": 4315341824, "quant": 1379729408,
+    ("wan14b_720p_block", "int8"): {"gemm": 4315627520, "quant": 1379685376,
                                     "source": "profiles/gemm_w4a4_kernel+quantize_rows_kernel.wan14b_720p_block.md"},
-    ("wan14b_720p_block", "bf6"): {"gemm": 6519596032, "quant": 1517335296,
+    ("wan14b_720p_block", "bf6"): {"gemm": 6489400320, "quant": 1517329408,
                                    "source": "profiles/gemm_bf6_persistent_kernel+quantize_rows_kernel.wan14b_720p_block.md"},
 }
 TRAFFIC_UNIT = "bytes leaving L2 per launch (Infinity Cache or HBM), mean of the step's four launches; from the profile named in traffic_source, not from this run"
