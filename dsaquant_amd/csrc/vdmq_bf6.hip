@@ -18,6 +18,7 @@
 // from its own address.  Rows are padded to 32 (zero codes), K to 128.
 #include <type_traits>
 
+#include "vdmq_bf6_tilemap.h"
 #include "vdmq_internal.h"
 
 namespace vdmq {
@@ -46,7 +47,7 @@ constexpr int kBlkBytes = 1536;                 /* 32 rows x 64 k */
 [[maybe_unused]] constexpr int kBlkPlaneB = 1024;                /* offset of the 8-byte plane */
 constexpr int KS = 128;                         /* K step: two k-blocks per stage */
 constexpr int kRbStage = (KS / 64) * kBlkBytes; /* bytes of one row-block per stage */
-constexpr int kXcds = 8;
+constexpr int kXcds = kBf6Xcds;
 // per wave, beside the stage ring: the fp16 token scales of its 128 rows, the channel scales and the bias of its 64
 // columns, fetched when the tile starts so that the epilogue does not wait for them
 [[maybe_unused]] constexpr int kSideAs = 0, kSideWs = 256, kSideBias = 384;
@@ -79,22 +80,11 @@ struct Bf6Cfg {
 };
 using Bf6Big = Bf6Cfg<256, 256, 2, 4, 3, 1>;
 
-struct Bf6TileMap {
-    int tiles_m, tiles_n, super_n, total_super;
-    int group_n_log2, per_log2; /* a super-tile is (per / group_n) x group_n tiles */
-    int contig;                 /* XCD x walks the super-tiles [start[x], start[x + 1]) instead of every eighth */
-    int start[kXcds + 1];
-};
-
-// workgroup b runs on XCD b % 8; each XCD walks super-tiles (see vdmq_gemm.hip)
+// workgroup b runs on XCD b % 8; each XCD walks super-tiles (vdmq_bf6_tilemap.h)
 [[maybe_unused]] __device__ __forceinline__ bool map_tile(const Bf6TileMap &tm, int bid, int &tile_m, int &tile_n) {
     const int xcd = bid % kXcds, slot = bid / kXcds;
-    const int j = slot & ((1 << tm.per_log2) - 1);
-    const int st = tm.contig ? tm.start[xcd] + (slot >> tm.per_log2) : (slot >> tm.per_log2) * kXcds + xcd;
-    if (st >= (tm.contig ? tm.start[xcd + 1] : tm.total_super)) return false;
-    tile_m = ((st / tm.super_n) << (tm.per_log2 - tm.group_n_log2)) + (j >> tm.group_n_log2);
-    tile_n = ((st % tm.super_n) << tm.group_n_log2) + (j & ((1 << tm.group_n_log2) - 1));
-    return tile_m < tm.tiles_m && tile_n < tm.tiles_n;
+    const int st = bf6_tilemap_super(tm, xcd, slot >> tm.per_log2);
+    return st >= 0 && bf6_tilemap_locate(tm, st, slot & ((1 << tm.per_log2) - 1), tile_m, tile_n);
 }
 
 [[maybe_unused]] __device__ __forceinline__ v8i ld_frag(const uint8_t *p, uint32_t la, uint32_t lb) {
@@ -429,15 +419,12 @@ __global__ __launch_bounds__(Cfg::kWaves * 64, (Cfg::kWaves * Cfg::kOcc + 3) / 4
     const int last_rb_m = (M + 31) / 32 - 1, last_rb_n = N / 32 - 1;
     const int ksteps = kblocks / (KS / 64);
     const int xcd = blockIdx.x % kXcds, place = blockIdx.x / kXcds; /* gridDim.x = kXcds << per_log2 */
-    const int st_end = tmap.contig ? tmap.start[xcd + 1] : tmap.total_super;
     // the seq-th super-tile of this XCD, and this workgroup's tile in it (false: none left; a super-tile at a ragged
     // edge may have no tile at this place: tile_m = -1)
     auto locate = [&](int seq, int &tile_m, int &tile_n) -> bool {
-        const int st = tmap.contig ? tmap.start[xcd] + seq : seq * kXcds + xcd;
-        if (st >= st_end) return false;
-        tile_m = ((st / tmap.super_n) << (tmap.per_log2 - tmap.group_n_log2)) + (place >> tmap.group_n_log2);
-        tile_n = ((st % tmap.super_n) << tmap.group_n_log2) + (place & ((1 << tmap.group_n_log2) - 1));
-        if (tile_m >= tmap.tiles_m || tile_n >= tmap.tiles_n) tile_m = -1;
+        const int st = bf6_tilemap_super(tmap, xcd, seq);
+        if (st < 0) return false;
+        if (!bf6_tilemap_locate(tmap, st, place, tile_m, tile_n)) tile_m = -1;
         return true;
     };
     // Advances seq to the next existing tile; `skipped` counts the super-tiles passed on the way in which this place
@@ -667,68 +654,50 @@ template <class Cfg>
 int launch_bf6_cfg(const uint8_t *xblocks, const __half *ascale, const uint8_t *wblocks, const __half *wscale, const __half *bias,
                    __half *out, int32_t *acc_out, int64_t M, int64_t N, int64_t K, int64_t ldo, const GemmTail &tail, hipStream_t s) {
     constexpr int per = 1 << Cfg::kPerLog2;
+    const int tiles_m = static_cast<int>(ceil_div(M, Cfg::BM)), tiles_n = static_cast<int>(ceil_div(N, Cfg::BN));
+    // Super-tile shape.  Candidates in order of preference: 8 x 4 tiles (2048 token rows x 1024 weight rows, the
+    // fewest operand bytes per tile and measured best wherever the work is even), the same with the edge super-tiles
+    // regrouped (fuller, so fewer of them), 16 x 2, 16 x 2 regrouped.  A later one replaces an earlier one when it
+    // saves the XCDs a round (super-tiles go round the XCDs in turn, and a workgroup that walks tiles spends a round
+    // on each, however full: six tile columns at M = 32760 take 4 rounds as 8 x 4 and 8 x 2, 3 with the last two
+    // columns as 16 x 2; M = 75600, N = 13824, 54 tile columns: 37 half-empty super-tiles become 19 full ones,
+    // 65 -> 63 rounds; M = 27280, N = 14336, three tile rows left over: 25 -> 24) or, at the same number of rounds,
+    // takes a tenth off the busiest XCD's tile count.  Problems of less than two tiles per CU keep their partly empty
+    // edge super-tiles: the few tiles are better spread over all XCDs than packed into the places of some.
+    const bool small = static_cast<int64_t>(tiles_m) * tiles_n < 2 * kXcds * per;
     Bf6TileMap tm;
-    tm.tiles_m = static_cast<int>(ceil_div(M, Cfg::BM));
-    tm.tiles_n = static_cast<int>(ceil_div(N, Cfg::BN));
-    tm.per_log2 = Cfg::kPerLog2;
-    // Super-tile shape: per / gn x gn tiles.  Super-tiles go round the XCDs in turn and a ragged edge leaves some
-    // of them partly empty -- six tile columns in groups of four give every other XCD half the work -- so groups of
-    // two columns replace the groups of four (2048 token rows x 1024 weight rows, the fewest operand bytes per tile
-    // and measured best wherever the work is even) when that takes at least a tenth off the busiest XCD's tile
-    // count (N = 1536 at M = 32760: +16 % at K = 1536, +23 % at K = 8960).
-    int64_t best_load = -1, total_super = 0;
-    for (int gn_log2 : {2, 1}) {
-        const int gn = 1 << gn_log2, gm = per >> gn_log2;
-        const int64_t sm = ceil_div(tm.tiles_m, gm), sn = ceil_div(tm.tiles_n, gn);
-        const int64_t last_m = tm.tiles_m - (sm - 1) * gm, last_n = tm.tiles_n - (sn - 1) * gn;
+    int64_t best_load = -1, best_rounds = 0;
+    for (int variant = 0; variant < 4; variant += small ? 2 : 1) {
+        Bf6TileMap cand;
+        bf6_tilemap_shape(cand, tiles_m, tiles_n, Cfg::kPerLog2, 2 - variant / 2, variant % 2 != 0);
         int64_t load[kXcds] = {};
-        const bool modelled = sm * sn <= 4096; /* beyond that the edges no longer matter: the first shape is taken */
+        const bool modelled = cand.total_super <= 4096; /* beyond that the edges no longer matter: the first shape is taken */
         if (modelled)
-            for (int64_t st = 0; st < sm * sn; ++st)
-                load[st % kXcds] += (st / sn == sm - 1 ? last_m : gm) * (st % sn == sn - 1 ? last_n : gn);
+            for (int st = 0; st < cand.total_super; ++st)
+                load[st % kXcds] += bf6_tilemap_tiles_before(cand, st + 1) - bf6_tilemap_tiles_before(cand, st);
         int64_t worst = 0;
         for (int x = 0; x < kXcds; ++x) worst = load[x] > worst ? load[x] : worst;
-        if (best_load < 0 || (modelled && best_load > 0 && worst * 10 <= best_load * 9)) {
+        const int64_t cand_rounds = ceil_div(cand.total_super, kXcds);
+        if (best_load < 0 || (modelled && best_load > 0 &&
+                              ((!small && cand_rounds < best_rounds) || ((small || cand_rounds == best_rounds) && worst * 10 <= best_load * 9)))) {
             best_load = worst;
-            tm.group_n_log2 = gn_log2;
-            tm.super_n = static_cast<int>(sn);
-            total_super = sm * sn;
+            best_rounds = cand_rounds;
+            tm = cand;
         }
     }
+    const int64_t total_super = tm.total_super;
     if (best_load < 0 || total_super * per + kXcds * per > (int64_t(1) << 30))
         return fail(VDMQ_ESHAPE, "M x N = %lld x %lld needs more workgroups than one launch can hold", (long long)M, (long long)N);
-    tm.total_super = static_cast<int>(total_super);
+    tm.contig = 0;
+    for (int x = 0; x <= kXcds; ++x) tm.start[x] = 0;
     int rounds = static_cast<int>(ceil_div(total_super, kXcds));
-    // Long K and wide N: every XCD takes one contiguous run of the super-tile sequence (n fastest), the runs cut so
-    // that they hold equal numbers of tiles; consecutive super-tiles of an XCD then share their token rows and,
-    // walking K in opposite directions, re-use what the previous one left in L2 (as in vdmq_gemm.hip).  Measured at
-    // M = 75600, K = 5120: 12...14 % fewer bytes from beyond L2 and 0...2 % less time for N = 13824 and 15360; with 20
-    // tile columns or fewer (N = 5120, 3072) it fetches 4 % more and is 3...5 % slower than taking turns.
-    tm.contig = K >= 2048 && tm.tiles_n >= 48;
-    if (tm.contig) {
-        const int gn = 1 << tm.group_n_log2, gm = per >> tm.group_n_log2;
-        const int64_t sm = total_super / tm.super_n;
-        const int64_t last_m = tm.tiles_m - (sm - 1) * gm;
-        auto tiles_before = [&](int64_t st) {
-            const int64_t r = st / tm.super_n, c = st % tm.super_n;
-            const int64_t rows_here = r == sm - 1 ? last_m : gm;
-            const int64_t cols_done = c * gn < tm.tiles_n ? c * gn : tm.tiles_n;
-            return r * gm * tm.tiles_n + rows_here * cols_done;
-        };
-        const int64_t all_tiles = static_cast<int64_t>(tm.tiles_m) * tm.tiles_n;
-        tm.start[0] = 0;
-        rounds = 0;
-        for (int x = 1; x <= kXcds; ++x) {
-            const int64_t want = (all_tiles * x + kXcds - 1) / kXcds;
-            int64_t lo = tm.start[x - 1], hi = total_super;
-            while (lo < hi) {
-                const int64_t mid = (lo + hi) / 2;
-                if (tiles_before(mid) >= want) hi = mid; else lo = mid + 1;
-            }
-            tm.start[x] = x == kXcds ? static_cast<int>(total_super) : static_cast<int>(lo);
-            rounds = rounds > tm.start[x] - tm.start[x - 1] ? rounds : tm.start[x] - tm.start[x - 1];
-        }
-    }
+    // Long K and wide N: every XCD takes one contiguous run of the super-tile sequence (n fastest); consecutive
+    // super-tiles of an XCD then share their token rows and, walking K in opposite directions, re-use what the
+    // previous one left in L2 (as in vdmq_gemm.hip).  Measured at M = 75600, K = 5120: 12...14 % fewer bytes from
+    // beyond L2 and 0...2 % less time for N = 13824 and 15360; with 20 tile columns or fewer (N = 5120, 3072) it
+    // fetches 4 % more and is 3...5 % slower than taking turns.
+    const bool contig = K >= 2048 && tm.tiles_n >= 48;
+    if (contig) rounds = bf6_tilemap_runs(tm, true);
     const dim3 grid(static_cast<unsigned>(rounds) * kXcds * per), block(Cfg::kWaves * 64);
     const bool stream_out = M * N * 2 > (int64_t(224) << 20);
     const bool has_tail = tail.gate != nullptr || tail.residual != nullptr;
@@ -748,19 +717,22 @@ int launch_bf6_cfg(const uint8_t *xblocks, const __half *ascale, const uint8_t *
         attr_done[dev][which] = true;
     }
     // The persistent kernel gives every CU position a fixed share -- its place in each super-tile of the XCD's
-    // sequence -- where the hardware dispatcher would refill a CU as soon as it is free: it pays when no XCD has many
-    // partly empty super-tiles (a ragged last row of super-tiles spread over an XCD's run costs whole rounds:
-    // measured -16 % on M = 27280, N = 14336, where that takes a third more rounds), i.e. when its rounds are within 15 % of
-    // the busiest XCD's tiles / places (M = 32760, N = 4608: 10 rounds for 9, still +4 %).  Every fp16 output mode has
-    // it (with the gated residual tail: 249 registers, +3...4 % on the 14B and 5B output projections).
+    // sequence -- where the hardware dispatcher would refill a CU as soon as it is free: it pays when few super-tiles
+    // are partly empty (each costs its XCD a whole round: before the edges were regrouped, M = 27280, N = 14336 took a
+    // third more rounds with the ragged last row in one XCD's run and ran 16 % slower), i.e. when its rounds are
+    // within 15 % of the busiest XCD's tiles / places (M = 32760, N = 4608: 10 rounds for 9, still +4 %).  Every fp16
+    // output mode has it (with the gated residual tail: 249 registers, +3...4 % on the 14B and 5B output projections).
     const int64_t all_tiles = static_cast<int64_t>(tm.tiles_m) * tm.tiles_n;
     const int64_t busiest = tm.contig || best_load == 0 ? ceil_div(all_tiles, kXcds) : best_load;
     // (one workgroup per CU position: only where the device has as many CUs as the kernel has positions; elsewhere the
     // hardware dispatcher places the one-tile workgroups)
     static int cu_count[kMaxDevices] = {};
     if (cu_count[dev] == 0 && hipDeviceGetAttribute(&cu_count[dev], hipDeviceAttributeMultiprocessorCount, dev) != hipSuccess) cu_count[dev] = -1;
-    const bool persistent = which != 2 && cu_count[dev] == kXcds * per && static_cast<int64_t>(rounds) * 100 <= ceil_div(busiest, per) * 115;
+    // (its contiguous runs hold equal numbers of super-tiles: a round each, however full)
+    const int64_t rounds_p = ceil_div(total_super, kXcds);
+    const bool persistent = which != 2 && cu_count[dev] == kXcds * per && rounds_p * 100 <= ceil_div(busiest, per) * 115;
     if (persistent) {
+        if (contig) bf6_tilemap_runs(tm, false);
         using PKernel = void (*)(const uint8_t *, const uint8_t *, const __half *, const __half *, const __half *, __half *, int, int, int,
                                  int64_t, Bf6TileMap, GemmTail);
         const PKernel pk[5] = {gemm_bf6_persistent_kernel<Cfg, 0>, gemm_bf6_persistent_kernel<Cfg, 1>, nullptr, gemm_bf6_persistent_kernel<Cfg, 3>,

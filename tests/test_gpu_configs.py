@@ -10,8 +10,9 @@ in seconds, so each case checks
 * rows are independent: the first 4113 rows of the full run equal a run on those rows alone (another launch
   geometry, other tiles, another tile order);
 * which kernel and tile order the library chose, where the choice has special cases: the bf6 path's kernel that walks
-  tiles, the one-workgroup-per-tile kernel it falls back to on a ragged super-tile column, 16 x 2 super-tiles for six
-  tile columns, contiguous runs for wide N; the int8 path's three tile shapes.
+  tiles (also where tile rows or columns are left over and regrouped), the one-workgroup-per-tile kernel it falls back
+  to on small problems, 16 x 2 super-tiles for six tile columns, contiguous runs for wide N; the int8 path's three
+  tile shapes.
 """
 import numpy as np
 import pytest
@@ -28,13 +29,13 @@ W4, BF6, BF6P = 1, 2, 3  # VDMQ_KERNEL_* of include/vdmq.h
 # (config, name, M, K, N, calls, {path: (kernel, tile_m, tile_n, group_n, contiguous)})
 CASES = [
     ("cfg1", "qkv", 32760, 1536, 4608, 1, {"int8": (W4, 256, 128, 4, 0), "bf6": (BF6P, 256, 256, 4, 0)}),
-    ("cfg1", "o", 32760, 1536, 1536, 1, {"int8": (W4, 256, 128, 4, 0), "bf6": (BF6P, 256, 256, 2, 0)}),       # six tile columns: 16 x 2
+    ("cfg1", "o", 32760, 1536, 1536, 1, {"int8": (W4, 256, 128, 4, 0), "bf6": (BF6P, 256, 256, 4, 0)}),       # six tile columns: four as 8 x 4, two as 16 x 2
     ("cfg1", "ffn_up", 32760, 1536, 8960, 1, {"int8": (W4, 256, 256, 4, 0), "bf6": (BF6P, 256, 256, 4, 0)}),
-    ("cfg1", "ffn_down", 32760, 8960, 1536, 1, {"int8": (W4, 256, 128, 4, 0), "bf6": (BF6P, 256, 256, 2, 0)}),
+    ("cfg1", "ffn_down", 32760, 8960, 1536, 1, {"int8": (W4, 256, 128, 4, 0), "bf6": (BF6P, 256, 256, 4, 0)}),
     ("cfg1", "cross_kv", 512, 1536, 3072, 1, {"int8": (W4, 128, 128, 4, 0), "bf6": (BF6P, 256, 256, 2, 0)}),
     ("cfg2", "qkv", 27280, 3072, 9216, 2, {"int8": (W4, 256, 256, 4, 1), "bf6": (BF6P, 256, 256, 4, 0)}),
     ("cfg2", "o", 27280, 3072, 3072, 2, {"int8": (W4, 256, 256, 4, 1), "bf6": (BF6P, 256, 256, 4, 0)}),
-    ("cfg2", "ffn_up", 27280, 3072, 14336, 2, {"int8": (W4, 256, 256, 4, 1), "bf6": (BF6, 256, 256, 4, 1)}),   # ragged super-tile row: not persistent
+    ("cfg2", "ffn_up", 27280, 3072, 14336, 2, {"int8": (W4, 256, 256, 4, 1), "bf6": (BF6P, 256, 256, 4, 1)}),  # three tile rows left over: regrouped
     ("cfg2", "ffn_down", 27280, 14336, 3072, 2, {"int8": (W4, 256, 256, 4, 1), "bf6": (BF6P, 256, 256, 4, 0)}),
     ("cfg3", "o", 75600, 5120, 5120, 1, {"int8": (W4, 256, 256, 4, 1), "bf6": (BF6P, 256, 256, 4, 0)}),
     ("cfg3", "ffn_up", 75600, 5120, 13824, 1, {"int8": (W4, 256, 256, 4, 1), "bf6": (BF6P, 256, 256, 4, 1)}),

@@ -478,3 +478,20 @@ def test_library_says_where_the_fp6_path_pays():
     assert pays(512, 10240, 5120)            # the skinny cross-attention K/V case of the 14B model: wide N, long K
     assert not pays(512, 3072, 1536)         # the same of the 1.3B model
     assert not pays(0, 128, 64) and not pays(-1, 128, 64)
+
+
+def test_bf6_tile_order_takes_every_tile_once(tmp_path):
+    """The tile order of the bf6 GEMM kernels (regrouped edge super-tiles, round-robin and both kinds of contiguous
+    runs) enumerated on the host for every grid up to 72 x 72 tiles and the benchmark shapes: tests/tilemap_check.cpp
+    includes the header the kernels and their launcher use."""
+    import shutil
+    import subprocess
+    cxx = shutil.which("g++") or shutil.which("c++")
+    if cxx is None:
+        pytest.skip("no host C++ compiler")
+    root = Path(__file__).resolve().parent.parent
+    exe = tmp_path / "tilemap_check"
+    subprocess.run([cxx, "-O1", "-std=c++17", "-Wall", "-Werror", "-I", str(root / "dsaquant_amd" / "csrc"),
+                    str(root / "tests" / "tilemap_check.cpp"), "-o", str(exe)], check=True)
+    res = subprocess.run([str(exe)], stdout=subprocess.PIPE, text=True)
+    assert res.returncode == 0 and res.stdout.startswith("ok "), res.stdout
