@@ -235,7 +235,7 @@ class Workload:
         }
 
 
-BF6_CODES = [0x00, 0x0C, 0x10, 0x12, 0x14, 0x15, 0x16, 0x17, 0x18]  # E3M2 codes of |q| = 0..8; the sign is bit 5
+BF6_CODES = [0, 1, 2, 3, 4, 5, 6, 7, 8]  # E3M2 codes of |q| / 16, |q| = 0..8, as the operand blocks hold them; the sign is bit 5
 
 
 def probe_operands(np, kind, data, rng):
@@ -362,7 +362,7 @@ def main():
         "value": round(r["step_tops"], 1), "unit": "TOPS", "n_gpus": 1, "steps": args.steps, "warmup": args.warmup,
         "ms_per_step": round(r["ms_per_step"], 4), "higher_is_better": True, "scaling": "weak", "vs_baseline": None,
         "dtype": ("int4 x int4 -> int32 (int8 MFMA), fp16 in/out" if path == "int8" else
-                  "int4 x int4 as exact E3M2 floats -> fp32 accumulator holding the exact integer (FP6 MFMA), fp16 in/out"),
+                  "int4 x int4 as exact E3M2 floats (q / 16) -> fp32 accumulator holding the exact integer / 256 (FP6 MFMA), fp16 in/out"),
         "data": "synthetic", "matrix_path": path,
         "config": {"workload": f"{args.workload}: M={wl['M']} tokens, linears " + ", ".join(f"{n} {k}->{o}" for n, k, o in wl["linears"])
                                + "; each = A4 quantizer + W4A4 GEMM + scale/bias epilogue, clip 1.0"},

@@ -211,9 +211,10 @@ __device__ __forceinline__ void quantize_held_row(const u32x4 (&v)[NCH], int lan
 // padding per 256 keep both the 16-byte writes and the 64-byte-per-lane reads free of bank
 // conflicts) and come back as 32 consecutive fp16 per lane.  Those are scaled, rounded to integers
 // (v_rndne_f32: half to even) and clamped exactly as in quantize_word_fast / quantize_word_exact,
-// and v_cvt_scalef32_pk32_bf6_f16 packs the 32 integers -- every one of [-8, 7] is an E3M2 value,
-// so the conversion is exact -- into the string.  Rows of the last row-block beyond M stay unwritten
-// (the GEMM never stores them); K is padded to 128 with zeros.
+// and the conversion instruction (v_cvt_scalef32_2xpk16_bf6_f32, or v_cvt_scalef32_pk32_bf6_f16 on the literal
+// path) packs the 32 integers into the string with a scale of 16: the block holds q / 16, an E3M2 value for every
+// q of [-8, 8] (code sign << 5 | |q|), so the conversion is exact.  Rows of the last row-block beyond M stay
+// unwritten (the GEMM never stores them); K is padded to 128 with zeros.
 typedef _Float16 f16x32 __attribute__((ext_vector_type(32)));
 typedef float f32x16 __attribute__((ext_vector_type(16)));
 typedef unsigned int u32x6 __attribute__((ext_vector_type(6)));
@@ -307,7 +308,7 @@ __device__ __forceinline__ void quantize_held_row_bf6(u32x4 (&v)[NCH], int lane,
                     odd[u * 4 + i] = __builtin_rintf(__builtin_amdgcn_fmed3f(__builtin_fmaf(static_cast<float>(h[1]), rscale, 0.0f), -8.0f, 7.0f));
                 }
             }
-            str = __builtin_amdgcn_cvt_scalef32_2xpk16_bf6_f32(even, odd, 1.0f);
+            str = __builtin_amdgcn_cvt_scalef32_2xpk16_bf6_f32(even, odd, 16.0f);
         } else {
             f16x32 q;
 #pragma unroll
@@ -323,7 +324,7 @@ __device__ __forceinline__ void quantize_held_row_bf6(u32x4 (&v)[NCH], int lane,
                     }
                 }
             }
-            str = __builtin_amdgcn_cvt_scalef32_pk32_bf6_f16(q, 1.0f);
+            str = __builtin_amdgcn_cvt_scalef32_pk32_bf6_f16(q, 16.0f);
         }
         // per-lane stores would scatter 16-byte pieces over 64 cache lines per instruction (measured: 2x
         // slower than the HBM-bound int4 quantizer): collect the workgroup's strings in LDS instead -- its

@@ -298,7 +298,8 @@ def clear_native_cache() -> None:
 
 # ------------------------------------------------- which matrix instructions run the GEMM
 # "int8": v_mfma_i32_32x32x32_i8 on nibbles widened in registers.  "bf6": v_mfma_f32_32x32x64_f8f6f4 on 6-bit
-# floats (twice the rate, no widening work; every int4 value is exact in E3M2, so is the fp32 accumulation).
+# floats (twice the rate, no widening work; every int4 value q is held as the E3M2 float q / 16, exactly, and the
+# fp32 accumulation of the products is exact too).
 # Both give bit-identical results.  "auto" asks the library (vdmq_bf6_pays: bf6 for problems with enough 256 x 256
 # output tiles, fewer when K is long, none needed when N is wide too).
 _MATRIX_PATH = os.environ.get("VDMQ_MATRIX_PATH", "auto")

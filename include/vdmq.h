@@ -217,7 +217,8 @@ int vdmq_linear_w4a4_noalloc(const void *x, int64_t M, int64_t K, int64_t ldx, f
 
 /* ---- bf6 matrix path (optional; no counterpart in the reference).
  * gfx950 multiplies 6-bit floats (E3M2) at twice its int8 rate, E3M2 holds every
- * int4 value exactly and fp32 accumulation of their products is exact for
+ * int4 value exactly -- the blocks hold q as the float q / 16, whose code is
+ * sign << 5 | |q| -- and fp32 accumulation of their products is exact for
  * K <= 65536, so the same GEMM can run on v_mfma_f32_32x32x64_f8f6f4 with
  * bit-identical results.  Operands are "bf6 blocks": per row and 32 consecutive
  * k one 192-bit string of six-bit codes, stored by panels of 8 rows (a panel holds

@@ -299,8 +299,10 @@ def np_gated_residual(y_h: np.ndarray, gate_h, res_h, rows_per_gate: int = 1) ->
     return out
 
 
-# E3M2 ("bf6") codes of the integers -8..8: sign << 5 | exponent << 2 | mantissa, value = 2^(e-3) * (1 + m/4)
-# for e > 0 (OCP Microscaling Formats specification, FP6 E3M2, bias 3; no infinities or NaNs).
+# E3M2 ("bf6") codes: sign << 5 | exponent << 2 | mantissa, value = 2^(e-3) * (1 + m/4) for e > 0 and m / 16 for
+# e = 0 (OCP Microscaling Formats specification, FP6 E3M2, bias 3; no infinities or NaNs).  The operand blocks hold
+# an int4 value q as the E3M2 float q / 16, whose code is sign << 5 | |q|.
+BF6_BLOCK_SCALE = 16.0
 def np_bf6_decode(code: np.ndarray) -> np.ndarray:
     """E3M2 code (0..63) -> value, straight from the format definition (subnormals included)."""
     code = code.astype(np.int64)
@@ -311,7 +313,7 @@ def np_bf6_decode(code: np.ndarray) -> np.ndarray:
 
 
 def np_unpack_bf6_blocks(blocks: np.ndarray, rows: int, K: int) -> np.ndarray:
-    """bf6 operand buffer (u8) -> values float64 [rows, K].  Layout: rows padded to 32 and stored in panels of 8, K padded
+    """bf6 operand buffer (u8) -> the integers it stands for, float64 [rows, K] (E3M2 value x 16).  Layout: rows padded to 32 and stored in panels of 8, K padded
     to 128 and cut into k-blocks of 64; a panel holds its k-blocks one after the other, 384 bytes each =
     [h = 0: 8 rows x 16 B][h = 1: 8 rows x 16 B][h = 0: 8 rows x 8 B][h = 1: 8 rows x 8 B].  A row's 16-byte and 8-byte
     parts for (k-block, h) form one 192-bit little-endian string holding the 32 six-bit codes of k = 64 kb + 32 h + e
@@ -325,7 +327,7 @@ def np_unpack_bf6_blocks(blocks: np.ndarray, rows: int, K: int) -> np.ndarray:
     s = np.concatenate([lo, hi], axis=4)                      # [panel, kb, h, row in panel, 24 bytes]
     bits = np.unpackbits(s, axis=4, bitorder="little")        # 192 bits
     codes = (bits.reshape(panels, kblocks, 2, 8, 32, 6) * (1 << np.arange(6))).sum(axis=5)
-    vals = np_bf6_decode(codes)                               # [panel, kb, h, j, e]
+    vals = np_bf6_decode(codes) * BF6_BLOCK_SCALE             # [panel, kb, h, j, e]
     full = vals.transpose(0, 3, 1, 2, 4).reshape(panels * 8, kblocks * 64)
     assert not full[rows:].any() and not full[:, K:].any(), "padding must be zero"
     return full[:rows, :K]

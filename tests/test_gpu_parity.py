@@ -650,7 +650,7 @@ def bf6_path():
 @pytest.mark.parametrize("M,K", [(257, 1536), (100, 64), (77, 192), (515, 5120), (19, 16384 + 64)])
 def test_bf6_blocks_hold_the_quantized_values(M, K):
     """native int4 -> bf6 blocks: decoding the blocks with the format's definition gives back the oracle's integers
-    (layout, E3M2 codes and zero padding of rows to 32 and K to 128)."""
+    (layout, E3M2 codes of q / 16 and zero padding of rows to 32 and K to 128)."""
     v = vk()
     x = special_rows(O.synth_linear(M, K, 128, seed=M + K)[0])
     qn, sc = v.quantize_activation_native(t16(x), 0.95)

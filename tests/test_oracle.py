@@ -443,7 +443,8 @@ def test_gated_residual_oracle_equals_torch_fp16_tensor_arithmetic():
 
 def test_bf6_decoder_follows_the_format_and_holds_every_int4_value():
     """np_bf6_decode against the E3M2 value table worked by hand (exponent bias 3, 2 mantissa bits, subnormals at
-    e = 0, maximum 28): all 32 magnitudes are listed; every integer -8..8 has exactly one code."""
+    e = 0, maximum 28): all 32 magnitudes are listed; every integer -8..8 has exactly one code, and so has every q / 16 -- the
+    form the operand blocks use."""
     table = [0, 0.0625, 0.125, 0.1875, 0.25, 0.3125, 0.375, 0.4375, 0.5, 0.625, 0.75, 0.875, 1, 1.25, 1.5, 1.75,
              2, 2.5, 3, 3.5, 4, 5, 6, 7, 8, 10, 12, 14, 16, 20, 24, 28]
     codes = np.arange(64)
@@ -452,10 +453,12 @@ def test_bf6_decoder_follows_the_format_and_holds_every_int4_value():
     assert np.array_equal(vals[32:], -np.array(table, dtype=np.float64))
     for q in range(-8, 9):
         assert (vals == q).sum() == (2 if q == 0 else 1)  # +0 and -0
+        # the blocks hold q / 16, whose code is the sign bit and the magnitude as a plain integer
+        assert O.np_bf6_decode(np.array([(32 if q < 0 else 0) | abs(q)]))[0] * O.BF6_BLOCK_SCALE == q
     # unpacker: a hand-built block buffer (row r, column k holds ((r + k) % 16) - 8) decodes to itself
     rows, K = 40, 192
     want = (np.add.outer(np.arange(rows), np.arange(K)) % 16 - 8).astype(np.int64)
-    enc = {int(v): int(c) for c, v in zip(codes, vals) if float(v).is_integer() and -8 <= v <= 8 and not (v == 0 and c >= 32)}
+    enc = {int(v * 16): int(c) for c, v in zip(codes, vals) if float(v * 16).is_integer() and -8 <= v * 16 <= 8 and not (v == 0 and c >= 32)}
     kblocks, panels = (K + 127) // 128 * 2, (rows + 31) // 32 * 4
     buf = np.zeros((panels, kblocks, 384), np.uint8)  # panels of 8 rows; per k-block [h0 16 B x 8][h1 16 B x 8][h0 8 B x 8][h1 8 B x 8]
     for r in range(rows):
