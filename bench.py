@@ -58,7 +58,7 @@ FP6_PEAK_TOPS = 10100.0  # MI355X dense FP6 MFMA, published
 TRAFFIC_FROM_PROFILES = {
     ("wan14b_720p_block", "int8"): {"gemm": 4315627520, "quant": 1379685376,
                                     "source": "profiles/gemm_w4a4_kernel+quantize_rows_kernel.wan14b_720p_block.md"},
-    ("wan14b_720p_block", "bf6"): {"gemm": 6358552576, "quant": 1517329408,
+    ("wan14b_720p_block", "bf6"): {"gemm": 6432161792, "quant": 1517329408,
                                    "source": "profiles/gemm_bf6_persistent_kernel+quantize_rows_kernel.wan14b_720p_block.md"},
 }
 TRAFFIC_UNIT = "bytes leaving L2 per launch (Infinity Cache or HBM), mean of the step's four launches; from the profile named in traffic_source, not from this run"
