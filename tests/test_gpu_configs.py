@@ -127,3 +127,41 @@ def test_persistent_bf6_kernel_with_one_to_six_k_steps():
         finally:
             v.set_matrix_path(old)
             v.clear_native_cache()
+
+
+@pytest.mark.parametrize("M,N,K,group_n,contig", [
+    (27280, 14336, 2048, 4, 1),   # three tile rows left over: bottom edge regrouped 3 x 10, contiguous runs of equal length
+    (18944 + 100, 13824, 128, 4, 0),  # 54 tile columns: the last two regrouped 16 x 2; a partly filled bottom row as well
+    (32760, 4608, 64, 4, 0),      # 18 tile columns: 10 -> 9 rounds with the last two regrouped
+    (27280, 35 * 256, 64, 4, 0),  # 107 x 35 tiles: three columns and three rows left over, both regrouped (16 -> 15 rounds)
+])
+def test_bf6_tile_orders_with_regrouped_edges(M, N, K, group_n, contig):
+    """Problems whose tile grid leaves rows or columns over and whose edge super-tiles the launcher regroups: every
+    output element against the int8 path (a tile left out or stored twice with other operands would show), sampled
+    rows against the oracle, and the launch the library reports."""
+    from dsaquant_amd import _lib
+    from dsaquant_amd.kernels import vdm_w4a4 as v
+
+    assert v.is_available(), v.load_error()
+    rng = np.random.default_rng(M + N + K)
+    qw = rng.integers(-8, 8, (N, K), dtype=np.int8)
+    x = O.synth_linear(M, K, 128, seed=K)[0]
+    _, _, ws, bias = O.synth_linear(1, 64, N, seed=K + 1)
+    print(f"regrouped edges M={M} N={N} K={K}", flush=True)
+    old = v.matrix_path()
+    try:
+        out = {}
+        for path in ("bf6", "int8"):
+            v.set_matrix_path(path)
+            out[path] = v.linear_vdm_w4a4(_dev(x), _dev(O.np_pack_wgt_v1(qw)), _dev(O.np_pack_wscales_v1(ws, K)), _dev(bias), clip_ratio=1.0)
+            if path == "bf6":
+                info = _lib.last_gemm_launch()
+                assert (info.kernel, info.group_n, info.contiguous_runs) == (BF6P, group_n, contig)
+        assert torch.equal(out["bf6"], out["int8"])
+        rows = np.r_[0:8, M // 2:M // 2 + 8, M - 8:M]
+        want = O.np_linear(x[rows], qw, ws, bias, 1.0)[0]
+        assert np.array_equal(out["bf6"][torch.from_numpy(rows).to(DEV)].cpu().numpy().view(np.uint16), want.view(np.uint16))
+    finally:
+        v.set_matrix_path(old)
+        v.clear_native_cache()
+        torch.cuda.empty_cache()
