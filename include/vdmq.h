@@ -169,7 +169,7 @@ int vdmq_gemm_w4a4_acc(const void *qact, const void *wq, int32_t *acc, int64_t M
 typedef struct vdmq_gemm_launch_info {
     int kernel;                 /* VDMQ_KERNEL_* */
     int tile_m, tile_n;         /* output tile of one workgroup: token rows x channels */
-    int group_m, group_n;       /* super-tile, in tiles */
+    int group_m, group_n;       /* super-tile, in tiles (the bf6 kernels may regroup the tile rows and columns left over at the edges) */
     int contiguous_runs;        /* 1: each XCD walks one contiguous run of super-tiles, K direction alternating */
     int split_k_tiles;          /* always 0: no launch splits the K range of its tiles (kept for the layout of the struct) */
     int64_t workgroups;         /* grid size */
