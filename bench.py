@@ -169,7 +169,7 @@ class Workload:
                 events[2 * li + 1].record(self.stream)
             if L["bf6"]:
                 _lib.check(lib.vdmq_gemm_w4a4_bf6(L["qact"].data_ptr(), L["scale"].data_ptr(), L["wq"].data_ptr(), L["ws"].data_ptr(),
-                                                  L["bias"].data_ptr(), L["out"].data_ptr(), M, L["N"], L["K"], L["N"], s))
+                                                  L["bias"].data_ptr(), L["out"].data_ptr(), _lib.VDMQ_OUT_F16, M, L["N"], L["K"], L["N"], s))
             else:
                 _lib.check(lib.vdmq_gemm_w4a4(L["qact"].data_ptr(), L["scale"].data_ptr(), L["wq"].data_ptr(), L["ws"].data_ptr(),
                                               L["bias"].data_ptr(), L["out"].data_ptr(), _lib.VDMQ_OUT_F16, M, L["N"], L["K"], L["N"], s))

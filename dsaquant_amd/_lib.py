@@ -13,6 +13,7 @@ CSRC = _PKG / "csrc"
 
 _LIB: Optional[ctypes.CDLL] = None
 
+VDMQ_VERSION = 2  # include/vdmq.h; also the version of the bf6 block format
 VDMQ_OUT_F16 = 0
 VDMQ_OUT_BF16 = 1
 VDMQ_ACT_NONE = 0
@@ -23,8 +24,7 @@ VDMQ_LN_AFFINE = 2
 class GemmLaunchInfo(ctypes.Structure):
     """vdmq_gemm_launch_info of include/vdmq.h."""
     _fields_ = [("kernel", ctypes.c_int), ("tile_m", ctypes.c_int), ("tile_n", ctypes.c_int), ("group_m", ctypes.c_int),
-                ("group_n", ctypes.c_int), ("contiguous_runs", ctypes.c_int), ("split_k_tiles", ctypes.c_int),
-                ("workgroups", ctypes.c_int64)]
+                ("group_n", ctypes.c_int), ("contiguous_runs", ctypes.c_int), ("workgroups", ctypes.c_int64)]
 
 
 KERNEL_GEMM_W4A4, KERNEL_GEMM_BF6, KERNEL_GEMM_BF6_PERSISTENT = 1, 2, 3
@@ -65,11 +65,12 @@ SIGNATURES = {
     "vdmq_quantize_act_ln_bf6": (_int, [_p, _i64, _i64, _i64, _f32, _int, _p, _p, _i64, _i64, _f32, _p, _p, _p]),
     "vdmq_workspace_bytes_bf6": (_i64, [_i64, _i64]),
     "vdmq_bf6_pays": (_int, [_i64, _i64, _i64]),
-    "vdmq_linear_w4a4_bf6": (_int, [_p, _i64, _i64, _i64, _f32, _int, _p, _p, _p, _p, _i64, _i64, _p, _i64, _p]),
+    "vdmq_linear_w4a4_bf6": (_int, [_p, _i64, _i64, _i64, _f32, _int, _p, _p, _p, _p, _int, _i64, _i64, _p, _i64, _p]),
     "vdmq_native_to_bf6": (_int, [_p, _i64, _i64, _p, _p]),
     "vdmq_weight_v1_to_bf6": (_int, [_p, _p, _i64, _i64, _p]),
-    "vdmq_gemm_w4a4_bf6": (_int, [_p, _p, _p, _p, _p, _p, _i64, _i64, _i64, _i64, _p]),
-    "vdmq_gemm_w4a4_bf6_ex": (_int, [_p, _p, _p, _p, _p, _p, _i64, _i64, _p, _i64, _p, _i64, _i64, _i64, _i64, _p]),
+    "vdmq_bf6_to_weight_v1": (_int, [_p, _p, _i64, _i64, _p]),
+    "vdmq_gemm_w4a4_bf6": (_int, [_p, _p, _p, _p, _p, _p, _int, _i64, _i64, _i64, _i64, _p]),
+    "vdmq_gemm_w4a4_bf6_ex": (_int, [_p, _p, _p, _p, _p, _p, _i64, _i64, _p, _i64, _p, _int, _i64, _i64, _i64, _i64, _p]),
     "vdmq_gemm_w4a4_bf6_acc": (_int, [_p, _p, _p, _i64, _i64, _i64, _p]),
     "vdmq_copy_u128": (_int, [_p, _p, _i64, _p]),
     "vdmq_mfma_probe_operand_bytes": (_i64, []),
@@ -106,6 +107,8 @@ def load() -> ctypes.CDLL:
         fn = getattr(lib, name)
         fn.restype = restype
         fn.argtypes = argtypes
+    if lib.vdmq_version() != VDMQ_VERSION:
+        raise RuntimeError(f"{LIB_PATH} has interface version {lib.vdmq_version()}, this package expects {VDMQ_VERSION}: rebuild it (make -C {CSRC})")
     _LIB = lib
     return lib
 

@@ -22,12 +22,11 @@ import torch
 import torch.nn as nn
 
 PACKED_CHECKPOINT_FORMAT = "vdm_w4a4_packed_v1"
-# checkpoints written by earlier tooling carry a different infix in the format
-# string and in the three buffer names (packed_checkpoint.py:19,25)
-_LEGACY_INFIX = "".join(("d", "i", "y", "_"))
-_LEGACY_PACKED_CHECKPOINT_FORMAT = PACKED_CHECKPOINT_FORMAT.replace("vdm_", "vdm_" + _LEGACY_INFIX, 1)
+# checkpoints written by earlier tooling carry another format string and other
+# names for the three buffers (packed_checkpoint.py:19,25)
+_LEGACY_PACKED_CHECKPOINT_FORMAT = "vdm_diy_w4a4_packed_v1"
 VDM_BUFFER_SUFFIXES = ("vdm_weight_packed", "vdm_weight_scale_packed", "vdm_weight_scale")
-_LEGACY_BUFFER_SUFFIXES = tuple(_LEGACY_INFIX + s[len("vdm_"):] for s in VDM_BUFFER_SUFFIXES)
+_LEGACY_BUFFER_SUFFIXES = ("diy_weight_packed", "diy_weight_scale_packed", "diy_weight_scale")
 _KNOWN_FORMATS = (PACKED_CHECKPOINT_FORMAT, _LEGACY_PACKED_CHECKPOINT_FORMAT)
 
 
@@ -93,14 +92,17 @@ def _ordinary_entries(state_dict: dict, fp_weight_keys: set) -> dict:
 
 
 def load_packed_quantized_model(model: nn.Module, packed_ckpt: dict, *, quant_linear_cls: type, dtype: torch.dtype,
-                                device: torch.device, require_vdm_kernel: bool = True) -> tuple:
+                                device: torch.device, require_vdm_kernel: bool = True, release_v1: bool = False) -> tuple:
     """Populate a freshly built model (Linear layers already swapped for
     ``quant_linear_cls``) from a packed checkpoint; returns ``(missing,
     unexpected)`` key lists (packed_checkpoint.py:52-148).
 
     Raises ValueError for an unknown format, AssertionError when the kernel
     library is required but unavailable, KeyError when a QuantLinear lacks any of
-    its three buffers, RuntimeError when no QuantLinear was populated.  The outcome
+    its three buffers, RuntimeError when no QuantLinear was populated.  ``release_v1``
+    (not in the reference): once every packed weight is relaid into the form the
+    kernels stream, free the memory of the v1 weight buffers -- ``state_dict()``
+    rebuilds them, see ``vdm_w4a4.release_v1_storage``.  The outcome
     on a file the reference's writer wrote is held to what the reference's loader
     leaves behind (tests/golden/reference_loader_outcome.json).
     """
@@ -145,12 +147,12 @@ def load_packed_quantized_model(model: nn.Module, packed_ckpt: dict, *, quant_li
     for module in model.modules():
         if isinstance(module, quant_linear_cls) and module.bias is not None:
             module._bias_half = module.bias.half().contiguous()
-    _prepare_for_kernels(model, device)
+    _prepare_for_kernels(model, device, release_v1)
     print(f"Loaded packed DSAQuant W4A4 checkpoint: {populated} QuantLinear layers")
     return list(missing), list(report.unexpected_keys)
 
 
-def _prepare_for_kernels(model: nn.Module, device) -> None:
+def _prepare_for_kernels(model: nn.Module, device, release_v1: bool = False) -> None:
     """The point at which the reference has its buffers attached and on the device (packed_checkpoint.py:102-148):
     relay them now, on the current stream, rather than inside the first forward (which may be under graph
     capture).  Nothing to do on a machine without the kernel library or for a model kept on the CPU."""
@@ -160,6 +162,8 @@ def _prepare_for_kernels(model: nn.Module, device) -> None:
 
     if vdm_w4a4.is_available():
         vdm_w4a4.prepare_model(model)
+        if release_v1:
+            vdm_w4a4.release_v1_storage(model)
 
 
 def enable_quant_kernels(model: nn.Module, *, quant_linear_cls: type) -> None:
@@ -202,9 +206,10 @@ def _prepare_fused(attention: nn.Module) -> None:
         layers = [getattr(attention, n) for n in names]
         if not all(l.vdm_weight_packed.is_cuda for l in layers) or not vdm_w4a4.is_available():
             continue
-        for l in layers:
-            vdm_w4a4.release_prepared(l.vdm_weight_packed)
-        vdm_w4a4.prepare_model(attention)
+        lean = any("_vdmq_v1_released" in l.vdm_weight_packed.__dict__ for l in layers)
+        vdm_w4a4.prepare_model(attention)  # (makes the concatenation; the projections' own forms go with their old buffers)
+        if lean:
+            vdm_w4a4.release_v1_storage(attention)
 
 
 def packed_state_dict_from_model(model: nn.Module, *, float_dtype: torch.dtype = torch.float16) -> dict:

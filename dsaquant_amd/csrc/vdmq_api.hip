@@ -108,7 +108,7 @@ int scratch_of_current_device(void **ptr) {
 
 extern "C" {
 
-int vdmq_version(void) { return 1; }
+int vdmq_version(void) { return VDMQ_VERSION; }
 const char *vdmq_arch(void) { return "gfx950"; }
 const char *vdmq_last_error(void) { return g_error; }
 int64_t vdmq_k_padded(int64_t K) { return k_padded(K); }
@@ -380,8 +380,17 @@ int vdmq_weight_v1_to_bf6(const void *qweight_v1, void *wblocks, int64_t N, int6
     return launch_weight_v1_to_bf6(static_cast<const uint8_t *>(qweight_v1), N, K, static_cast<uint8_t *>(wblocks), as_stream(stream));
 }
 
+int vdmq_bf6_to_weight_v1(const void *wblocks, void *qweight_v1, int64_t N, int64_t K, vdmq_stream_t stream) {
+    VDMQ_TRY(check_k(K));
+    VDMQ_TRY(check_n(N));
+    VDMQ_TRY(check_ptr(qweight_v1, "qweight_v1"));
+    VDMQ_TRY(check_ptr(wblocks, "wblocks"));
+    return launch_bf6_to_weight_v1(static_cast<const uint8_t *>(wblocks), N, K, static_cast<uint8_t *>(qweight_v1), as_stream(stream));
+}
+
 static int gemm_bf6_checked(const void *xblocks, const void *ascale, const void *wblocks, const void *wscale, const void *bias, void *out,
-                            int32_t *acc, int64_t M, int64_t N, int64_t K, int64_t ldo, const GemmTail &tail, vdmq_stream_t stream) {
+                            int out_dtype, int32_t *acc, int64_t M, int64_t N, int64_t K, int64_t ldo, const GemmTail &tail,
+                            vdmq_stream_t stream) {
     VDMQ_TRY(check_k(K));
     VDMQ_TRY(check_n(N));
     VDMQ_TRY(check_m(M));
@@ -393,26 +402,30 @@ static int gemm_bf6_checked(const void *xblocks, const void *ascale, const void 
         VDMQ_TRY(check_ptr(wscale, "wscale"));
         VDMQ_TRY(check_ptr(out, "out"));
         if (bias != nullptr) VDMQ_TRY(check_ptr(bias, "bias"));
+        if (out_dtype != VDMQ_OUT_F16 && out_dtype != VDMQ_OUT_BF16) return fail(VDMQ_EINVAL, "unknown out_dtype %d", out_dtype);
         if (ldo < (tail.split_cols ? tail.split_cols : N) || ldo % 8 != 0 || ldo > kMaxLdo)
             return fail(VDMQ_ESHAPE, "ldo must be >= the columns of a row, a multiple of 8 and at most %lld (got %lld)", (long long)kMaxLdo, (long long)ldo);
-        VDMQ_TRY(check_tail(tail, N));
+        if (tail.gate != nullptr || tail.residual != nullptr || tail.split_cols != 0) {
+            if (out_dtype != VDMQ_OUT_F16) return fail(VDMQ_EINVAL, "gate, residual and a split output need an fp16 output");
+            VDMQ_TRY(check_tail(tail, N));
+        }
     } else {
         VDMQ_TRY(check_ptr(acc, "acc"));
     }
     return launch_gemm_bf6(static_cast<const uint8_t *>(xblocks), static_cast<const __half *>(ascale), static_cast<const uint8_t *>(wblocks),
-                           static_cast<const __half *>(wscale), static_cast<const __half *>(bias), static_cast<__half *>(out), acc, M, N, K,
-                           ldo, tail, as_stream(stream));
+                           static_cast<const __half *>(wscale), static_cast<const __half *>(bias), out, out_dtype, acc, M, N, K, ldo, tail,
+                           as_stream(stream));
 }
 
 int vdmq_gemm_w4a4_bf6(const void *xblocks, const void *ascale, const void *wblocks, const void *wscale, const void *bias, void *out,
-                       int64_t M, int64_t N, int64_t K, int64_t ldo, vdmq_stream_t stream) {
-    return gemm_bf6_checked(xblocks, ascale, wblocks, wscale, bias, out, nullptr, M, N, K, ldo, GemmTail{}, stream);
+                       int out_dtype, int64_t M, int64_t N, int64_t K, int64_t ldo, vdmq_stream_t stream) {
+    return gemm_bf6_checked(xblocks, ascale, wblocks, wscale, bias, out, out_dtype, nullptr, M, N, K, ldo, GemmTail{}, stream);
 }
 
 int vdmq_gemm_w4a4_bf6_ex(const void *xblocks, const void *ascale, const void *wblocks, const void *wscale, const void *bias,
-                          const void *gate, int64_t ldg, int64_t rows_per_gate, const void *residual, int64_t ldr, void *out, int64_t M,
-                          int64_t N, int64_t K, int64_t ldo, vdmq_stream_t stream) {
-    return gemm_bf6_checked(xblocks, ascale, wblocks, wscale, bias, out, nullptr, M, N, K, ldo,
+                          const void *gate, int64_t ldg, int64_t rows_per_gate, const void *residual, int64_t ldr, void *out, int out_dtype,
+                          int64_t M, int64_t N, int64_t K, int64_t ldo, vdmq_stream_t stream) {
+    return gemm_bf6_checked(xblocks, ascale, wblocks, wscale, bias, out, out_dtype, nullptr, M, N, K, ldo,
                             make_tail(gate, ldg, rows_per_gate, residual, ldr), stream);
 }
 
@@ -420,13 +433,13 @@ int vdmq_gemm_w4a4_bf6_split(const void *xblocks, const void *ascale, const void
                              int64_t M, int64_t N, int64_t K, int64_t ldo, int64_t split_cols, int64_t part_stride, vdmq_stream_t stream) {
     GemmTail tail;
     VDMQ_TRY(check_split(tail, N, split_cols, part_stride));
-    return gemm_bf6_checked(xblocks, ascale, wblocks, wscale, bias, out, nullptr, M, N, K, ldo, tail, stream);
+    return gemm_bf6_checked(xblocks, ascale, wblocks, wscale, bias, out, VDMQ_OUT_F16, nullptr, M, N, K, ldo, tail, stream);
 }
 
 int vdmq_gemm_w4a4_bf6_acc(const void *xblocks, const void *wblocks, int32_t *acc, int64_t M, int64_t N, int64_t K,
                            vdmq_stream_t stream) {
     if (acc == nullptr && M != 0) return fail(VDMQ_EINVAL, "acc is null");
-    return gemm_bf6_checked(xblocks, nullptr, wblocks, nullptr, nullptr, nullptr, acc, M, N, K, N, GemmTail{}, stream);
+    return gemm_bf6_checked(xblocks, nullptr, wblocks, nullptr, nullptr, nullptr, VDMQ_OUT_F16, acc, M, N, K, N, GemmTail{}, stream);
 }
 
 int vdmq_bf6_pays(int64_t M, int64_t N, int64_t K) {
@@ -447,7 +460,7 @@ int64_t vdmq_workspace_bytes_bf6(int64_t M, int64_t K) {
 }
 
 int vdmq_linear_w4a4_bf6(const void *x, int64_t M, int64_t K, int64_t ldx, float clip, int act, const void *wblocks, const void *wscale,
-                         const void *bias, void *out, int64_t N, int64_t ldo, void *workspace, int64_t workspace_bytes,
+                         const void *bias, void *out, int out_dtype, int64_t N, int64_t ldo, void *workspace, int64_t workspace_bytes,
                          vdmq_stream_t stream) {
     VDMQ_TRY(check_k(K));
     VDMQ_TRY(check_n(N));
@@ -460,7 +473,7 @@ int vdmq_linear_w4a4_bf6(const void *x, int64_t M, int64_t K, int64_t ldx, float
     uint8_t *xblocks = static_cast<uint8_t *>(workspace);
     void *scale = xblocks + (bf6_bytes(M, K) + 255) / 256 * 256;
     VDMQ_TRY(vdmq_quantize_act_bf6(x, M, K, ldx, clip, act, xblocks, scale, stream));
-    return vdmq_gemm_w4a4_bf6(xblocks, scale, wblocks, wscale, bias, out, M, N, K, ldo, stream);
+    return vdmq_gemm_w4a4_bf6(xblocks, scale, wblocks, wscale, bias, out, out_dtype, M, N, K, ldo, stream);
 }
 
 int vdmq_weight_v1_to_native(const void *qweight_v1, void *wq_native, int64_t N, int64_t K, vdmq_stream_t stream) {

@@ -55,7 +55,7 @@ constexpr int kRbStage = (KS / 64) * kBlkBytes; /* bytes of one row-block per st
 constexpr int kXcds = kBf6Xcds;
 // The operand blocks hold q / 16, so an accumulator holds the integer sum / 256 (as exact as the sum itself: a power
 // of two); the factor goes into the channel scales of the epilogue.
-constexpr float kBf6AccScale = 256.0f;
+[[maybe_unused]] constexpr float kBf6AccScale = 256.0f;
 // per wave, beside the stage ring: the fp16 token scales of its 128 rows, the channel scales and the bias of its 64
 // columns, fetched when the tile starts so that the epilogue does not wait for them
 [[maybe_unused]] constexpr int kSideAs = 0, kSideWs = 256, kSideBias = 384;
@@ -151,8 +151,7 @@ struct Bf6KLoop {
                                                  kpos * (KS / 64) * kBf6PanelKb, 0, 0);
     }
     // LOAD_B / LOAD_A: this step issues the second half of stage kt + 2 / the first half of stage kt + 3; READ_NEXT: a
-    // step follows; YOUNGER: stage kt + 2 exists, i.e. six loads may stay in flight across the barrier (-1: look at kt;
-    // 2: stage kt + 1 is known to have landed, no wait for loads at all)
+    // step follows; YOUNGER: stage kt + 2 exists, i.e. six loads may stay in flight across the barrier (-1: look at kt)
     template <bool LOAD_B, bool LOAD_A, bool READ_NEXT, int YOUNGER>
     __device__ __forceinline__ void step(int kt, int &cur, v16f (&acc)[NI][MI], v8i (&wfa)[NI], v8i (&xfa)[MI], v8i (&wfb)[NI],
                                          v8i (&xfb)[MI]) const {
@@ -167,9 +166,7 @@ struct Bf6KLoop {
         }
         // one barrier per step: behind it stage kt + 1 is complete for every wave (the stage after it may still be on
         // its way: six loads), and nobody reads slot `cur` any more
-        if (YOUNGER == 2)
-            __builtin_amdgcn_s_waitcnt(waitcnt_imm(63, 0));
-        else if (YOUNGER > 0 || (YOUNGER < 0 && kt + 2 < ksteps))
+        if (YOUNGER > 0 || (YOUNGER < 0 && kt + 2 < ksteps))
             __builtin_amdgcn_s_waitcnt(waitcnt_imm(kLoads, 0));
         else
             __builtin_amdgcn_s_waitcnt(waitcnt_imm(0, 0));
@@ -183,15 +180,13 @@ struct Bf6KLoop {
         }
         cur = nxt;
     }
-    // TWO_LANDED: stage 1 has landed too (the kernel that walks tiles requests a tile's first stages under the epilogue
-    // of the tile before and waits for them there).  Step 0 then waits for no load: the one counter that tracks
-    // loads also tracks the output stores issued in between, and waiting for "all but the last six" would wait
-    // for every one of those.
-    template <bool TWO_LANDED>
+    // (The kernel that walks tiles has a tile's first two stages landed when it gets here, so its step 0 could skip
+    // the wait -- which, loads and stores sharing one counter, also waits for the output stores of the tile before --
+    // but a build that does measured the same time to 0.1 % on the 14B and 1.3B blocks: one form for both kernels.)
     __device__ __forceinline__ void run(int &cur, v16f (&acc)[NI][MI], v8i (&wfa)[NI], v8i (&xfa)[MI], v8i (&wfb)[NI], v8i (&xfb)[MI]) const {
         int kt = 0;
         if (ksteps > S) {
-            step<false, true, true, TWO_LANDED ? 2 : 1>(0, cur, acc, wfa, xfa, wfb, xfb);
+            step<false, true, true, 1>(0, cur, acc, wfa, xfa, wfb, xfb);
             for (kt = 1; kt + S < ksteps; ++kt) step<true, true, true, 1>(kt, cur, acc, wfa, xfa, wfb, xfb);
             step<true, false, true, 1>(kt, cur, acc, wfa, xfa, wfb, xfb);
             ++kt;
@@ -205,8 +200,9 @@ struct Bf6KLoop {
 // out = fp16(float(acc) * (float(as) * float(ws))) (+ bias in fp16) [then residual + y * gate]; one 32-row strip at
 // a time is transposed through the wave's staging area so that rows leave as whole 128-byte lines.  `side` holds the
 // wave's token scales, channel scales and bias; (m0, n0) is the corner's first output element.  `before_first_store`
-// runs once, after the first strip has been converted and staged.
-template <class Cfg, bool STREAM_OUT, bool TAIL, class Hook>
+// runs once, after the first strip has been converted and staged.  BF16: the same fp32 product, the fp16 bias added in
+// fp32 and one rounding (to nearest even) to bf16, as the int8 kernel writes a bf16 output; no tail.
+template <class Cfg, bool STREAM_OUT, bool TAIL, bool BF16, class Hook>
 __device__ __forceinline__ void bf6_epilogue(const v16f (&acc)[Cfg::NI][Cfg::MI], const uint8_t *side, uint8_t *stg, int lane, int m0, int n0,
                                              __half *out, int64_t ldo, int M, int N, const GemmTail &tail, Hook &&before_first_store) {
     constexpr int MI = Cfg::MI, NI = Cfg::NI, PR = Cfg::kPiecesPerRow, RS = Cfg::kStageRowBytes;
@@ -260,17 +256,30 @@ __device__ __forceinline__ void bf6_epilogue(const v16f (&acc)[Cfg::NI][Cfg::MI]
         for (int ni = 0; ni < NI; ++ni)
 #pragma unroll
             for (int rg = 0; rg < 4; ++rg) {
-                f16x4 h;
+                if (BF16) {
+                    const f16x4 b4 = *reinterpret_cast<const f16x4 *>(side + kSideBias + (ni * 32 + rg * 8 + lh * 4) * 2);
+                    uint32_t o[2] = {0, 0};
 #pragma unroll
-                for (int e = 0; e < 4; ++e) h[e] = static_cast<_Float16>(acc[ni][mi][rg * 4 + e] * (as * wsf[ni][rg][e]));
-                *reinterpret_cast<f16x4 *>(stg + l32 * RS + (ni * 32 + rg * 8 + lh * 4) * 2) = h;
+                    for (int e = 0; e < 4; ++e) {
+                        const float f = acc[ni][mi][rg * 4 + e] * (as * wsf[ni][rg][e]) + static_cast<float>(b4[e]); /* -0: no bias */
+                        uint32_t u = __float_as_uint(f);
+                        u = (f != f) ? 0x7FC00000u : u + 0x7FFFu + ((u >> 16) & 1u);
+                        o[e / 2] |= (u >> 16) << (16 * (e % 2));
+                    }
+                    *reinterpret_cast<u32x2 *>(stg + l32 * RS + (ni * 32 + rg * 8 + lh * 4) * 2) = u32x2{o[0], o[1]};
+                } else {
+                    f16x4 h;
+#pragma unroll
+                    for (int e = 0; e < 4; ++e) h[e] = static_cast<_Float16>(acc[ni][mi][rg * 4 + e] * (as * wsf[ni][rg][e]));
+                    *reinterpret_cast<f16x4 *>(stg + l32 * RS + (ni * 32 + rg * 8 + lh * 4) * 2) = h;
+                }
             }
         if (mi == 0) before_first_store();
 #pragma unroll
         for (int it = 0; it < PR / 2; ++it) {
             const int row = it * (64 / PR) + lane / PR;
             f16x8 hv = *reinterpret_cast<const f16x8 *>(stg + row * RS + (lane % PR) * 16);
-            hv += bv;
+            if (!BF16) hv += bv;
             const int mrow = m0 + mi * 32 + row;
             if (TAIL && tail.gate != nullptr && mrow < M) hv *= gv[it];
             if (TAIL && tail.residual != nullptr && mrow < M) hv = rv[it] + hv;
@@ -283,7 +292,8 @@ __device__ __forceinline__ void bf6_epilogue(const v16f (&acc)[Cfg::NI][Cfg::MI]
 #endif
 
 // OUT_MODE: 0 = scaled fp16 output, 1 = the same with non-temporal stores, 2 = raw accumulators as int32,
-// 3 / 4 = 0 / 1 followed by the gated residual update out = residual + y * gate (see vdmq_gemm.hip)
+// 3 / 4 = 0 / 1 followed by the gated residual update out = residual + y * gate (see vdmq_gemm.hip), 5 / 6 = 0 / 1 with
+// a bf16 output
 template <class Cfg, int OUT_MODE>
 __global__ __launch_bounds__(Cfg::kWaves * 64, (Cfg::kWaves * Cfg::kOcc + 3) / 4) void gemm_bf6_kernel(const uint8_t *__restrict__ X, const uint8_t *__restrict__ W,
                                                                          const __half *__restrict__ ascale,
@@ -292,7 +302,8 @@ __global__ __launch_bounds__(Cfg::kWaves * 64, (Cfg::kWaves * Cfg::kOcc + 3) / 4
                                                                          int32_t *__restrict__ acc_out, int M, int N, int kblocks,
                                                                          int64_t ldo, Bf6TileMap tmap, GemmTail tail) {
 #if defined(__HIP_DEVICE_COMPILE__) /* the host pass needs the kernel's stub only; it does not know the buffer builtins */
-    constexpr bool ACC_OUT = OUT_MODE == 2, STREAM_OUT = OUT_MODE == 1 || OUT_MODE == 4, TAIL = OUT_MODE >= 3;
+    constexpr bool ACC_OUT = OUT_MODE == 2, STREAM_OUT = OUT_MODE == 1 || OUT_MODE == 4 || OUT_MODE == 6;
+    constexpr bool TAIL = OUT_MODE == 3 || OUT_MODE == 4, BF16 = OUT_MODE >= 5;
     constexpr int BM = Cfg::BM, BN = Cfg::BN, S = Cfg::S, MI = Cfg::MI, NI = Cfg::NI, kWaves = Cfg::kWaves, kWavesN = Cfg::kWavesN;
     constexpr int kLoads = Cfg::kLoads, kStageBytes = Cfg::kStageBytes;
     constexpr int kStagingBytes = Cfg::kStagingBytes;
@@ -380,7 +391,7 @@ __global__ __launch_bounds__(Cfg::kWaves * 64, (Cfg::kWaves * Cfg::kOcc + 3) / 4
     read(wfa, xfa, lds, 0);
     int cur = 0;
     const Bf6KLoop<Cfg> k_loop{lds, src, lane_off, wave, wn, wm, la, lb, ksteps, k_reverse};
-    k_loop.template run<false>(cur, acc, wfa, xfa, wfb, xfb);
+    k_loop.run(cur, acc, wfa, xfa, wfb, xfb);
 
     const int l32 = lane & 31, lh = lane >> 5;
     if (ACC_OUT) {
@@ -403,7 +414,7 @@ __global__ __launch_bounds__(Cfg::kWaves * 64, (Cfg::kWaves * Cfg::kOcc + 3) / 4
         return;
     }
     if (n0 + wn0 >= N || m0 + wm0 >= M) return; /* nothing to store: the same for the whole wave */
-    bf6_epilogue<Cfg, STREAM_OUT, TAIL>(acc, side, lds + wave * kStagingBytes, lane, m0 + wm0, n0 + wn0, out, ldo, M, N, tail, [] {});
+    bf6_epilogue<Cfg, STREAM_OUT, TAIL, BF16>(acc, side, lds + wave * kStagingBytes, lane, m0 + wm0, n0 + wn0, out, ldo, M, N, tail, [] {});
 #endif
 }
 
@@ -416,7 +427,7 @@ __global__ __launch_bounds__(Cfg::kWaves * 64, (Cfg::kWaves * Cfg::kOcc + 3) / 4
     const uint8_t *__restrict__ X, const uint8_t *__restrict__ W, const __half *__restrict__ ascale, const __half *__restrict__ wscale,
     const __half *__restrict__ bias, __half *out, int M, int N, int kblocks, int64_t ldo, Bf6TileMap tmap, GemmTail tail) {
 #if defined(__HIP_DEVICE_COMPILE__)
-    constexpr bool STREAM_OUT = OUT_MODE == 1 || OUT_MODE == 4, TAIL = OUT_MODE >= 3;
+    constexpr bool STREAM_OUT = OUT_MODE == 1 || OUT_MODE == 4 || OUT_MODE == 6, TAIL = OUT_MODE == 3 || OUT_MODE == 4, BF16 = OUT_MODE >= 5;
     constexpr int BM = Cfg::BM, BN = Cfg::BN, S = Cfg::S, MI = Cfg::MI, NI = Cfg::NI, kWaves = Cfg::kWaves, kWavesN = Cfg::kWavesN;
     constexpr int kLoads = Cfg::kLoads, kStageBytes = Cfg::kStageBytes;
     static_assert(S == 3, "the prefetch under the epilogue uses ring slots 1 and 2");
@@ -511,7 +522,7 @@ __global__ __launch_bounds__(Cfg::kWaves * 64, (Cfg::kWaves * Cfg::kOcc + 3) / 4
 #pragma unroll
         for (int s = 0; s < S; ++s)
             if (s < ksteps) issue(src, k_reverse, s, s);
-        if (ksteps >= S) /* stages 0 and 1, as for every later tile (Bf6KLoop::run<true>) */
+        if (ksteps >= S) /* stages 0 and 1, as for every later tile */
             __builtin_amdgcn_s_waitcnt(waitcnt_imm(kLoads * (S - 2), 15));
         else
             __builtin_amdgcn_s_waitcnt(waitcnt_imm(0, 15));
@@ -530,7 +541,7 @@ __global__ __launch_bounds__(Cfg::kWaves * 64, (Cfg::kWaves * Cfg::kOcc + 3) / 4
                 for (int r = 0; r < 16; ++r) acc[ni][mi][r] = 0.f;
         read(wfa, xfa, lds + cur * kStageBytes, 0);
         const Bf6KLoop<Cfg> k_loop{lds, src, lane_off, wave, wn, wm, la, lb, ksteps, k_reverse};
-        k_loop.template run<false>(cur, acc, wfa, xfa, wfb, xfb);
+        k_loop.run(cur, acc, wfa, xfa, wfb, xfb);
 
         // ---- the next tile: its first two K steps go into slots 1 and 2 now (every wave is past the last barrier of
         // the K loop, behind which nothing reads the ring any more); slot 0 holds the epilogue's staging.  Not so when
@@ -560,8 +571,8 @@ __global__ __launch_bounds__(Cfg::kWaves * 64, (Cfg::kWaves * Cfg::kOcc + 3) / 4
             if (prefetch) __builtin_amdgcn_s_waitcnt(waitcnt_imm(0, 15));
         };
         if (n0 + wn0 < N && m0 + wm0 < M) /* the same for the whole wave */
-            bf6_epilogue<Cfg, STREAM_OUT, TAIL>(acc, side, lds + wave * Cfg::kStagingBytes, lane, m0 + wm0, n0 + wn0, out, ldo, M, N, tail,
-                                                prefetch_landed);
+            bf6_epilogue<Cfg, STREAM_OUT, TAIL, BF16>(acc, side, lds + wave * Cfg::kStagingBytes, lane, m0 + wm0, n0 + wn0, out, ldo, M, N,
+                                                      tail, prefetch_landed);
         else
             prefetch_landed();
         if (!more) break;
@@ -630,6 +641,39 @@ __global__ __launch_bounds__(256) void nibbles_to_bf6_kernel(const uint8_t *__re
     *reinterpret_cast<u32x2 *>(dst + bf6_piece(rb * 32 + (l & 31), kb, h, true, kblocks)) = u32x2{regs[4], regs[5]};
 }
 
+// bf6 weight blocks -> the checkpoint's v1 buffer: nibbles_to_bf6_kernel<true> backwards, one thread per (row-block,
+// k-block, lane).  A thread decodes its 32 codes into four 32-bit words of eight nibbles and stores them where that
+// kernel read them, so every word of the v1 buffer is written exactly once.
+__global__ __launch_bounds__(256) void bf6_to_v1_kernel(const uint8_t *__restrict__ blocks, int64_t rows, int kblocks, int dst_kblocks,
+                                                        uint8_t *__restrict__ dst, int64_t total) {
+    const int64_t idx = static_cast<int64_t>(blockIdx.x) * blockDim.x + threadIdx.x;
+    if (idx >= total) return;
+    const int l = static_cast<int>(idx & 63);
+    const int64_t blk = idx >> 6;
+    const int kb = static_cast<int>(blk % kblocks);
+    const int64_t r = (blk / kblocks) * 32 + (l & 31);
+    const int h = l >> 5;
+    if (r >= rows || kb >= dst_kblocks) return; /* padding */
+    const u32x4 a = *reinterpret_cast<const u32x4 *>(blocks + bf6_piece(r, kb, h, false, kblocks));
+    const u32x2 b = *reinterpret_cast<const u32x2 *>(blocks + bf6_piece(r, kb, h, true, kblocks));
+    const uint32_t regs[7] = {a.x, a.y, a.z, a.w, b.x, b.y, 0};
+    uint32_t w[4] = {0, 0, 0, 0};
+#pragma unroll
+    for (int e = 0; e < 32; ++e) {
+        const int bit = 6 * e, word = bit / 32, sh = bit % 32;
+        uint32_t code = regs[word] >> sh;
+        if (sh > 26) code |= regs[word + 1] << (32 - sh);
+        const uint32_t mag = code & 31u; /* |q|, 0...8 */
+        const uint32_t nib = (code & 32u) != 0 ? (0u - mag) & 0xFu : mag & 0xFu;
+        w[e / 8] |= nib << (4 * (e % 8));
+    }
+    const int r16 = static_cast<int>(r & 15);
+    const int64_t group = (((r >> 7) * dst_kblocks + kb) * 8 + ((r >> 4) & 7)) * 32 + 4 * (r16 & 7);
+    uint32_t *words = reinterpret_cast<uint32_t *>(dst);
+#pragma unroll
+    for (int t = 0; t < 4; ++t) words[(group + t) * 4 + 2 * (r16 >> 3) + h] = w[t];
+}
+
 }  // namespace
 
 int64_t bf6_kblocks(int64_t K) { return (K + 127) / 128 * 2; }
@@ -653,11 +697,21 @@ int launch_weight_v1_to_bf6(const uint8_t *qweight_v1, int64_t N, int64_t K, uin
     return check_launch("nibbles_to_bf6_kernel");
 }
 
+int launch_bf6_to_weight_v1(const uint8_t *blocks, int64_t N, int64_t K, uint8_t *qweight_v1, hipStream_t s) {
+    if (N == 0) return VDMQ_OK;
+    const int64_t kblocks = bf6_kblocks(K);
+    const int64_t total = (N + 31) / 32 * kblocks * 64;
+    hipLaunchKernelGGL(bf6_to_v1_kernel, dim3(static_cast<unsigned>(ceil_div(total, 256))), dim3(256), 0, s, blocks, N, static_cast<int>(kblocks),
+                       static_cast<int>(K / 64), qweight_v1, total);
+    return check_launch("bf6_to_v1_kernel");
+}
+
 namespace {
 
 template <class Cfg>
 int launch_bf6_cfg(const uint8_t *xblocks, const __half *ascale, const uint8_t *wblocks, const __half *wscale, const __half *bias,
-                   __half *out, int32_t *acc_out, int64_t M, int64_t N, int64_t K, int64_t ldo, const GemmTail &tail, hipStream_t s) {
+                   __half *out, bool out_bf16, int32_t *acc_out, int64_t M, int64_t N, int64_t K, int64_t ldo, const GemmTail &tail,
+                   hipStream_t s) {
     constexpr int per = 1 << Cfg::kPerLog2;
     const int tiles_m = static_cast<int>(ceil_div(M, Cfg::BM)), tiles_n = static_cast<int>(ceil_div(N, Cfg::BN));
     // Super-tile shape.  Candidates in order of preference: 8 x 4 tiles (2048 token rows x 1024 weight rows, the
@@ -706,13 +760,13 @@ int launch_bf6_cfg(const uint8_t *xblocks, const __half *ascale, const uint8_t *
     const dim3 grid(static_cast<unsigned>(rounds) * kXcds * per), block(Cfg::kWaves * 64);
     const bool stream_out = M * N * 2 > (int64_t(224) << 20);
     const bool has_tail = tail.gate != nullptr || tail.residual != nullptr;
-    const int which = acc_out != nullptr ? 2 : (stream_out ? 1 : 0) + (has_tail ? 3 : 0);
+    const int which = acc_out != nullptr ? 2 : (stream_out ? 1 : 0) + (has_tail ? 3 : out_bf16 ? 5 : 0); /* (a tail comes with fp16 only) */
     using Kernel = void (*)(const uint8_t *, const uint8_t *, const __half *, const __half *, const __half *, __half *, int32_t *, int, int,
                             int, int64_t, Bf6TileMap, GemmTail);
-    const Kernel kernels[5] = {gemm_bf6_kernel<Cfg, 0>, gemm_bf6_kernel<Cfg, 1>, gemm_bf6_kernel<Cfg, 2>, gemm_bf6_kernel<Cfg, 3>,
-                               gemm_bf6_kernel<Cfg, 4>};
+    const Kernel kernels[7] = {gemm_bf6_kernel<Cfg, 0>, gemm_bf6_kernel<Cfg, 1>, gemm_bf6_kernel<Cfg, 2>, gemm_bf6_kernel<Cfg, 3>,
+                               gemm_bf6_kernel<Cfg, 4>, gemm_bf6_kernel<Cfg, 5>, gemm_bf6_kernel<Cfg, 6>};
     constexpr int kMaxDevices = 64;
-    static bool attr_done[kMaxDevices][5] = {};
+    static bool attr_done[kMaxDevices][7] = {};
     int dev = 0;
     if (hipGetDevice(&dev) != hipSuccess || dev < 0 || dev >= kMaxDevices) return fail(VDMQ_ELAUNCH, "no current HIP device");
     if (!attr_done[dev][which]) {
@@ -740,9 +794,9 @@ int launch_bf6_cfg(const uint8_t *xblocks, const __half *ascale, const uint8_t *
         if (contig) bf6_tilemap_runs(tm, false);
         using PKernel = void (*)(const uint8_t *, const uint8_t *, const __half *, const __half *, const __half *, __half *, int, int, int,
                                  int64_t, Bf6TileMap, GemmTail);
-        const PKernel pk[5] = {gemm_bf6_persistent_kernel<Cfg, 0>, gemm_bf6_persistent_kernel<Cfg, 1>, nullptr, gemm_bf6_persistent_kernel<Cfg, 3>,
-                               gemm_bf6_persistent_kernel<Cfg, 4>};
-        static bool pattr[kMaxDevices][5] = {};
+        const PKernel pk[7] = {gemm_bf6_persistent_kernel<Cfg, 0>, gemm_bf6_persistent_kernel<Cfg, 1>, nullptr, gemm_bf6_persistent_kernel<Cfg, 3>,
+                               gemm_bf6_persistent_kernel<Cfg, 4>, gemm_bf6_persistent_kernel<Cfg, 5>, gemm_bf6_persistent_kernel<Cfg, 6>};
+        static bool pattr[kMaxDevices][7] = {};
         if (!pattr[dev][which]) {
             hipError_t e = hipFuncSetAttribute(reinterpret_cast<const void *>(pk[which]), hipFuncAttributeMaxDynamicSharedMemorySize,
                                                Cfg::kLdsBytes);
@@ -751,23 +805,30 @@ int launch_bf6_cfg(const uint8_t *xblocks, const __half *ascale, const uint8_t *
         }
         hipLaunchKernelGGL(pk[which], dim3(kXcds * per), block, Cfg::kLdsBytes, s, xblocks, wblocks, ascale, wscale, bias, out,
                            static_cast<int>(M), static_cast<int>(N), static_cast<int>(bf6_kblocks(K)), ldo, tm, tail);
-        record_gemm_launch({VDMQ_KERNEL_GEMM_BF6_PERSISTENT, Cfg::BM, Cfg::BN, per >> tm.group_n_log2, 1 << tm.group_n_log2, tm.contig, 0,
-                            static_cast<int64_t>(kXcds * per)});
-        return check_launch("gemm_bf6_persistent_kernel");
+        const int rc = check_launch("gemm_bf6_persistent_kernel");
+        if (rc == VDMQ_OK)
+            record_gemm_launch({VDMQ_KERNEL_GEMM_BF6_PERSISTENT, Cfg::BM, Cfg::BN, per >> tm.group_n_log2, 1 << tm.group_n_log2, tm.contig,
+                                static_cast<int64_t>(kXcds * per)});
+        return rc;
     }
     hipLaunchKernelGGL(kernels[which], grid, block, Cfg::kLdsBytes, s, xblocks, wblocks, ascale, wscale, bias, out, acc_out,
                        static_cast<int>(M), static_cast<int>(N), static_cast<int>(bf6_kblocks(K)), ldo, tm, tail);
-    record_gemm_launch({VDMQ_KERNEL_GEMM_BF6, Cfg::BM, Cfg::BN, per >> tm.group_n_log2, 1 << tm.group_n_log2, tm.contig, 0,
-                        static_cast<int64_t>(grid.x)});
-    return check_launch("gemm_bf6_kernel");
+    const int rc = check_launch("gemm_bf6_kernel");
+    if (rc == VDMQ_OK)
+        record_gemm_launch({VDMQ_KERNEL_GEMM_BF6, Cfg::BM, Cfg::BN, per >> tm.group_n_log2, 1 << tm.group_n_log2, tm.contig,
+                            static_cast<int64_t>(grid.x)});
+    return rc;
 }
 
 }  // namespace
 
 int launch_gemm_bf6(const uint8_t *xblocks, const __half *ascale, const uint8_t *wblocks, const __half *wscale, const __half *bias,
-                    __half *out, int32_t *acc_out, int64_t M, int64_t N, int64_t K, int64_t ldo, const GemmTail &tail, hipStream_t s) {
+                    void *out, int out_dtype, int32_t *acc_out, int64_t M, int64_t N, int64_t K, int64_t ldo, const GemmTail &tail,
+                    hipStream_t s) {
     if (M == 0 || N == 0) return VDMQ_OK;
-    return launch_bf6_cfg<Bf6Big>(xblocks, ascale, wblocks, wscale, bias, out, acc_out, M, N, K, ldo, tail, s);
+    // (both 16-bit output types go through the same staging and stores; the kernels take the pointer as fp16)
+    return launch_bf6_cfg<Bf6Big>(xblocks, ascale, wblocks, wscale, bias, static_cast<__half *>(out), out_dtype == VDMQ_OUT_BF16, acc_out, M, N,
+                                  K, ldo, tail, s);
 }
 
 }  // namespace vdmq

@@ -572,8 +572,9 @@ int launch_cfg(const uint8_t *qact, const __half *ascale, const uint8_t *wq, con
     }
     hipLaunchKernelGGL(kernels[which], grid, block, Cfg::kLdsBytes, s, qact, wq, ascale, wscale, bias, out, out_dtype, acc_out,
                        static_cast<int>(M), static_cast<int>(N), ldk, ldo, tm, tail);
-    record_gemm_launch({VDMQ_KERNEL_GEMM_W4A4, Cfg::BM, Cfg::BN, kGroupM, kGroupN, tm.contig, 0, static_cast<int64_t>(grid.x)});
-    return check_launch("gemm_w4a4_kernel");
+    const int rc = check_launch("gemm_w4a4_kernel");
+    if (rc == VDMQ_OK) record_gemm_launch({VDMQ_KERNEL_GEMM_W4A4, Cfg::BM, Cfg::BN, kGroupM, kGroupN, tm.contig, static_cast<int64_t>(grid.x)});
+    return rc;
 }
 
 }  // namespace

@@ -67,8 +67,9 @@ int64_t bf6_kblocks(int64_t K);
 int64_t bf6_bytes(int64_t rows, int64_t K);
 int launch_nibbles_to_bf6(const uint8_t *native, int64_t rows, int64_t K, uint8_t *blocks, hipStream_t stream);
 int launch_weight_v1_to_bf6(const uint8_t *qweight_v1, int64_t N, int64_t K, uint8_t *blocks, hipStream_t stream);
+int launch_bf6_to_weight_v1(const uint8_t *blocks, int64_t N, int64_t K, uint8_t *qweight_v1, hipStream_t stream);
 int launch_gemm_bf6(const uint8_t *xblocks, const __half *ascale, const uint8_t *wblocks, const __half *wscale, const __half *bias,
-                    __half *out, int32_t *acc_out, int64_t M, int64_t N, int64_t K, int64_t ldo, const GemmTail &tail,
+                    void *out, int out_dtype, int32_t *acc_out, int64_t M, int64_t N, int64_t K, int64_t ldo, const GemmTail &tail,
                     hipStream_t stream);
 
 // matrix-pipe ceiling probe (vdmq_probe.hip)

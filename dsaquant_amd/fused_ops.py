@@ -246,7 +246,7 @@ def qkv_projections_ln(attn, pre: LnInput):
 
     w, b = _cat_prepared(attn, ["to_q", "to_k", "to_v"], "qkv")
     n = attn.to_q.vdm_weight_packed.shape[0]
-    if getattr(attn, "qkv_contiguous_outputs", True):
+    if getattr(attn, "qkv_contiguous_outputs", False):
         return linear_fused(pre, w, None, None, attn.to_q.kernel_clip_ratio, bias_half=b, split_cols=n).unbind(0)
     return linear_ln_vdm_w4a4(pre, w, None, None, attn.to_q.kernel_clip_ratio, bias_half=b).split(n, dim=-1)
 
@@ -258,6 +258,6 @@ def kv_projections(attn, encoder_hidden_states):
 
     w, b = _cat_prepared(attn, ["to_k", "to_v"], "kv")
     n = attn.to_k.vdm_weight_packed.shape[0]
-    if getattr(attn, "qkv_contiguous_outputs", True):
+    if getattr(attn, "qkv_contiguous_outputs", False):
         return linear_fused(encoder_hidden_states, w, None, None, attn.to_k.kernel_clip_ratio, bias_half=b, split_cols=n).unbind(0)
     return linear_fused(encoder_hidden_states, w, None, None, attn.to_k.kernel_clip_ratio, bias_half=b).split(n, dim=-1)

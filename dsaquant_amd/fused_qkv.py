@@ -9,13 +9,19 @@ self-attention), ``use_fused_qkv_kernel`` and ``qkv_kernel_backend``; optional
 
 Self-attention: ONE activation quantization and ONE GEMM against the cached
 row-concatenation Wq|Wk|Wv, split three ways.  Cross-attention: ``to_q`` on the
-tokens, one fused K|V GEMM on the encoder states.  The concatenated weight is
-relaid once from the projections' own packed buffers into the form the kernels
-stream (no concatenated v1 copy is made); the concatenated bias is cached on
-the module under the reference's attribute name (``_vdm_qkv_bias_half`` ...).
+tokens, one fused K|V GEMM on the encoder states.  The concatenated v1 buffers
+and the concatenated bias are cached on the module under the reference's
+attribute names (``_vdm_qkv_weight_packed``, ``_vdm_qkv_weight_scale``,
+``_vdm_qkv_bias_half``, ``_vdm_kv_*``), made at first need like there
+(attention.py:44-66, 80-98); the projections' own buffers then become views of
+the concatenation, so the weights are not held twice.  Results are three views
+of one ``[..., 3N]`` tensor as in the reference; a module with
+``qkv_contiguous_outputs = True`` gets three contiguous tensors instead (the
+GEMM epilogue writes them in place: the same bits).
 """
 from __future__ import annotations
 
+import weakref
 from typing import List, Optional
 
 import torch
@@ -32,16 +38,57 @@ def fused_parts(module):
     return [["to_q", "to_k", "to_v"]] if module.cross_attention_dim_head is None else [["to_k", "to_v"]]
 
 
+_PREFIX = {("to_q", "to_k", "to_v"): "qkv", ("to_k", "to_v"): "kv"}
+
+
+def concatenated(attn, names: List[str]):
+    """``(attn._vdm_<qkv|kv>_weight_packed, attn._vdm_<qkv|kv>_weight_scale)``: the row-concatenation of the
+    projections' v1 weight and scale buffers, cached on the module under the names the reference uses and made when
+    first needed (attention.py:44-54, 80-88).  Where the projections hold their buffers as registered buffers these
+    are then replaced by views of the concatenation (same values, shapes and state-dict entries; one copy of the
+    weights instead of two).  The cache is made anew when a projection's buffer is no longer such a view, e.g.
+    after ``model.to(...)`` or a checkpoint load replaced it -- the projections' buffers are what counts."""
+    from dsaquant_amd.kernels import vdm_w4a4 as k
+
+    prefix = _PREFIX[tuple(names)]
+    w_attr, s_attr = f"_vdm_{prefix}_weight_packed", f"_vdm_{prefix}_weight_scale"
+    layers = [getattr(attn, n) for n in names]
+    cat_w, cat_s = getattr(attn, w_attr, None), getattr(attn, s_attr, None)
+    if cat_w is not None and cat_s is not None:
+        owners = [l.vdm_weight_packed.__dict__.get("_vdmq_v1_owner") for l in layers]
+        views = all(o is not None and o() is cat_w for o in owners)
+        copies = all(o is None for o in owners) and getattr(attn, "_vdm_cat_is_copy", False) and cat_w.device == layers[0].vdm_weight_packed.device
+        if views or copies:
+            return cat_w, cat_s
+    for l in layers:
+        k.ensure_v1(l.vdm_weight_packed)
+    cat_w = torch.cat([l.vdm_weight_packed for l in layers], dim=0).contiguous()
+    cat_s = torch.cat([l.vdm_weight_scale_packed for l in layers], dim=0).contiguous()
+    shared = all("vdm_weight_packed" in getattr(l, "_buffers", {}) for l in layers)
+    row = 0
+    for l in layers:
+        n = l.vdm_weight_packed.shape[0]
+        if shared:
+            if l.vdm_weight_packed.is_cuda and k.is_available():
+                k.release_prepared(l.vdm_weight_packed, concatenations=True)  # the old tensor's forms go with it
+            view_w, view_s = cat_w[row:row + n], cat_s[row:row + n]
+            view_w.__dict__["_vdmq_v1_owner"] = weakref.ref(cat_w)
+            l._buffers["vdm_weight_packed"], l._buffers["vdm_weight_scale_packed"] = view_w, view_s
+        row += n
+    attn._vdm_cat_is_copy = not shared
+    setattr(attn, w_attr, cat_w)
+    setattr(attn, s_attr, cat_s)
+    return cat_w, cat_s
+
+
 def _cat_prepared(attn, names: List[str], prefix: str):
-    """The concatenated weight of ``attn.<name>`` for the kernels and the concatenated fp16 bias (or None).  The
-    reference caches concatenated v1 buffers on the module (``_vdm_qkv_weight_packed`` ..., attention.py:44-54); the
-    kernels here never read a concatenated v1 buffer -- the operand is relaid from the projections' own buffers and
-    kept with them -- so only the bias keeps its cache attribute."""
+    """The concatenated weight of ``attn.<name>`` in the kernels' form and the concatenated fp16 bias (or None), the
+    latter cached as ``_vdm_<prefix>_bias_half`` (attention.py:55-66, 89-98)."""
     from dsaquant_amd.kernels import vdm_w4a4 as k
 
     b_attr = f"_vdm_{prefix}_bias_half"
     layers = [getattr(attn, n) for n in names]
-    weight = k._prepared([(l.vdm_weight_packed, l.vdm_weight_scale_packed) for l in layers])
+    weight = k._prepared_weight(*concatenated(attn, names))
     if getattr(attn, b_attr, None) is None:
         biases = [l._bias_half for l in layers]
         if any(b is not None for b in biases):
@@ -58,9 +105,9 @@ def _project_cat(attn, names: List[str], prefix: str, x: torch.Tensor, clip_rati
 
     weight, bias = _cat_prepared(attn, names, prefix)
     n = getattr(attn, names[0]).vdm_weight_packed.shape[0]
-    if getattr(attn, "qkv_contiguous_outputs", True):
-        # each projection's output as its own contiguous tensor, written in place by the GEMM epilogue: the values of
-        # the reference's strided views (vdm_w4a4.py:297-298) without the strides
+    if getattr(attn, "qkv_contiguous_outputs", False):
+        # opt-in: each projection's output as its own contiguous tensor, written in place by the GEMM epilogue -- the
+        # values of the reference's strided views (vdm_w4a4.py:297-298) without the strides
         return k.linear_vdm_w4a4_prepared(x, weight, bias, clip_ratio, split_cols=n).unbind(0)
     return k.linear_vdm_w4a4_prepared(x, weight, bias, clip_ratio).split(n, dim=-1)
 

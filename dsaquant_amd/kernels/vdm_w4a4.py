@@ -126,7 +126,10 @@ def k_padded(K: int) -> int:
 
 
 def _version_of(t: torch.Tensor):
-    # inference tensors do not count versions (reading ._version raises): they cannot be written in place either
+    # Inference tensors count no versions (reading ._version raises) although code under torch.inference_mode() may
+    # write them in place (copy_, load_state_dict into existing buffers).  Such a write is invisible here: whoever
+    # makes one calls release_prepared(tensor, concatenations=True); prepare_weight / prepare_model -- what the loader
+    # and enable_vdm_kernel_mode run -- do not trust a form kept on an inference tensor and make it anew.
     return None if t.is_inference() else t._version
 
 
@@ -151,6 +154,10 @@ class PreparedWeight:
         self.native: Optional[torch.Tensor] = None
         self.bf6: Optional[torch.Tensor] = None
         self._used = {"native": False, "bf6": False}
+        # name of a form -> (event recorded behind the kernels that made it, the stream they ran on, streams that have
+        # waited for the event since): a form made lazily inside a forward is made on whatever stream is current
+        # then, and a later call on another stream has to be ordered behind it
+        self._ready: Dict[str, tuple] = {}
         lib = _load_ext()
         with torch.cuda.device(self.device):
             self.wscale = torch.empty((self.N,), dtype=torch.float16, device=self.device)
@@ -158,6 +165,34 @@ class PreparedWeight:
             for (q, s), n in zip(parts, self.rows):
                 _lib.check(lib.vdmq_wscale_v1_to_plain(s.data_ptr(), self.wscale[row:].data_ptr(), n, self.K, _stream(self.device)))
                 row += n
+            self._made("wscale")
+
+    def _made(self, name: str) -> None:
+        stream = torch.cuda.current_stream(self.device)
+        if torch.cuda.is_current_stream_capturing():
+            return  # inside a graph the capture orders the work; nothing outside the graph may depend on it
+        event = torch.cuda.Event()
+        event.record(stream)
+        self._ready[name] = (event, stream.cuda_stream, set())
+
+    def _order_behind(self, name: str) -> None:
+        """Make the current stream wait for the kernels that made form ``name`` if they ran on another stream."""
+        ready = self._ready.get(name)
+        if ready is None:
+            return
+        event, made_on, waited = ready
+        stream = torch.cuda.current_stream(self.device)
+        if stream.cuda_stream == made_on or stream.cuda_stream in waited:
+            return
+        if torch.cuda.is_current_stream_capturing():
+            return  # (torch.cuda.graph synchronises the device before it starts capturing)
+        stream.wait_event(event)
+        waited.add(stream.cuda_stream)
+
+    def adopt(self, form: str, tensor: torch.Tensor) -> None:
+        """Take ``tensor``, just made on the current stream, as this weight's ``form`` ("native" or "bf6")."""
+        setattr(self, form, tensor)
+        self._made(form)
 
     def matches(self, parts) -> bool:
         if len(parts) != len(self._parts):
@@ -185,6 +220,8 @@ class PreparedWeight:
     def _build(self, form: str) -> torch.Tensor:
         lib = _load_ext()
         K = self.K
+        for q, _ in self._sources():
+            ensure_v1(q)  # (freed by release_v1: comes back from the form that is there)
         with torch.cuda.device(self.device):
             s = _stream(self.device)
             if form == "bf6":
@@ -199,22 +236,109 @@ class PreparedWeight:
             for (q, _), n in zip(self._sources(), self.rows):
                 _lib.check(convert(q.data_ptr(), flat[row * row_bytes:].data_ptr(), n, K, s))
                 row += n
+            setattr(self, form, out)
+            self._made(form)
         return out
+
+    # -- the v1 weight buffers' storage: with a prepared form resident the kernels never read them again; they only
+    # remain what state_dict() returns.  release_v1 frees their memory (the tensor objects keep shape, dtype and
+    # device: they are the module's buffers), restore_v1 brings the bytes back from the prepared form.
+    def release_v1(self) -> int:
+        """Free the storage of the packed v1 weight tensors this weight was made from (not the small scale tensors);
+        returns the bytes freed.  Needs a prepared form to restore from, and tensors that own their whole storage."""
+        if self.bf6 is None and self.native is None:
+            return 0
+        freed = 0
+        for index, (q, _) in enumerate(self._sources()):
+            storage = q.untyped_storage()
+            if "_vdmq_v1_released" in q.__dict__ or q.storage_offset() != 0 or storage.nbytes() != q.numel() * q.element_size():
+                continue
+            freed += storage.nbytes()
+            self._order_behind("bf6" if self.bf6 is not None else "native")
+            q.__dict__["_vdmq_v1_released"] = (self, index)  # (keeps this weight, i.e. the only copy of the integers, alive)
+            storage.resize_(0)
+        return freed
+
+    def restore_v1(self, index: int) -> None:
+        q = self._sources()[index][0]
+        if q.__dict__.get("_vdmq_v1_released", (None,))[0] is not self:
+            return
+        lib = _load_ext()
+        bf6 = self.bf6 is not None
+        form = self.bf6 if bf6 else self.native
+        if form is None:
+            raise _lib.VdmqError("the prepared form this packed weight was to be restored from is gone")
+        row_bytes = int(lib.vdmq_bf6_bytes(32, self.K)) // 32 if bf6 else k_padded(self.K) // 2
+        row = sum(self.rows[:index])
+        with torch.cuda.device(self.device):
+            q.untyped_storage().resize_(q.numel() * q.element_size())
+            self._order_behind("bf6" if bf6 else "native")
+            convert = lib.vdmq_bf6_to_weight_v1 if bf6 else lib.vdmq_weight_native_to_v1
+            _lib.check(convert(form.view(-1)[row * row_bytes:].data_ptr(), q.data_ptr(), self.rows[index], self.K, _stream(self.device)))
+        del q.__dict__["_vdmq_v1_released"]
 
     def operand(self, bf6: bool, eager: bool = False) -> torch.Tensor:
         """The weights as bf6 blocks (``bf6``) or native int4 rows.  ``eager``: made ahead of use -- it does not count
         as a use and drops nothing."""
         form, other = ("bf6", "native") if bf6 else ("native", "bf6")
         if getattr(self, form) is None:
-            setattr(self, form, self._build(form))
+            self._build(form)
         if not eager:
             self._used[form] = True
             if getattr(self, other) is not None and not self._used[other]:
                 setattr(self, other, None)  # made ahead for a call pattern that did not come
+                self._ready.pop(other, None)
+        self._order_behind("wscale")
+        self._order_behind(form)
         return getattr(self, form)
 
     def extra_bytes(self) -> int:
         return sum(t.numel() * t.element_size() for t in (self.native, self.bf6, self.wscale) if t is not None)
+
+
+def ensure_v1(qweight: torch.Tensor) -> None:
+    """Bring back the bytes of a packed v1 weight whose storage release_v1_storage freed (a no-op otherwise).  A
+    projection's buffer that is a view of its attention module's concatenation comes back with that."""
+    owner = qweight.__dict__.get("_vdmq_v1_owner")
+    if owner is not None and owner() is not None:
+        qweight = owner()
+    released = qweight.__dict__.get("_vdmq_v1_released")
+    if released is not None:
+        released[0].restore_v1(released[1])
+
+
+def _restore_before_state_dict(module, prefix, keep_vars) -> None:
+    ensure_v1(module.vdm_weight_packed)
+
+
+def release_v1_storage(model) -> int:
+    """Free the memory of every packed v1 weight buffer of ``model`` whose prepared form is resident: 3/4 (bf6
+    blocks) or 1/2 (native rows) byte per weight stays, instead of 1/2 more beside it.  The buffers remain the
+    modules' ``vdm_weight_packed`` (same objects, shape, dtype, device); ``state_dict()`` -- and with it
+    ``save_packed_checkpoint`` -- brings the bytes back first (vdmq_bf6_to_weight_v1 / vdmq_weight_native_to_v1
+    reproduce them exactly).  Call ``restore_v1_storage(model)`` before anything else that reads or moves the
+    buffers (``model.to(...)``, ``load_state_dict``).  Returns the bytes freed."""
+    freed = 0
+    for module in model.modules():
+        q = getattr(module, "vdm_weight_packed", None)
+        if q is None or not q.is_cuda:
+            continue
+        owner = q.__dict__.get("_vdmq_v1_owner")
+        holder = owner() if owner is not None and owner() is not None else q
+        for pw in holder.__dict__.get(_ATTR, []):
+            if pw.current() and len(pw.rows) == 1:
+                freed += pw.release_v1()
+                break
+        if "_vdmq_v1_released" in holder.__dict__ and not hasattr(module, "_vdmq_v1_hook"):
+            module._vdmq_v1_hook = module.register_state_dict_pre_hook(_restore_before_state_dict)
+    return freed
+
+
+def restore_v1_storage(model) -> None:
+    for module in model.modules():
+        q = getattr(module, "vdm_weight_packed", None)
+        if q is not None:
+            ensure_v1(q)
 
 
 _ATTR = "_vdmq_prepared"
@@ -249,6 +373,8 @@ def _prepared_weight(qweight: torch.Tensor, wscales: torch.Tensor) -> PreparedWe
 def prepare_weight(qweight: torch.Tensor, wscales: torch.Tensor, tokens: Optional[int] = None, path: Optional[str] = None) -> PreparedWeight:
     """Relayout a packed weight now (load time, a known stream) instead of at its first call.  ``tokens``: the number
     of rows its calls will have, which decides the matrix path under "auto" (default: a video-sized sequence)."""
+    if qweight.is_inference():
+        release_prepared(qweight, concatenations=True)  # written in place since? not visible: see _version_of
     pw = _prepared_weight(qweight, wscales)
     pw.operand(_use_bf6(32768 if tokens is None else int(tokens), pw.N, pw.K, path=path), eager=True)
     return pw
@@ -259,15 +385,15 @@ def prepare_model(model, tokens: Optional[int] = None, path: Optional[str] = Non
     reference attaches those buffers: packed_checkpoint.py:102-148, quant_linear.py:146-160).  Attention modules
     marked for the fused QKV / KV path get the concatenated form instead of one per projection.  Returns the bytes
     of HBM the prepared forms take beside the v1 buffers."""
-    from ..fused_qkv import fused_parts
+    from ..fused_qkv import concatenated, fused_parts
 
     done, total = set(), 0
     for module in model.modules():
         for names in fused_parts(module):
             layers = [getattr(module, n) for n in names]
-            pw = _prepared([(l.vdm_weight_packed, l.vdm_weight_scale_packed) for l in layers])
-            pw.operand(_use_bf6(32768 if tokens is None else int(tokens), pw.N, pw.K, path=path), eager=True)
-            total += pw.extra_bytes()
+            if not all(l.vdm_weight_packed.is_cuda for l in layers):
+                continue
+            total += prepare_weight(*concatenated(module, names), tokens, path).extra_bytes()
             done.update(id(l) for l in layers)
     for module in model.modules():
         if id(module) in done or not getattr(module, "use_vdm_kernel", False) or getattr(module, "vdm_weight_packed", None) is None:
@@ -283,6 +409,7 @@ def release_prepared(qweight: torch.Tensor, concatenations: bool = False) -> Non
     leads): a projection that is only ever used through its attention module's fused weight needs none of its own."""
     kept = qweight.__dict__.get(_ATTR)
     if kept is not None:
+        ensure_v1(qweight)  # a form about to go may hold the only copy of the integers
         kept[:] = [pw for pw in kept if len(pw.rows) > 1 and not concatenations]
 
 
@@ -290,10 +417,6 @@ def _native_weights(qweight: torch.Tensor, wscales: torch.Tensor) -> Tuple[torch
     """(native int4 rows, plain fp16 channel scales) of a packed weight."""
     pw = _prepared_weight(qweight, wscales)
     return pw.operand(False), pw.wscale
-
-
-def clear_native_cache() -> None:
-    """Kept for callers of the earlier cache: prepared forms now live on the packed tensors and go with them."""
 
 
 # ------------------------------------------------- which matrix instructions run the GEMM
@@ -318,9 +441,7 @@ def matrix_path() -> str:
 
 def _use_bf6(M: int, N: int, K: int, out_dtype: torch.dtype = torch.float16, path: Optional[str] = None) -> bool:
     path = _MATRIX_PATH if path is None else path
-    if path == "bf6" and out_dtype != torch.float16:
-        raise _lib.VdmqError("the bf6 matrix path writes fp16 only; use matrix path 'int8' or 'auto' for a bf16 output")
-    if out_dtype != torch.float16 or path == "int8" or M == 0:
+    if path == "int8" or M == 0:
         return False
     if path == "bf6":
         return True
@@ -380,11 +501,11 @@ def _gemm_dispatch(operand: torch.Tensor, scales: torch.Tensor, bf6: bool, weigh
     gate_p, ldg = (None, 0) if gate is None else (gate.data_ptr(), gate.stride(0))
     res_p, ldr = (None, 0) if residual is None else (residual.data_ptr(), residual.stride(0))
     w, wscale = weight.operand(bf6), weight.wscale
+    code = _lib.VDMQ_OUT_F16 if out.dtype == torch.float16 else _lib.VDMQ_OUT_BF16
     if bf6:
         _lib.check(lib.vdmq_gemm_w4a4_bf6_ex(operand.data_ptr(), scales.data_ptr(), w.data_ptr(), wscale.data_ptr(), bias_p, gate_p, ldg,
-                                             rows_per_gate, res_p, ldr, out.data_ptr(), M, N, K, out.stride(0), s))
+                                             rows_per_gate, res_p, ldr, out.data_ptr(), code, M, N, K, out.stride(0), s))
         return
-    code = _lib.VDMQ_OUT_F16 if out.dtype == torch.float16 else _lib.VDMQ_OUT_BF16
     _lib.check(lib.vdmq_gemm_w4a4_ex(operand.data_ptr(), scales.data_ptr(), w.data_ptr(), wscale.data_ptr(), bias_p, gate_p, ldg,
                                      rows_per_gate, res_p, ldr, out.data_ptr(), code, M, N, K, out.stride(0), s))
 
@@ -418,7 +539,7 @@ def pack_weight_with_scale(weight: torch.Tensor, channel_scale: torch.Tensor):
         _lib.check(lib.vdmq_wscale_plain_to_v1(scale_h.data_ptr(), packed_scales.data_ptr(), N, K, s))
     # the native form is already at hand: a first GEMM on the int8 path needs no relayout (an eager form: the bf6
     # path, if that is what the calls take, drops it)
-    _prepared([(qweight, packed_scales)]).native = native
+    _prepared([(qweight, packed_scales)]).adopt("native", native)
     return qweight, packed_scales, scale_h
 
 

@@ -153,6 +153,9 @@ class Attention(nn.Module):
         self.fused_projections = False
         self.use_fused_qkv_kernel = False
         self.qkv_kernel_backend = None
+        # q, k and v leave the fused GEMM as three contiguous tensors (the default, as in the reference, is three
+        # strided views of one [tokens, 3 * dim] tensor): rotary embedding and SDPA then read contiguous rows
+        self.qkv_contiguous_outputs = True
         self._cross_kv = {}
 
     # Cross-attention K (after norm_k) and V depend on the context only, which is the same tensor in every denoise

@@ -57,6 +57,9 @@ extern "C" {
 
 typedef void *vdmq_stream_t; /* hipStream_t */
 
+/* Version of this interface AND of the bf6 block format below: 2 = blocks hold q / 16 (code sign << 5 | |q|).  A host
+ * compares vdmq_version() with the VDMQ_VERSION it was compiled against before it hands the library blocks it kept. */
+#define VDMQ_VERSION 2
 int vdmq_version(void);
 const char *vdmq_arch(void);       /* "gfx950" */
 const char *vdmq_last_error(void); /* message of the last failure on this thread */
@@ -171,7 +174,6 @@ typedef struct vdmq_gemm_launch_info {
     int tile_m, tile_n;         /* output tile of one workgroup: token rows x channels */
     int group_m, group_n;       /* super-tile, in tiles (the bf6 kernels may regroup the tile rows and columns left over at the edges) */
     int contiguous_runs;        /* 1: each XCD walks one contiguous run of super-tiles, K direction alternating */
-    int split_k_tiles;          /* always 0: no launch splits the K range of its tiles (kept for the layout of the struct) */
     int64_t workgroups;         /* grid size */
 } vdmq_gemm_launch_info;
 int vdmq_last_gemm_launch(vdmq_gemm_launch_info *info);
@@ -227,10 +229,14 @@ int vdmq_linear_w4a4_noalloc(const void *x, int64_t M, int64_t K, int64_t ldx, f
  * and K to 128 with zeros (vdmq_bf6_bytes gives the size).  vdmq_native_to_bf6 converts a native int4
  * buffer (weights once per module; activations per call unless the quantizer
  * writes blocks itself); vdmq_gemm_w4a4_bf6 is vdmq_gemm_w4a4 on such operands
- * (fp16 output only), vdmq_gemm_w4a4_bf6_acc the int32 accumulator view.
+ * (fp16 or bf16 output), vdmq_gemm_w4a4_bf6_acc the int32 accumulator view.
  * vdmq_quantize_act_bf6 / vdmq_quantize_act_ln_bf6 are vdmq_quantize_act_ex /
  * vdmq_quantize_act_ln writing bf6 blocks (xblocks, vdmq_bf6_bytes(M, K) bytes)
- * instead of native rows: same scales, same integers; K <= 16384. */
+ * instead of native rows: same scales, same integers; K <= 16384.
+ * bf6 blocks are NOT a persistent or cross-build format: their codes changed once already (VDMQ_VERSION 1 held the
+ * integers themselves, 2 holds q / 16, and the GEMM's epilogue carries the matching factor), so blocks made by another
+ * build give results off by a power of two without any error.  They must come from this build's vdmq_quantize_act*_bf6
+ * / vdmq_native_to_bf6 / vdmq_weight_v1_to_bf6; what is stored on disk is the v1 layout. */
 int64_t vdmq_bf6_bytes(int64_t rows, int64_t K);
 /* 1 when the bf6 path is the faster one for an fp16 linear of this size (quantizer + GEMM, measured on MI355X), 0
  * otherwise: its kernel has one tile shape, 256 x 256, so it wants at least 512 output tiles -- or, when K >= 3072
@@ -246,18 +252,23 @@ int vdmq_quantize_act_ln_bf6(const void *x, int64_t M, int64_t K, int64_t ldx, f
  * native weights; workspace of vdmq_workspace_bytes_bf6(M, K) bytes. */
 int64_t vdmq_workspace_bytes_bf6(int64_t M, int64_t K);
 int vdmq_linear_w4a4_bf6(const void *x, int64_t M, int64_t K, int64_t ldx, float clip, int act, const void *wblocks, const void *wscale,
-                         const void *bias, void *out, int64_t N, int64_t ldo, void *workspace, int64_t workspace_bytes,
+                         const void *bias, void *out, int out_dtype, int64_t N, int64_t ldo, void *workspace, int64_t workspace_bytes,
                          vdmq_stream_t stream);
 int vdmq_native_to_bf6(const void *native, int64_t rows, int64_t K, void *blocks, vdmq_stream_t stream);
 /* A checkpoint's v1 weight buffer (u8 [N, K/2], weight_quantize_per_channel_kernel's order, vdm_w4a4_kernel.cu:518-551)
  * straight to bf6 blocks: the one relayout a module needs when the bf6 path serves it, made once at load.
  * Same bytes as vdmq_weight_v1_to_native followed by vdmq_native_to_bf6.  N % 128 == 0, K % 64 == 0. */
 int vdmq_weight_v1_to_bf6(const void *qweight_v1, void *wblocks, int64_t N, int64_t K, vdmq_stream_t stream);
+/* The inverse: bf6 weight blocks of this build back to the checkpoint's v1 buffer, byte for byte what vdmq_weight_v1_to_bf6
+ * was given.  A loader that keeps only the blocks resident (3/4 byte per weight instead of 1/2 + 3/4) rebuilds the
+ * state-dict tensor with it when one is asked for.  No counterpart in the reference (its kernel reads the v1 buffer). */
+int vdmq_bf6_to_weight_v1(const void *wblocks, void *qweight_v1, int64_t N, int64_t K, vdmq_stream_t stream);
+/* out_dtype VDMQ_OUT_F16 or VDMQ_OUT_BF16, with vdmq_gemm_w4a4's arithmetic for either */
 int vdmq_gemm_w4a4_bf6(const void *xblocks, const void *ascale, const void *wblocks, const void *wscale, const void *bias, void *out,
-                       int64_t M, int64_t N, int64_t K, int64_t ldo, vdmq_stream_t stream);
+                       int out_dtype, int64_t M, int64_t N, int64_t K, int64_t ldo, vdmq_stream_t stream);
 int vdmq_gemm_w4a4_bf6_ex(const void *xblocks, const void *ascale, const void *wblocks, const void *wscale, const void *bias,
-                          const void *gate, int64_t ldg, int64_t rows_per_gate, const void *residual, int64_t ldr, void *out, int64_t M,
-                          int64_t N, int64_t K, int64_t ldo, vdmq_stream_t stream); /* with vdmq_gemm_w4a4_ex's tail */
+                          const void *gate, int64_t ldg, int64_t rows_per_gate, const void *residual, int64_t ldr, void *out, int out_dtype,
+                          int64_t M, int64_t N, int64_t K, int64_t ldo, vdmq_stream_t stream); /* with vdmq_gemm_w4a4_ex's tail (fp16 only) */
 int vdmq_gemm_w4a4_bf6_split(const void *xblocks, const void *ascale, const void *wblocks, const void *wscale, const void *bias, void *out,
                              int64_t M, int64_t N, int64_t K, int64_t ldo, int64_t split_cols, int64_t part_stride,
                              vdmq_stream_t stream); /* vdmq_gemm_w4a4_split on bf6 operands */

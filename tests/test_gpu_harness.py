@@ -30,15 +30,23 @@ def test_small_dit_structure_and_numerics():
     assert len(quant) == 10 * args.num_layers  # 300 at 30 layers, as the reference's build smoke test counts
     assert sum(isinstance(m, W.Attention) and m.use_fused_qkv_kernel for m in model.modules()) == 2 * args.num_layers
     assert all(m.use_vdm_kernel and m.weight is None for m in quant)
-    # the loader relaid every weight once: the fused q|k|v and k|v weights as one operand each, nothing for the
-    # projections they replace; every prepared weight holds exactly one form
+    # the loader relaid every weight once: the fused q|k|v and k|v weights as one operand each -- made from the
+    # concatenated v1 buffers that hang on the attention module under the reference's attribute names, of which the
+    # projections' own buffers are views -- and nothing for the projections they replace; every prepared weight holds
+    # exactly one form
     prepared = []
     for blk in model.blocks:
-        for attn, lead, fused in ((blk.attn1, "to_q", ("to_k", "to_v")), (blk.attn2, "to_k", ("to_v",))):
-            kept = getattr(attn, lead).vdm_weight_packed.__dict__["_vdmq_prepared"]
-            assert [len(p.rows) for p in kept] == [1 + len(fused)]
+        for attn, cat, names in ((blk.attn1, "_vdm_qkv", ("to_q", "to_k", "to_v")), (blk.attn2, "_vdm_kv", ("to_k", "to_v"))):
+            cat_w, cat_s = getattr(attn, cat + "_weight_packed"), getattr(attn, cat + "_weight_scale")
+            kept = cat_w.__dict__["_vdmq_prepared"]
+            assert [p.rows for p in kept] == [[cat_w.shape[0]]] and cat_w.shape[0] == len(names) * args.dim
             prepared += kept
-            assert all("_vdmq_prepared" not in getattr(attn, n).vdm_weight_packed.__dict__ or not getattr(attn, n).vdm_weight_packed.__dict__["_vdmq_prepared"] for n in fused)
+            row = 0
+            for n in names:
+                part = getattr(attn, n)
+                assert not part.vdm_weight_packed.__dict__.get("_vdmq_prepared")
+                assert part.vdm_weight_packed.data_ptr() == cat_w[row:].data_ptr() and part.vdm_weight_scale_packed.data_ptr() == cat_s[row:].data_ptr()
+                row += part.vdm_weight_packed.shape[0]
         for lay in (blk.attn1.to_out[0], blk.attn2.to_q, blk.attn2.to_out[0], blk.ffn.up, blk.ffn.down):
             prepared += lay.vdm_weight_packed.__dict__["_vdmq_prepared"]
     assert len(prepared) == 7 * args.num_layers

@@ -182,27 +182,38 @@ def test_linear_leading_dims_bias_half_precedence_and_dtype():
     assert np.array_equal(y.reshape(-1, 128).cpu().numpy().view(np.uint16), want.view(np.uint16))
 
 
-def test_bf16_output_within_tolerance():
-    from dsaquant_amd import _lib
-
+@pytest.mark.parametrize("path", ["int8", "bf6"])
+@pytest.mark.parametrize("M,K,N,use_bias", [(300, 512, 256, True), (2300, 1536, 4608, False)])
+def test_bf16_output_within_tolerance(path, M, K, N, use_bias):
+    """A bf16 output (not offered by the reference) on either matrix path: the fp32 product float(acc) * (as * ws), the
+    fp16 bias added in fp32, one rounding to nearest even -- within half a bf16 ulp of the exact value plus the fp32
+    roundings, and the same bits on both paths (the larger case runs on the tile-walking bf6 kernel and the large int8
+    tiles)."""
     v = vk()
-    M, K, N = 300, 512, 256
     x, qw, ws, bias = O.synth_linear(M, K, N, seed=6)
+    if not use_bias:
+        bias = None
     qv1, sv1 = t16(O.np_pack_wgt_v1(qw)), t16(O.np_pack_wscales_v1(ws, K))  # (a prepared weight lives with its packed tensors)
     weight = v._prepared_weight(qv1, sv1)
-    y = v._linear_2d(t16(x), weight, t16(bias), 1.0, out_dtype=torch.bfloat16)
-    want, _, as_h, acc = O.np_linear(x, qw, ws, bias, 1.0)
-    exact = acc.astype(np.float64) * as_h.astype(np.float64)[:, None] * ws.astype(np.float64)[None, :] + bias.astype(np.float64)
-    err = np.abs(y.float().cpu().numpy().astype(np.float64) - exact)
-    assert err.max() <= 2.0 ** -8 * np.abs(exact).max()
-    # the bf6 matrix path writes fp16 only: asked for by name with a bf16 output it says so instead of switching paths
     old = v.matrix_path()
-    v.set_matrix_path("bf6")
+    got = {}
     try:
-        with pytest.raises(RuntimeError, match="fp16 only"):
-            v._linear_2d(t16(x), weight, t16(bias), 1.0, out_dtype=torch.bfloat16)
+        for p in ("int8", "bf6"):
+            v.set_matrix_path(p)
+            got[p] = v._linear_2d(t16(x), weight, None if bias is None else t16(bias), 1.0, out_dtype=torch.bfloat16)
+            assert got[p].dtype == torch.bfloat16
     finally:
         v.set_matrix_path(old)
+    assert torch.equal(got["int8"].view(torch.int16), got["bf6"].view(torch.int16))
+    _, _, as_h, acc = O.np_linear(x, qw, ws, bias, 1.0)
+    prod = (acc.astype(np.float32) * (as_h.astype(np.float32)[:, None] * ws.astype(np.float32)[None, :])).astype(np.float32)
+    if bias is not None:
+        prod = (prod + bias.astype(np.float32)[None, :]).astype(np.float32)
+    want = torch.from_numpy(prod).to(torch.bfloat16)  # torch rounds to nearest even
+    assert torch.equal(got[path].cpu().view(torch.int16), want.view(torch.int16))
+    exact = acc.astype(np.float64) * as_h.astype(np.float64)[:, None] * ws.astype(np.float64)[None, :] + (0 if bias is None else bias.astype(np.float64))
+    err = np.abs(got[path].float().cpu().numpy().astype(np.float64) - exact)
+    assert err.max() <= 2.0 ** -8 * np.abs(exact).max()
 
 
 def test_shape_and_dtype_errors():
@@ -773,7 +784,6 @@ def test_matrix_paths_give_the_same_fp16_outputs():
                              else v.linear_vdm_w4a4(*args, clip_ratio=0.95))
             torch.cuda.synchronize()
             assert torch.equal(got["int8"].view(torch.int16), got["bf6"].view(torch.int16)), (M, N, K, tail)
-            v.clear_native_cache()
     finally:
         v.set_matrix_path(old)
 
@@ -817,12 +827,12 @@ def test_bf6_linear_through_the_c_abi():
     wsp = torch.empty(need, dtype=torch.uint8, device=DEV)
     s = torch.cuda.current_stream().cuda_stream
     _lib.check(lib.vdmq_linear_w4a4_bf6(xs.data_ptr(), M, K, ldx, 1.0, _lib.VDMQ_ACT_GELU_TANH, wb.data_ptr(), wsd.data_ptr(), bd.data_ptr(),
-                                        out.data_ptr(), N, N, wsp.data_ptr(), need, s))
+                                        out.data_ptr(), _lib.VDMQ_OUT_F16, N, N, wsp.data_ptr(), need, s))
     torch.cuda.synchronize()
     _, table = gpu_gelu_table()
     want = O.np_linear(table[x.view(np.uint16)], qw, ws, bias, 1.0)[0]
     assert np.array_equal(out.cpu().numpy().view(np.uint16), want.view(np.uint16))
-    assert lib.vdmq_linear_w4a4_bf6(xs.data_ptr(), M, K, ldx, 1.0, 0, wb.data_ptr(), wsd.data_ptr(), bd.data_ptr(), out.data_ptr(), N, N,
+    assert lib.vdmq_linear_w4a4_bf6(xs.data_ptr(), M, K, ldx, 1.0, 0, wb.data_ptr(), wsd.data_ptr(), bd.data_ptr(), out.data_ptr(), 0, N, N,
                                     wsp.data_ptr(), need - 1, s) == -4
 
 

@@ -25,7 +25,7 @@ def test_library_exports_every_declared_symbol():
         assert hasattr(lib, name), f"libvdmq.so does not export {name}"
     assert declared == set(_lib.SIGNATURES), "ctypes signatures and header disagree"
     # pure host calls
-    assert lib.vdmq_version() >= 1
+    assert lib.vdmq_version() == _lib.VDMQ_VERSION == 2
     assert lib.vdmq_arch() == b"gfx950"
     assert lib.vdmq_k_padded(64) % 64 == 0 and lib.vdmq_k_padded(64) >= 64
     assert lib.vdmq_k_padded(5120) == 5120
@@ -257,6 +257,39 @@ def test_fused_qkv_dispatch_falls_through_to_separate_projections_on_cpu():
     attn.to_qkv = nn.Linear(128, 384)
     q, k, v = get_qkv_projections(attn, x, None)
     assert torch.equal(torch.cat([q, k, v], -1), attn.to_qkv(x))
+
+
+def test_concatenated_buffers_carry_the_reference_names_and_share_storage():
+    """fused_qkv.concatenated on CPU tensors (no kernel involved): `_vdm_qkv_weight_packed` / `_vdm_qkv_weight_scale`
+    (`_vdm_kv_*` for cross-attention) are torch.cat of the projections' v1 buffers as attention.py:44-54, 80-88 of the
+    reference builds them; the projections' buffers become views of them (state dict unchanged); a replaced buffer
+    makes the cache stale and it is rebuilt."""
+    from dsaquant_amd.checkpoints import packed_checkpoint as pc
+    from dsaquant_amd.fused_qkv import concatenated
+    from dsaquant_amd.quantization.quant_linear import QuantLinear
+
+    torch.manual_seed(1)
+    model = _Toy()
+    pc.load_packed_quantized_model(model, _synthetic_packed_ckpt(_Toy()), quant_linear_cls=QuantLinear, dtype=torch.float16,
+                                   device=torch.device("cpu"), require_vdm_kernel=False)
+    sd0 = {k: v.clone() for k, v in model.state_dict().items()}
+    attn, cross = model.blocks
+    w, s = concatenated(attn, ["to_q", "to_k", "to_v"])
+    assert w is attn._vdm_qkv_weight_packed and s is attn._vdm_qkv_weight_scale
+    assert torch.equal(w, torch.cat([sd0[f"blocks.0.{n}.vdm_weight_packed"] for n in ("to_q", "to_k", "to_v")]))
+    assert torch.equal(s, torch.cat([sd0[f"blocks.0.{n}.vdm_weight_scale_packed"] for n in ("to_q", "to_k", "to_v")]))
+    assert attn.to_k.vdm_weight_packed.data_ptr() == w[128:].data_ptr() and attn.to_k.vdm_weight_packed.is_contiguous()
+    wkv, _ = concatenated(cross, ["to_k", "to_v"])
+    assert wkv is cross._vdm_kv_weight_packed and wkv.shape == (256, 64) and not hasattr(cross, "_vdm_qkv_weight_packed")
+    assert cross.to_q.vdm_weight_packed.data_ptr() != wkv.data_ptr()
+    sd1 = model.state_dict()
+    assert set(sd1) == set(sd0) and all(torch.equal(sd1[k], sd0[k]) for k in sd0)
+    assert concatenated(attn, ["to_q", "to_k", "to_v"])[0] is w  # cached
+    # a buffer replaced behind the cache's back (what model.to(...) or a checkpoint load does)
+    new_k = torch.randint(0, 256, (128, 64), dtype=torch.uint8)
+    attn.to_k._buffers["vdm_weight_packed"] = new_k.clone()
+    w2, _ = concatenated(attn, ["to_q", "to_k", "to_v"])
+    assert w2 is not w and torch.equal(w2[128:256], new_k) and torch.equal(w2[:128], sd0["blocks.0.to_q.vdm_weight_packed"])
 
 
 # ---- the reference's torch floating-point path, from vectors recorded with its own quant_linear.py ----
