@@ -23,15 +23,26 @@ timed region.  Prints ONE JSON line.
   cpu_baseline  the torch QuantLinear floating-point path (oracle/quantlinear_torch.py,
              a restatement of the reference's CPU-runnable path) on config 0
 
-Beside the headline fields the line carries, all measured in the same run:
+Beside the headline fields the line carries, all measured in the same run (the figures a reader needs are repeated
+as flat numbers inside the `roofline` object: int8_path_*, quantizer_*, <workload>_gemm_*, <case>_*, config4_*):
   int8_path     the same workload with the GEMM forced onto the int8 matrix instructions (gemm_w4a4_kernel), with its
                 own roofline object against the 5.0 POP/s INT8 peak
   workloads     whole-step TOPS of the other block workloads (Wan-2.1 1.3B at 480p, Wan-2.2 5B) on the path the
-                library picks, with the per-linear figures
+                library picks
+  cases         single linears: config 0's fused QKV at M = 4096 (the shape the CPU baseline is timed on), the 14B
+                model's cross-attention K/V projection (M = 512 text tokens) and its fused QKV with a ragged last tile
+                (M = 75600 + 37)
+  config4       the end-to-end Wan-2.1 1.3B DiT harness (30 blocks, 32760 tokens, cond + uncond, 5 steps; bench_dit.py):
+                ms per step and the shares of the W4A4 calls and of attention
   mfma_ceiling  what the two MFMA instructions sustain in a loop with nothing else (vdmq_mfma_probe) on all-zero
                 operands, on int4-valued operands and on operands with the workload's statistics: the published peaks
                 assume the top clock, which the part does not hold under matrix load
---ubench prints only that probe (longer runs), for counter collection with rocprofv3.
+--per-linear adds the per-launch table of every workload.  --ubench prints only the probe (longer runs), for counter
+collection with rocprofv3.
+
+Weights start as a checkpoint holds them -- int4 in the v1 byte order, scales replicated per 64-deep k-group -- and go
+through the library's own load-time relayout (vdmq_weight_v1_to_bf6 / vdmq_weight_v1_to_native, vdmq_wscale_v1_to_plain),
+untimed, as a loaded module's do.
 """
 from __future__ import annotations
 
@@ -61,7 +72,7 @@ TRAFFIC_FROM_PROFILES = {
     ("wan14b_720p_block", "bf6"): {"gemm": 6432161792, "quant": 1517329408,
                                    "source": "profiles/gemm_bf6_persistent_kernel+quantize_rows_kernel.wan14b_720p_block.md"},
 }
-TRAFFIC_UNIT = "bytes leaving L2 per launch (Infinity Cache or HBM), mean of the step's four launches; from the profile named in traffic_source, not from this run"
+TRAFFIC_UNIT = "bytes leaving L2 per launch, mean of the step's 4 launches; from traffic_source, not from this run"
 HBM_PEAK_GBS = 8000.0    # MI355X HBM3E, published
 
 # (name, K, N) at M tokens
@@ -69,6 +80,11 @@ WAN14B_720P = dict(M=75600, linears=[("qkv", 5120, 15360), ("o", 5120, 5120), ("
 WAN13B_480P = dict(M=32760, linears=[("qkv", 1536, 4608), ("o", 1536, 1536), ("ffn_up", 1536, 8960), ("ffn_down", 8960, 1536)])
 WAN5B = dict(M=27280, linears=[("qkv", 3072, 9216), ("o", 3072, 3072), ("ffn_up", 3072, 14336), ("ffn_down", 14336, 3072)])
 WORKLOADS = {"wan14b_720p_block": WAN14B_720P, "wan1.3b_480p_block": WAN13B_480P, "wan5b_704x1280_block": WAN5B}
+# single linears (BASELINE configs 0 and 3), timed next to the blocks
+CASES = {"cfg0_qkv_m4096": dict(M=4096, linears=[("qkv", 1536, 4608)]),
+         "cfg3_cross_kv_m512": dict(M=512, linears=[("cross_kv", 5120, 10240)]),
+         "cfg3_qkv_ragged_m75637": dict(M=75637, linears=[("qkv", 5120, 15360)])}
+SHORT = {"wan1.3b_480p_block": "wan1p3b", "wan5b_704x1280_block": "wan5b", "wan14b_720p_block": "wan14b"}
 
 
 def quant_bytes(M, K, bf6=False):
@@ -77,9 +93,9 @@ def quant_bytes(M, K, bf6=False):
     return 2 * M * K + M * K // 2 + 2 * M
 
 
-def synth_inputs(torch, M, K, N, seed, dev):
-    """X fp16 ~ N(0,1) with 1% of channels x20; int4 weights uniform in [-7,7]
-    packed straight into the native layout; fp16 scales ~U(1e-3,1e-2); bias ~N(0,0.02)."""
+def synth_inputs(torch, lib, check, M, K, N, seed, dev, stream):
+    """X fp16 ~ N(0,1) with 1% of channels x20; int4 weights uniform in [-7,7] and fp16 scales ~U(1e-3,1e-2) as a
+    packed checkpoint holds them (v1 byte order, scales repeated per k-group); bias ~N(0,0.02)."""
     g = torch.Generator(device=dev).manual_seed(seed)
     x = torch.randn((M, K), generator=g, device=dev, dtype=torch.float32)
     cols = torch.randperm(K, generator=g, device=dev)[: -(-K // 100)]
@@ -87,10 +103,14 @@ def synth_inputs(torch, M, K, N, seed, dev):
     x = x.half()
     q = torch.randint(-7, 8, (N, K), generator=g, device=dev, dtype=torch.int32)
     nib = (q & 0xF).to(torch.uint8)
-    wq = (nib[:, 0::2] | (nib[:, 1::2] << 4)).contiguous()
+    rows = (nib[:, 0::2] | (nib[:, 1::2] << 4)).contiguous()
     ws = (1e-3 + 9e-3 * torch.rand(N, generator=g, device=dev)).half()
     bias = (0.02 * torch.randn(N, generator=g, device=dev)).half()
-    return x, wq, ws, bias
+    wq_v1 = torch.empty((N, K // 2), dtype=torch.uint8, device=dev)
+    ws_v1 = torch.empty((N, K // 64), dtype=torch.float16, device=dev)
+    check(lib.vdmq_weight_native_to_v1(rows.data_ptr(), wq_v1.data_ptr(), N, K, stream))
+    check(lib.vdmq_wscale_plain_to_v1(ws.data_ptr(), ws_v1.data_ptr(), N, K, stream))
+    return x, wq_v1, ws_v1, bias
 
 
 def cpu_baseline(torch, budget_s=16.0):
@@ -133,22 +153,27 @@ class Workload:
         from dsaquant_amd import _lib
 
         self.torch, self.lib, self._lib, self.name, self.dev = torch, lib, _lib, name, dev
-        wl = WORKLOADS[name]
+        wl = WORKLOADS.get(name) or CASES[name]
         self.M = M = wl["M"]
         self.stream = torch.cuda.current_stream(dev)
         s = self.stream.cuda_stream
         self.layers = []
         for i, (lname, K, N) in enumerate(wl["linears"]):
-            x, wq, ws, bias = synth_inputs(torch, M, K, N, seed=i, dev=dev)
+            x, wq_v1, ws_v1, bias = synth_inputs(torch, lib, _lib.check, M, K, N, seed=i, dev=dev, stream=s)
             assert v.k_padded(K) == K
             bf6 = v._use_bf6(M, N, K, path=path)
-            if bf6:  # operands of the bf6 path: 6-bit blocks (weights converted once, as a loaded module holds them)
-                wblocks = torch.empty(int(lib.vdmq_bf6_bytes(N, K)), dtype=torch.uint8, device=dev)
-                _lib.check(lib.vdmq_native_to_bf6(wq.data_ptr(), N, K, wblocks.data_ptr(), s))
-                wq = wblocks
+            # the load-time relayout of a packed checkpoint's buffers into the one form the chosen kernels stream
+            ws = torch.empty((N,), dtype=torch.float16, device=dev)
+            _lib.check(lib.vdmq_wscale_v1_to_plain(ws_v1.data_ptr(), ws.data_ptr(), N, K, s))
+            if bf6:
+                wq = torch.empty(int(lib.vdmq_bf6_bytes(N, K)), dtype=torch.uint8, device=dev)
+                _lib.check(lib.vdmq_weight_v1_to_bf6(wq_v1.data_ptr(), wq.data_ptr(), N, K, s))
                 qact = torch.empty(int(lib.vdmq_bf6_bytes(M, K)), dtype=torch.uint8, device=dev)
             else:
+                wq = torch.empty((N, K // 2), dtype=torch.uint8, device=dev)
+                _lib.check(lib.vdmq_weight_v1_to_native(wq_v1.data_ptr(), wq.data_ptr(), N, K, s))
                 qact = torch.empty((M, K // 2), dtype=torch.uint8, device=dev)
+            del wq_v1, ws_v1
             self.layers.append(dict(name=lname, K=K, N=N, x=x, wq=wq, ws=ws, bias=bias, bf6=bf6, qact=qact,
                                     scale=torch.empty((M,), dtype=torch.float16, device=dev),
                                     out=torch.empty((M, N), dtype=torch.float16, device=dev)))
@@ -220,15 +245,13 @@ class Workload:
             "path": path, "ms_per_step": ms_per_step, "step_tops": total_ops / (ms_per_step * 1e-3) / 1e12, "total_ops": total_ops,
             "roofline": {"bound": "mfma", "achieved": round(gemm_tops, 1), "peak": peak, "unit": "TOP/s", "frac": round(gemm_tops / peak, 4),
                          "frac_of_int8_peak": round(gemm_tops / INT8_PEAK_TOPS, 4), "traffic": traffic.get("gemm"),
-                         "traffic_unit": TRAFFIC_UNIT, "traffic_source": traffic.get("source"), "kernel": " + ".join(kernels),
+                         "traffic_unit": TRAFFIC_UNIT if traffic else None, "traffic_source": traffic.get("source"), "kernel": " + ".join(kernels),
                          "algorithmic_ops_per_launch": total_ops / n, "avg_launch_ms": round(gemm_ms / n, 4)},
             "quantizer": {"bound": "hbm", "achieved": round(block_bytes / quant_ms / 1e6, 1), "peak": HBM_PEAK_GBS, "unit": "GB/s",
                           "frac": round(block_bytes / quant_ms / 1e6 / HBM_PEAK_GBS, 4),
-                          "bytes_counted": "what the kernel moves: 2K in, 3K/4 (bf6 blocks) or K/2 (int4 rows) out, 2 per scale",
                           "achieved_int4_bytes": round(int4_bytes / quant_ms / 1e6, 1),
                           "frac_int4_bytes": round(int4_bytes / quant_ms / 1e6 / HBM_PEAK_GBS, 4),
-                          "int4_bytes_counted": "2MK + MK/2 + 2M per launch whatever the output form: the path's algorithmic bytes",
-                          "traffic": traffic.get("quant"), "traffic_unit": TRAFFIC_UNIT, "traffic_source": traffic.get("source"),
+                          "traffic": traffic.get("quant"),
                           "kernel": "quantize_rows_kernel", "algorithmic_bytes_per_launch": block_bytes / n,
                           "avg_launch_ms": round(quant_ms / n, 4)},
             "per_linear": per_layer,
@@ -313,13 +336,16 @@ def mfma_ceiling(torch, lib, dev, ms_target=30.0, repeats=3):
 def main():
     ap = argparse.ArgumentParser()
     ap.add_argument("--gpus", type=int, default=1)
-    ap.add_argument("--steps", type=int, default=20)
+    ap.add_argument("--steps", type=int, default=50)
     ap.add_argument("--warmup", type=int, default=5)
     ap.add_argument("--workload", default="wan14b_720p_block", choices=sorted(WORKLOADS))
     ap.add_argument("--matrix-path", default="auto", choices=["auto", "int8", "bf6"],
                     help="matrix instructions of the GEMM: auto = what the library picks for the shape")
     ap.add_argument("--no-cpu-baseline", action="store_true")
-    ap.add_argument("--no-extras", action="store_true", help="skip the int8-path run, the other workloads and the MFMA probe")
+    ap.add_argument("--no-extras", action="store_true",
+                    help="skip the int8-path run, the other workloads, the single-linear cases, the config-4 harness and the MFMA probe")
+    ap.add_argument("--no-config4", action="store_true", help="skip the end-to-end DiT harness (about 15 s)")
+    ap.add_argument("--per-linear", action="store_true", help="add the per-launch table of every workload to the line")
     ap.add_argument("--ubench", action="store_true", help="only the MFMA-only probe, 200 ms per case (for counter collection)")
     ap.add_argument("--calibrate-copy", action="store_true",
                     help="also run the library's plain 1 GiB copy kernel three times first, so that a rocprofv3 --pmc FETCH_SIZE / WRITE_SIZE "
@@ -353,10 +379,21 @@ def main():
         torch.cuda.synchronize()
         del src, dst
 
+    def run(name, path, steps, warmup):
+        w = Workload(torch, lib, v, name, path, dev)
+        r = w.measure(steps, warmup)
+        del w
+        torch.cuda.empty_cache()
+        return r
+
     wl = WORKLOADS[args.workload]
-    main_wl = Workload(torch, lib, v, args.workload, args.matrix_path, dev)
-    r = main_wl.measure(args.steps, args.warmup)
+    r = run(args.workload, args.matrix_path, args.steps, args.warmup)
     path = r["path"]
+    roof = r["roofline"]
+    # the quantizer's figures next to the GEMM's, where a reader of the roofline object finds them
+    roof.update({"quantizer_achieved_gbs": r["quantizer"]["achieved"], "quantizer_frac": r["quantizer"]["frac"],
+                 "quantizer_achieved_gbs_int4_bytes": r["quantizer"]["achieved_int4_bytes"],
+                 "quantizer_frac_int4_bytes": r["quantizer"]["frac_int4_bytes"], "quantizer_peak_gbs": HBM_PEAK_GBS})
     result = {
         "metric": "W4A4 GEMM TOPS (% INT8-MFMA peak) at Wan-14B 720p shapes; A4-quant GB/s",
         "value": round(r["step_tops"], 1), "unit": "TOPS", "n_gpus": 1, "steps": args.steps, "warmup": args.warmup,
@@ -366,35 +403,71 @@ def main():
         "data": "synthetic", "matrix_path": path,
         "config": {"workload": f"{args.workload}: M={wl['M']} tokens, linears " + ", ".join(f"{n} {k}->{o}" for n, k, o in wl["linears"])
                                + "; each = A4 quantizer + W4A4 GEMM + scale/bias epilogue, clip 1.0"},
-        "roofline": r["roofline"], "quantizer": r["quantizer"], "per_linear": r["per_linear"],
+        "roofline": roof, "quantizer": r["quantizer"],
     }
-    del main_wl
-    torch.cuda.empty_cache()
+    per_linear = {args.workload: r["per_linear"]}
     if not args.no_extras:
-        extra_steps, extra_warmup = max(3, args.steps // 4), 2
+        extra_steps, extra_warmup = max(10, args.steps // 4), 3
         if path != "int8":  # the instruction the path was specified on: the same workload on the int8 matrix path
-            w8 = Workload(torch, lib, v, args.workload, "int8", dev)
-            r8 = w8.measure(extra_steps, extra_warmup)
+            r8 = run(args.workload, "int8", extra_steps, extra_warmup)
             result["int8_path"] = {"steps": extra_steps, "warmup": extra_warmup, "step_tops": round(r8["step_tops"], 1),
-                                   "ms_per_step": round(r8["ms_per_step"], 4), "roofline": r8["roofline"], "quantizer": r8["quantizer"],
-                                   "per_linear": r8["per_linear"]}
-            del w8
-            torch.cuda.empty_cache()
+                                   "ms_per_step": round(r8["ms_per_step"], 4), "roofline": r8["roofline"], "quantizer": r8["quantizer"]}
+            per_linear[args.workload + " (int8 path)"] = r8["per_linear"]
+            roof.update({"int8_path_achieved": r8["roofline"]["achieved"], "int8_path_peak": INT8_PEAK_TOPS,
+                         "int8_path_frac": r8["roofline"]["frac"], "int8_path_kernel": r8["roofline"]["kernel"],
+                         "int8_path_quantizer_frac": r8["quantizer"]["frac"], "int8_path_step_tops": round(r8["step_tops"], 1)})
         result["workloads"] = {}
         for other in sorted(WORKLOADS):
             if other == args.workload:
                 continue
-            wo = Workload(torch, lib, v, other, args.matrix_path, dev)
-            ro = wo.measure(extra_steps, extra_warmup)
+            ro = run(other, args.matrix_path, extra_steps, extra_warmup)
             result["workloads"][other] = {"M": WORKLOADS[other]["M"], "steps": extra_steps, "warmup": extra_warmup,
                                           "step_tops": round(ro["step_tops"], 1), "ms_per_step": round(ro["ms_per_step"], 4),
                                           "gemm_tops": ro["roofline"]["achieved"], "gemm_frac": ro["roofline"]["frac"],
                                           "gemm_frac_of_int8_peak": ro["roofline"]["frac_of_int8_peak"],
-                                          "quant_gbs": ro["quantizer"]["achieved"], "quant_gbs_int4_bytes": ro["quantizer"]["achieved_int4_bytes"],
-                                          "per_linear": ro["per_linear"]}
-            del wo
-            torch.cuda.empty_cache()
-        result["mfma_ceiling"] = mfma_ceiling(torch, lib, dev)
+                                          "quant_gbs": ro["quantizer"]["achieved"], "quant_gbs_int4_bytes": ro["quantizer"]["achieved_int4_bytes"]}
+            per_linear[other] = ro["per_linear"]
+            k = SHORT[other]
+            roof.update({f"{k}_gemm_achieved": ro["roofline"]["achieved"], f"{k}_gemm_frac": ro["roofline"]["frac"],
+                         f"{k}_gemm_frac_of_int8_peak": ro["roofline"]["frac_of_int8_peak"], f"{k}_step_tops": round(ro["step_tops"], 1),
+                         f"{k}_quantizer_frac_int4_bytes": ro["quantizer"]["frac_int4_bytes"]})
+        # single linears: launches of 15 ... 2400 us, so more repetitions for the short ones
+        result["cases"] = {}
+        for case, spec in CASES.items():
+            steps_c = 200 if spec["M"] <= 4096 else extra_steps
+            rc = run(case, args.matrix_path, steps_c, 5)
+            lin = next(iter(rc["per_linear"].values()))
+            result["cases"][case] = {"M": spec["M"], "K": lin["K"], "N": lin["N"], "steps": steps_c, "kernel": lin["kernel"],
+                                     "gemm_us": round(lin["gemm_ms"] * 1e3, 2), "gemm_tops": lin["gemm_tops"],
+                                     "quant_us": round(lin["quant_ms"] * 1e3, 2), "quant_gbs_int4_bytes": lin["quant_gbs_int4_bytes"],
+                                     "linear_tops": round(rc["step_tops"], 1), "linear_us": round(rc["ms_per_step"] * 1e3, 2)}
+            roof.update({f"{case}_gemm_achieved": lin["gemm_tops"], f"{case}_gemm_frac": round(lin["gemm_tops"] / rc["roofline"]["peak"], 4),
+                         f"{case}_linear_tops": round(rc["step_tops"], 1), f"{case}_kernel": lin["kernel"]})
+        ceiling = mfma_ceiling(torch, lib, dev)
+        result["mfma_ceiling"] = ceiling
+        roof.update({"mfma_only_loop_bf6_workload_data": ceiling["bf6"]["workload"]["tops"],
+                     "mfma_only_loop_int8_workload_data": ceiling["int8"]["workload"]["tops"]})
+        if not args.no_config4:
+            import contextlib
+
+            import bench_dit
+
+            with contextlib.redirect_stdout(sys.stderr):  # (the loader reports what it loaded; this program prints one line)
+                c4 = bench_dit.measure(torch, steps=5, warmup_steps=1, fuse_ln=True, fuse_gelu=True, fuse_residual=True, reuse_context=True)
+                c4_plain = bench_dit.measure(torch, steps=2, warmup_steps=0)
+            result["config4"] = {"workload": "Wan-2.1 1.3B DiT, 30 blocks, 32760 tokens, cond + uncond, 5 steps after 1 warm-up step; LayerNorm, GELU and "
+                                             "residual updates fused into the W4A4 kernels, context quantized once",
+                                 "ms_per_step": c4["ms_per_step"], "w4a4_share": c4["value"], "attention_share": c4["attention_share"],
+                                 "w4a4_ms_per_forward": c4["w4a4_ms_per_forward"], "attention_ms_per_forward": c4["attention_ms_per_forward"],
+                                 "w4a4_calls_per_forward": c4["w4a4_calls_per_forward"], "forwards": c4["forwards"],
+                                 "unfused": {"steps": 2, "ms_per_step": c4_plain["ms_per_step"], "w4a4_share": c4_plain["value"],
+                                             "w4a4_ms_per_forward": c4_plain["w4a4_ms_per_forward"],
+                                             "w4a4_calls_per_forward": c4_plain["w4a4_calls_per_forward"]}}
+            roof.update({"config4_ms_per_step": c4["ms_per_step"], "config4_w4a4_share": c4["value"], "config4_attention_share": c4["attention_share"],
+                         "config4_w4a4_calls_per_forward": c4["w4a4_calls_per_forward"], "config4_unfused_ms_per_step": c4_plain["ms_per_step"],
+                         "config4_unfused_w4a4_share": c4_plain["value"]})
+    if args.per_linear:
+        result["per_linear"] = per_linear
     if not args.no_cpu_baseline:
         result["cpu_baseline"] = cpu_baseline(torch)
     print(json.dumps(result))

@@ -202,3 +202,52 @@ def test_first_call_after_load_can_be_captured():
             want = [layer(x), *W.get_qkv_projections(attn, x, None)]
         torch.cuda.synchronize()
         assert all(torch.equal(a, b) for a, b in zip(got, want)), it
+
+
+def test_config4_at_full_size_unfused_against_fused():
+    """The fifth benchmark configuration at its real size: the 30-block Wan-2.1 1.3B harness (dit_block.py:83-117,
+    text2video.py:522-609 of the reference) on one 32760-token sample (21 x 30 x 52 patches of a [16, 21, 60, 104]
+    latent) with a 512-token context.  One forward as the reference runs it -- 210 W4A4 calls, 7 per block -- and the
+    same forward with LayerNorm + modulation, GELU and the gated residual updates inside the W4A4 kernels and the
+    context's quantization and K/V projections kept per prompt (180 calls from the second forward of a prompt on; 186 on
+    average over the ten forwards of a five-step cond + uncond run): finite, and equal
+    within the tolerance of the small test above (the fused LayerNorm and GELU differ from torch's kernels by a few fp16
+    ulp on isolated values, which thirty blocks carry along)."""
+    from dsaquant_amd import wan_harness as W
+
+    dev = "cuda:0"
+    args = W.WAN21_1P3B
+    assert (args.num_layers, args.dim, args.ffn_dim) == (30, 1536, 8960)
+    print("config 4 at full size: building", flush=True)
+    model = W.build_quantized(args, dev, seed=0)
+    g = torch.Generator(device=dev).manual_seed(0)
+    latent = torch.randn((1, args.in_channels, 21, 60, 104), generator=g, device=dev).half()
+    ctx = torch.randn((1, 512, args.text_dim), generator=g, device=dev).half()
+    t = torch.tensor([922.0], device=dev)
+
+    def forward():
+        timers = W.KernelTimers()
+        with torch.no_grad(), W.time_w4a4_calls(timers):
+            y = model(latent, t, ctx, timers)
+        timers.collect()
+        return y, timers.counts()
+
+    print("config 4 at full size: unfused forward", flush=True)
+    y, counts = forward()
+    assert y.shape == latent.shape and torch.isfinite(y).all()
+    assert counts == {"w4a4": 210, "attention": 60}
+    saved = (W.FeedForward.fuse_gelu, W.Block.fuse_ln, W.Block.fuse_residual, W.WanDiT.reuse_context, W.Attention.cache_cross_kv)
+    W.FeedForward.fuse_gelu = W.Block.fuse_ln = W.Block.fuse_residual = True
+    W.WanDiT.reuse_context = W.Attention.cache_cross_kv = True
+    try:
+        print("config 4 at full size: fused forwards", flush=True)
+        y1, counts1 = forward()  # fills the per-prompt caches
+        y2, counts2 = forward()
+    finally:
+        W.FeedForward.fuse_gelu, W.Block.fuse_ln, W.Block.fuse_residual, W.WanDiT.reuse_context, W.Attention.cache_cross_kv = saved
+    assert counts1 == {"w4a4": 210, "attention": 60} and counts2 == {"w4a4": 180, "attention": 60}
+    assert torch.isfinite(y2).all() and torch.equal(y1, y2)
+    scale = y.float().abs().max().item()
+    err = (y2.float() - y.float()).abs().max().item()
+    print(f"config 4 at full size: max |fused - unfused| = {err:.4g}, max |y| = {scale:.4g}", flush=True)
+    assert err <= 1e-2 * scale + 1e-3
