@@ -60,6 +60,8 @@ constexpr int kXcds = kBf6Xcds;
 // columns, fetched when the tile starts so that the epilogue does not wait for them
 [[maybe_unused]] constexpr int kSideAs = 0, kSideWs = 256, kSideBias = 384;
 constexpr int kSideBytes = 512;
+// the tile-walking kernel's list of its tiles, behind the waves' side vectors: (tile_m, tile_n) per round
+constexpr int kTileTableEntries = 1024, kTileTableBytes = kTileTableEntries * 8;
 
 // Tile configuration.  BM token rows x BN weight rows per workgroup, WAVES_M x WAVES_N waves (a wave owns
 // 128 x 64: 4 x 2 MFMA tiles), STAGES ring slots of (BM + BN) / 32 row-blocks, OCC workgroups per CU.  One
@@ -74,7 +76,8 @@ struct Bf6Cfg {
     static constexpr int kStageBytes = (BM + BN) / 32 * kRbStage;
     static constexpr int kLoads = kStageBytes / 1024 / kWaves;
     static constexpr int kRingBytes = S * kStageBytes;
-    static constexpr int kLdsBytes = kRingBytes + kWaves * kSideBytes; /* stage ring + the waves' scale and bias vectors */
+    static constexpr int kTableOffset = kRingBytes + kWaves * kSideBytes;
+    static constexpr int kLdsBytes = kTableOffset + kTileTableBytes; /* stage ring + the waves' scale and bias vectors + tile list */
     static constexpr int kWaveN = NI * 32;
     static constexpr int kStageRowBytes = kWaveN * 2 + 16; /* epilogue staging: fp16 strip rows padded by 16 bytes */
     static constexpr int kStagingBytes = 32 * kStageRowBytes;
@@ -151,15 +154,19 @@ struct Bf6KLoop {
                                                  kpos * (KS / 64) * kBf6PanelKb, 0, 0);
     }
     // LOAD_B / LOAD_A: this step issues the second half of stage kt + 2 / the first half of stage kt + 3; READ_NEXT: a
-    // step follows; YOUNGER: stage kt + 2 exists, i.e. six loads may stay in flight across the barrier (-1: look at kt)
-    template <bool LOAD_B, bool LOAD_A, bool READ_NEXT, int YOUNGER>
+    // step follows; YOUNGER: stage kt + 2 exists, i.e. six loads may stay in flight across the barrier (-1: look at kt);
+    // FIRST: the tile's first step, whose first eight MFMAs start the accumulators from the constant zero, so that
+    // nobody clears 128 registers per wave between two tiles (the Wan-1.3B block's GEMMs, 12-step tiles: +2.4 %)
+    template <bool LOAD_B, bool LOAD_A, bool READ_NEXT, int YOUNGER, bool FIRST = false>
     __device__ __forceinline__ void step(int kt, int &cur, v16f (&acc)[NI][MI], v8i (&wfa)[NI], v8i (&xfa)[MI], v8i (&wfb)[NI],
                                          v8i (&xfb)[MI]) const {
         const uint8_t *stage = lds + cur * Cfg::kStageBytes;
         const int nxt = cur + 1 == S ? 0 : cur + 1, prv = cur == 0 ? S - 1 : cur - 1;
 #pragma unroll
         for (int i = 0; i < NI * MI; ++i) {
-            acc[i / MI][i % MI] = __builtin_amdgcn_mfma_scale_f32_32x32x64_f8f6f4(wfa[i / MI], xfa[i % MI], acc[i / MI][i % MI], 3, 3, 0, 0, 0, 0); /* bf6 x bf6, no scaling */
+            const v16f zero = {0.f, 0.f, 0.f, 0.f, 0.f, 0.f, 0.f, 0.f, 0.f, 0.f, 0.f, 0.f, 0.f, 0.f, 0.f, 0.f};
+            acc[i / MI][i % MI] = __builtin_amdgcn_mfma_scale_f32_32x32x64_f8f6f4(wfa[i / MI], xfa[i % MI], FIRST ? zero : acc[i / MI][i % MI], 3, 3, 0, 0,
+                                                                                 0, 0); /* bf6 x bf6, no scaling */
             if (i < NI + MI) put(wfb, xfb, i, frag_at(stage, i, 1));
             if (LOAD_B && ((kLoadSlotsB >> i) & 1)) load_one(kLoads / 2 + __builtin_popcount(kLoadSlotsB & ((1 << i) - 1)), kt + 2, prv);
             __builtin_amdgcn_sched_barrier(0);
@@ -186,10 +193,18 @@ struct Bf6KLoop {
     __device__ __forceinline__ void run(int &cur, v16f (&acc)[NI][MI], v8i (&wfa)[NI], v8i (&xfa)[MI], v8i (&wfb)[NI], v8i (&xfb)[MI]) const {
         int kt = 0;
         if (ksteps > S) {
-            step<false, true, true, 1>(0, cur, acc, wfa, xfa, wfb, xfb);
+            step<false, true, true, 1, true>(0, cur, acc, wfa, xfa, wfb, xfb);
             for (kt = 1; kt + S < ksteps; ++kt) step<true, true, true, 1>(kt, cur, acc, wfa, xfa, wfb, xfb);
             step<true, false, true, 1>(kt, cur, acc, wfa, xfa, wfb, xfb);
             ++kt;
+        } else { /* (at most three K steps: cleared the plain way; a second first-step variant here and the register
+                    allocator no longer finds one home for the accumulators of both paths) */
+#pragma unroll
+            for (int ni = 0; ni < NI; ++ni)
+#pragma unroll
+                for (int mi = 0; mi < MI; ++mi)
+#pragma unroll
+                    for (int r = 0; r < 16; ++r) acc[ni][mi][r] = 0.f;
         }
         for (; kt + 1 < ksteps; ++kt) step<false, false, true, -1>(kt, cur, acc, wfa, xfa, wfb, xfb);
         step<false, false, false, 0>(kt, cur, acc, wfa, xfa, wfb, xfb);
@@ -291,6 +306,16 @@ __device__ __forceinline__ void bf6_epilogue(const v16f (&acc)[Cfg::NI][Cfg::MI]
 }
 #endif
 
+// Timing aid, off in the shipped library: a build with -DVDMQ_DBG_TIMELINE stamps the 100 MHz clock at five points of
+// every tile of the tile-walking kernel (thread 0 of each workgroup, first 64 tiles) into a device array that
+// vdmq_debug_timeline copies out: K loop, next tile's requests, epilogue, wait at the barrier.
+#ifdef VDMQ_DBG_TIMELINE
+__device__ uint64_t g_timeline[256][64][6];
+#define VDMQ_STAMP(tile, i) do { if (threadIdx.x == 0 && (tile) < 64) g_timeline[blockIdx.x][tile][i] = wall_clock64(); } while (0)
+#else
+#define VDMQ_STAMP(tile, i) do { } while (0)
+#endif
+
 // OUT_MODE: 0 = scaled fp16 output, 1 = the same with non-temporal stores, 2 = raw accumulators as int32,
 // 3 / 4 = 0 / 1 followed by the gated residual update out = residual + y * gate (see vdmq_gemm.hip), 5 / 6 = 0 / 1 with
 // a bf16 output
@@ -352,13 +377,7 @@ __global__ __launch_bounds__(Cfg::kWaves * 64, (Cfg::kWaves * Cfg::kOcc + 3) / 4
 #pragma unroll
         for (int mi = 0; mi < MI; ++mi) xf[mi] = ld_frag(stage + ((BN / 32 + wm * MI + mi) * 2 + kb) * kBlkBytes, la, lb);
     };
-    v16f acc[NI][MI];
-#pragma unroll
-    for (int ni = 0; ni < NI; ++ni)
-#pragma unroll
-        for (int mi = 0; mi < MI; ++mi)
-#pragma unroll
-            for (int r = 0; r < 16; ++r) acc[ni][mi][r] = 0.f;
+    v16f acc[NI][MI]; /* (started from zero by the K loop's first MFMAs) */
     // weight rows are the A operand, token rows the B operand: accumulator register r of a 32 x 32
     // tile holds n = 8 * (r / 4) + 4 * (lane / 32) + r % 4, m = lane % 32
     const int ksteps = kblocks / (KS / 64);
@@ -446,13 +465,35 @@ __global__ __launch_bounds__(Cfg::kWaves * 64, (Cfg::kWaves * Cfg::kOcc + 3) / 4
         if (!bf6_tilemap_locate(tmap, st, place, tile_m, tile_n)) tile_m = -1;
         return true;
     };
+    // The workgroup's tiles, round by round, are worked out once, 512 rounds at a time by the 512 threads, and kept in
+    // LDS: between two tiles -- matrix pipes idle, every wave running the same scalar code -- finding the next tile
+    // is then one LDS read instead of the map's divisions and case distinctions (150 scalar instructions per wave
+    // and tile).  Entry: tile_m (-1: no tile at this place in that round, -2: no such round), tile_n.  Launches with
+    // more rounds than the table holds work the map out tile by tile as before.
+    int2 *tile_table = reinterpret_cast<int2 *>(lds + Cfg::kTableOffset);
+    const bool tabled = (tmap.contig ? tmap.start[xcd + 1] - tmap.start[xcd] : (tmap.total_super + kXcds - 1) / kXcds) < kTileTableEntries;
+    if (tabled) {
+        for (int e = threadIdx.x; e < kTileTableEntries; e += Cfg::kWaves * 64) {
+            int2 ent = {-2, 0};
+            if (!locate(e, ent.x, ent.y)) ent.x = -2;
+            tile_table[e] = ent;
+        }
+        __syncthreads();
+    }
     // Advances seq to the next existing tile; `skipped` counts the super-tiles passed on the way in which this place
     // has no tile (a ragged edge).
     auto next_tile = [&](int &seq, int &tile_m, int &tile_n, int &skipped) -> bool {
         skipped = 0;
         for (;;) {
             ++seq;
-            if (!locate(seq, tile_m, tile_n)) return false;
+            if (tabled) {
+                const int2 ent = tile_table[seq]; /* (seq stays below the table's size: the entry behind the last round says -2) */
+                tile_m = __builtin_amdgcn_readfirstlane(ent.x);
+                tile_n = __builtin_amdgcn_readfirstlane(ent.y);
+                if (tile_m == -2) return false;
+            } else if (!locate(seq, tile_m, tile_n)) {
+                return false;
+            }
             if (tile_m >= 0) return true;
             ++skipped;
         }
@@ -531,17 +572,14 @@ __global__ __launch_bounds__(Cfg::kWaves * 64, (Cfg::kWaves * Cfg::kOcc + 3) / 4
     }
     int cur = 0; /* ring slot of the tile's K step under work */
     v8i wfa[NI], xfa[MI], wfb[NI], xfb[MI];
+    [[maybe_unused]] int dbg_tile = 0;
     for (;;) {
         const uint64_t tile_started = wall_clock64(); /* 100 MHz */
-#pragma unroll
-        for (int ni = 0; ni < NI; ++ni)
-#pragma unroll
-            for (int mi = 0; mi < MI; ++mi)
-#pragma unroll
-                for (int r = 0; r < 16; ++r) acc[ni][mi][r] = 0.f;
+        VDMQ_STAMP(dbg_tile, 0);
         read(wfa, xfa, lds + cur * kStageBytes, 0);
         const Bf6KLoop<Cfg> k_loop{lds, src, lane_off, wave, wn, wm, la, lb, ksteps, k_reverse};
         k_loop.run(cur, acc, wfa, xfa, wfb, xfb);
+        VDMQ_STAMP(dbg_tile, 1);
 
         // ---- the next tile: its first two K steps go into slots 1 and 2 now (every wave is past the last barrier of
         // the K loop, behind which nothing reads the ring any more); slot 0 holds the epilogue's staging.  Not so when
@@ -563,6 +601,7 @@ __global__ __launch_bounds__(Cfg::kWaves * 64, (Cfg::kWaves * Cfg::kOcc + 3) / 4
             if (ksteps > 1) issue(src, next_reverse, 1, 2);
         };
         if (prefetch) request_next();
+        VDMQ_STAMP(dbg_tile, 2);
 
         // ---- fp16 epilogue of this tile.  The prefetched steps have to be in LDS, for every wave, before the next tile
         // reads them.  Loads and stores share one counter, so the wave waits for its loads before its first store --
@@ -575,6 +614,7 @@ __global__ __launch_bounds__(Cfg::kWaves * 64, (Cfg::kWaves * Cfg::kOcc + 3) / 4
                                                       tail, prefetch_landed);
         else
             prefetch_landed();
+        VDMQ_STAMP(dbg_tile, 3);
         if (!more) break;
         if (!prefetch) {
             const uint64_t now = wall_clock64(), until = now + static_cast<uint64_t>(skipped) * (now - tile_started);
@@ -584,6 +624,8 @@ __global__ __launch_bounds__(Cfg::kWaves * 64, (Cfg::kWaves * Cfg::kOcc + 3) / 4
         }
         __builtin_amdgcn_s_waitcnt(waitcnt_imm(63, 0)); /* the staging reads of this wave are done */
         lds_barrier();
+        VDMQ_STAMP(dbg_tile, 4);
+        ++dbg_tile;
         side_publish(next_side);
         if (ksteps > 2) issue(src, next_reverse, 2, 0);
         tile_m = next_m;
@@ -675,6 +717,17 @@ __global__ __launch_bounds__(256) void bf6_to_v1_kernel(const uint8_t *__restric
 }
 
 }  // namespace
+
+#ifdef VDMQ_DBG_TIMELINE
+extern "C" int vdmq_debug_timeline(void *host_out, int clear) {
+    if (clear) {
+        void *p = nullptr;
+        if (hipGetSymbolAddress(&p, HIP_SYMBOL(g_timeline)) != hipSuccess) return -1;
+        return hipMemset(p, 0, sizeof(uint64_t) * 256 * 64 * 6) == hipSuccess ? 0 : -1;
+    }
+    return hipMemcpyFromSymbol(host_out, HIP_SYMBOL(g_timeline), sizeof(uint64_t) * 256 * 64 * 6) == hipSuccess ? 0 : -1;
+}
+#endif
 
 int64_t bf6_kblocks(int64_t K) { return (K + 127) / 128 * 2; }
 int64_t bf6_bytes(int64_t rows, int64_t K) { return (rows + 31) / 32 * bf6_kblocks(K) * kBlkBytes; }

