@@ -34,6 +34,8 @@ as flat numbers inside the `roofline` object: int8_path_*, quantizer_*, <workloa
                 (M = 75600 + 37)
   config4       the end-to-end Wan-2.1 1.3B DiT harness (30 blocks, 32760 tokens, cond + uncond, 5 steps; bench_dit.py):
                 ms per step and the shares of the W4A4 calls and of attention
+  stream_ceiling  what a kernel that only streams sustains with the quantizer's mix of reads and writes over the same
+                volumes (vdmq_stream_probe), the memory system's ceiling for that mix: the quantizer is read against it
   mfma_ceiling  what the two MFMA instructions sustain in a loop with nothing else (vdmq_mfma_probe) on all-zero
                 operands, on int4-valued operands and on operands with the workload's statistics: the published peaks
                 assume the top clock, which the part does not hold under matrix load
@@ -297,6 +299,46 @@ def probe_operands(np, kind, data, rng):
     return img
 
 
+def stream_ceiling(torch, lib, dev, M, Ks, bf6, repeats=10):
+    """What a kernel that only streams sustains with the quantizer's mix of reads and writes (vdmq_stream_probe:
+    11 : 4 for 6-bit operand blocks, 4 : 1 for int4 rows; a wave reads consecutive kilobytes and writes fewer
+    consecutive ones) over the byte volumes of the workload's quantizer launches; also a plain copy and reads alone
+    at the largest volume.  GB/s of bytes moved (read + written)."""
+    from dsaquant_amd import _lib
+
+    stream = torch.cuda.current_stream(dev)
+    reads, writes = (11, 4) if bf6 else (4, 1)
+    biggest = max(M * K * 2 for K in Ks)
+    src = torch.zeros(biggest, dtype=torch.uint8, device=dev)
+    dst = torch.empty(biggest, dtype=torch.uint8, device=dev)
+
+    def timed(threads, r, w):
+        run = lambda: _lib.check(lib.vdmq_stream_probe(src.data_ptr(), dst.data_ptr(), threads, r, w, stream.cuda_stream))
+        for _ in range(2):
+            run()
+        a, b = torch.cuda.Event(enable_timing=True), torch.cuda.Event(enable_timing=True)
+        a.record(stream)
+        for _ in range(repeats):
+            run()
+        b.record(stream)
+        torch.cuda.synchronize()
+        return a.elapsed_time(b) / repeats  # ms
+
+    moved, ms, per_k = 0.0, 0.0, {}
+    for K in Ks:
+        threads = M * K * 2 // (reads * 16) // 64 * 64
+        t = timed(threads, reads, writes)
+        per_k[str(K)] = round(threads * (reads + writes) * 16 / t / 1e6, 1)
+        moved += threads * (reads + writes) * 16
+        ms += t
+    threads = biggest // 16 // 64 * 64
+    res = {"mix": f"{reads}:{writes}", "gbs": round(moved / ms / 1e6, 1), "gbs_by_row_length": per_k,
+           "copy_gbs": round(threads * 32 / timed(threads, 1, 1) / 1e6, 1), "read_only_gbs": round(threads // 4 * 64 / timed(threads // 4, 4, 0) / 1e6, 1)}
+    del src, dst
+    torch.cuda.empty_cache()
+    return res
+
+
 def mfma_ceiling(torch, lib, dev, ms_target=30.0, repeats=3):
     """TOP/s of the MFMA-only loop per instruction and operand data, HIP events around each launch."""
     import ctypes
@@ -443,6 +485,12 @@ def main():
                                      "linear_tops": round(rc["step_tops"], 1), "linear_us": round(rc["ms_per_step"] * 1e3, 2)}
             roof.update({f"{case}_gemm_achieved": lin["gemm_tops"], f"{case}_gemm_frac": round(lin["gemm_tops"] / rc["roofline"]["peak"], 4),
                          f"{case}_linear_tops": round(rc["step_tops"], 1), f"{case}_kernel": lin["kernel"]})
+        # the quantizer against a kernel that only streams the same mix of reads and writes over the same volumes
+        sc = stream_ceiling(torch, lib, dev, wl["M"], [k for _, k, _ in wl["linears"]], path != "int8")
+        result["stream_ceiling"] = sc
+        roof.update({"quantizer_stream_ceiling_gbs": sc["gbs"], "quantizer_stream_mix": sc["mix"],
+                     "quantizer_frac_of_stream_ceiling": round(r["quantizer"]["achieved"] / sc["gbs"], 4),
+                     "stream_copy_gbs": sc["copy_gbs"], "stream_read_only_gbs": sc["read_only_gbs"]})
         ceiling = mfma_ceiling(torch, lib, dev)
         result["mfma_ceiling"] = ceiling
         roof.update({"mfma_only_loop_bf6_workload_data": ceiling["bf6"]["workload"]["tops"],

@@ -73,6 +73,7 @@ SIGNATURES = {
     "vdmq_gemm_w4a4_bf6_ex": (_int, [_p, _p, _p, _p, _p, _p, _i64, _i64, _p, _i64, _p, _int, _i64, _i64, _i64, _i64, _p]),
     "vdmq_gemm_w4a4_bf6_acc": (_int, [_p, _p, _p, _i64, _i64, _i64, _p]),
     "vdmq_copy_u128": (_int, [_p, _p, _i64, _p]),
+    "vdmq_stream_probe": (_int, [_p, _p, _i64, _int, _int, _p]),
     "vdmq_mfma_probe_operand_bytes": (_i64, []),
     "vdmq_mfma_probe": (_int, [_int, _p, _i64, _i64, _p, ctypes.POINTER(ctypes.c_double), _p]),
 }

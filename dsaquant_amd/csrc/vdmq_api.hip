@@ -28,6 +28,7 @@ int check_launch(const char *what) {
 
 int launch_weight_relayout(const void *src, void *dst, int64_t N, int64_t K, bool to_native, hipStream_t s);
 int launch_copy_u128(const void *src, void *dst, int64_t bytes, hipStream_t s);
+int launch_stream_mix(const void *src, void *dst, int64_t threads, int reads, int writes, hipStream_t s);
 int launch_wscale_relayout(const void *src, void *dst, int64_t N, int64_t K, bool to_plain, hipStream_t s);
 int launch_act_to_v1(const void *qact, const void *scale_h, int64_t M, int64_t K, void *qact_v1, void *ascales_v1, hipStream_t s);
 int launch_act_to_native(const void *qact_v1, const void *ascales_v1, int64_t M, int64_t K, void *qact, void *scale_h, hipStream_t s);
@@ -548,6 +549,15 @@ int vdmq_copy_u128(const void *src, void *dst, int64_t bytes, vdmq_stream_t stre
     VDMQ_TRY(check_ptr(src, "src"));
     VDMQ_TRY(check_ptr(dst, "dst"));
     return launch_copy_u128(src, dst, bytes, as_stream(stream));
+}
+
+int vdmq_stream_probe(const void *src, void *dst, int64_t threads, int reads, int writes, vdmq_stream_t stream) {
+    if (threads < 0 || threads % 64 != 0 || threads > (int64_t(1) << 31) * 255)
+        return fail(VDMQ_ESHAPE, "threads must be a non-negative multiple of 64 (got %lld)", (long long)threads);
+    if (threads == 0) return VDMQ_OK;
+    VDMQ_TRY(check_ptr(src, "src"));
+    VDMQ_TRY(check_ptr(dst, "dst"));
+    return launch_stream_mix(src, dst, threads, reads, writes, as_stream(stream));
 }
 
 int vdmq_quantize_weight_native(const void *w, const void *scale_h, void *wq_native, int64_t N, int64_t K, vdmq_stream_t stream) {

@@ -145,6 +145,32 @@ __global__ __launch_bounds__(256) void copy_u128_kernel(const u32x4 *__restrict_
     if (i < n) dst[i] = __builtin_nontemporal_load(src + i);
 }
 
+// Streaming probe with another mix of reads and writes than the copy's 1 : 1: a wave loads READS consecutive
+// kilobytes of src (one per instruction, 16 bytes per lane) and stores WRITES consecutive kilobytes of dst derived
+// from all of them -- the quantizers' pattern: a wave reads a contiguous row and writes a shorter contiguous one.
+// With 11 : 4 it moves the A4 quantizer's 2.75 bytes read per byte written (6-bit operand blocks), with 4 : 1 the
+// int4 rows' ratio, and does nothing else: what it sustains is what the memory system gives a kernel of that mix.
+template <int READS, int WRITES>
+__global__ __launch_bounds__(256) void stream_mix_kernel(const u32x4 *__restrict__ src, u32x4 *__restrict__ dst, int64_t threads) {
+    const int64_t t = static_cast<int64_t>(blockIdx.x) * blockDim.x + threadIdx.x;
+    if (t >= threads) return;
+    const int64_t wave = t >> 6, lane = t & 63;
+    src += wave * READS * 64 + lane;
+    dst += wave * WRITES * 64 + lane;
+    u32x4 v[READS];
+#pragma unroll
+    for (int j = 0; j < READS; ++j) v[j] = __builtin_nontemporal_load(src + j * 64);
+    u32x4 x = v[0];
+#pragma unroll
+    for (int j = 1; j < READS; ++j) x ^= v[j];
+    if (WRITES == 0) asm volatile("" ::"v"(x.x), "v"(x.y), "v"(x.z), "v"(x.w)); /* (keeps the loads of a read-only run) */
+#pragma unroll
+    for (int j = 0; j < WRITES; ++j) {
+        __builtin_nontemporal_store(x, dst + j * 64);
+        x += u32x4{1u, 1u, 1u, 1u};
+    }
+}
+
 unsigned blocks_for(int64_t n) { return static_cast<unsigned>(ceil_div(n > 0 ? n : 1, 256)); }
 
 }  // namespace
@@ -155,6 +181,23 @@ int launch_copy_u128(const void *src, void *dst, int64_t bytes, hipStream_t s) {
     hipLaunchKernelGGL(copy_u128_kernel, dim3(blocks_for(n)), dim3(256), 0, s, static_cast<const u32x4 *>(src),
                        static_cast<u32x4 *>(dst), n);
     return check_launch("copy_u128_kernel");
+}
+
+int launch_stream_mix(const void *src, void *dst, int64_t threads, int reads, int writes, hipStream_t s) {
+    if (threads == 0) return VDMQ_OK;
+    const u32x4 *in = static_cast<const u32x4 *>(src);
+    u32x4 *out = static_cast<u32x4 *>(dst);
+    if (reads == 11 && writes == 4)
+        hipLaunchKernelGGL((stream_mix_kernel<11, 4>), dim3(blocks_for(threads)), dim3(256), 0, s, in, out, threads);
+    else if (reads == 4 && writes == 1)
+        hipLaunchKernelGGL((stream_mix_kernel<4, 1>), dim3(blocks_for(threads)), dim3(256), 0, s, in, out, threads);
+    else if (reads == 1 && writes == 1)
+        hipLaunchKernelGGL((stream_mix_kernel<1, 1>), dim3(blocks_for(threads)), dim3(256), 0, s, in, out, threads);
+    else if (reads == 4 && writes == 0)
+        hipLaunchKernelGGL((stream_mix_kernel<4, 0>), dim3(blocks_for(threads)), dim3(256), 0, s, in, out, threads);
+    else
+        return fail(VDMQ_EINVAL, "stream probe mixes: 11 : 4, 4 : 1, 1 : 1, 4 : 0 (got %d : %d)", reads, writes);
+    return check_launch("stream_mix_kernel");
 }
 
 int launch_weight_relayout(const void *src, void *dst, int64_t N, int64_t K, bool to_native, hipStream_t s) {
