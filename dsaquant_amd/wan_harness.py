@@ -124,11 +124,14 @@ class SharedContext:
 
 
 def _version_of(tensor: torch.Tensor):
-    # inference tensors keep no version counter (reading it raises) and cannot be written in place
     return None if tensor.is_inference() else tensor._version
 
 
 def _weak_lookup(cache: dict, tensor: torch.Tensor):
+    # A tensor made under torch.inference_mode() counts no versions (reading the counter raises) yet can still be
+    # written in place there, so nothing derived from one is reused: such a tensor is always a miss.
+    if tensor.is_inference():
+        return None
     hit = cache.get(id(tensor))
     if hit is not None and hit[0]() is tensor and hit[1] == _version_of(tensor):
         return hit[2]

@@ -11,7 +11,11 @@
  * The functions replace the six pybind entry points of the reference
  * extension (vdm_infer/kernels/csrc/vdm_w4a4_kernel.cu:924-940) and the kernel
  * launches behind them; the citation on each declaration names the part it
- * stands in for.
+ * stands in for.  Four utilities with no counterpart there live in the same
+ * library, so that measurements and the product come from one build:
+ * vdmq_copy_u128 (a plain copy), vdmq_stream_probe (a fixed mix of streamed
+ * reads and writes), vdmq_mfma_probe (a loop of matrix instructions only) and
+ * vdmq_last_gemm_launch (which kernel and tile order the launcher chose).
  *
  * Layouts
  *   "v1"      the byte order the reference's CUDA packers emit and packed
