@@ -478,8 +478,9 @@ def test_loader_errors_read_as_the_reference_loader_errors():
 
 
 def test_cache_keys_work_for_tensors_made_under_inference_mode():
-    """Inference tensors keep no version counter (reading ``_version`` raises); the caches that watch for in-place
-    writes must not read it on them."""
+    """Inference tensors keep no version counter (reading ``_version`` raises) although they can be written in place
+    under inference mode: the caches that watch for in-place writes must not read the counter on them, and must not
+    reuse anything derived from one."""
     from dsaquant_amd import wan_harness
     from dsaquant_amd.kernels import vdm_w4a4 as v
 
@@ -490,9 +491,10 @@ def test_cache_keys_work_for_tensors_made_under_inference_mode():
     assert v._version_of(t) is None and wan_harness._version_of(t) is None
     cache = {}
     wan_harness._weak_store(cache, t, "kept")
-    assert wan_harness._weak_lookup(cache, t) == "kept"
+    assert wan_harness._weak_lookup(cache, t) is None
     u = torch.zeros(4)
     wan_harness._weak_store(cache, u, "kept too")
+    assert wan_harness._weak_lookup(cache, u) == "kept too"
     u.add_(1)  # an ordinary tensor written in place is a miss
     assert wan_harness._weak_lookup(cache, u) is None
 
