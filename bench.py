@@ -69,9 +69,9 @@ FP6_PEAK_TOPS = 10100.0  # MI355X dense FP6 MFMA, published
 # or by HBM -- no counter available here separates the two -- so for the GEMM, whose operands fit that cache, this is
 # an upper bound of its HBM bytes; for the quantizer (a stream far larger than the cache) it is the HBM traffic.
 TRAFFIC_FROM_PROFILES = {
-    ("wan14b_720p_block", "int8"): {"gemm": 4315627520, "quant": 1379685376,
+    ("wan14b_720p_block", "int8"): {"gemm": 4315445555, "quant": 1379725133,
                                     "source": "profiles/gemm_w4a4_kernel+quantize_rows_kernel.wan14b_720p_block.md"},
-    ("wan14b_720p_block", "bf6"): {"gemm": 6432161792, "quant": 1517329408,
+    ("wan14b_720p_block", "bf6"): {"gemm": 6469260928, "quant": 1517356237,
                                    "source": "profiles/gemm_bf6_persistent_kernel+quantize_rows_kernel.wan14b_720p_block.md"},
 }
 TRAFFIC_UNIT = "bytes leaving L2 per launch, mean of the step's 4 launches; from traffic_source, not from this run"
@@ -301,13 +301,13 @@ def probe_operands(np, kind, data, rng):
 
 def stream_ceiling(torch, lib, dev, M, Ks, bf6, repeats=10):
     """What a kernel that only streams sustains with the quantizer's mix of reads and writes (vdmq_stream_probe:
-    11 : 4 for 6-bit operand blocks, 4 : 1 for int4 rows; a wave reads consecutive kilobytes and writes fewer
+    8 : 3 for 6-bit operand blocks, 4 : 1 for int4 rows; a wave reads consecutive kilobytes and writes fewer
     consecutive ones) over the byte volumes of the workload's quantizer launches; also a plain copy and reads alone
     at the largest volume.  GB/s of bytes moved (read + written)."""
     from dsaquant_amd import _lib
 
     stream = torch.cuda.current_stream(dev)
-    reads, writes = (11, 4) if bf6 else (4, 1)
+    reads, writes = (8, 3) if bf6 else (4, 1)
     biggest = max(M * K * 2 for K in Ks)
     src = torch.zeros(biggest, dtype=torch.uint8, device=dev)
     dst = torch.empty(biggest, dtype=torch.uint8, device=dev)
@@ -337,6 +337,38 @@ def stream_ceiling(torch, lib, dev, M, Ks, bf6, repeats=10):
     del src, dst
     torch.cuda.empty_cache()
     return res
+
+
+def quantizers_alone(torch, lib, dev, M, Ks, repeats=20):
+    """The two A4 quantizers (6-bit operand blocks, int4 rows) on the workload's row lengths, back to back launches
+    timed with HIP events: GB/s of the bytes each really moves.  For reading next to stream_ceiling in one run."""
+    from dsaquant_amd import _lib
+
+    stream = torch.cuda.current_stream(dev)
+    s = stream.cuda_stream
+    out = {"bf6_blocks": {}, "int4_rows": {}}
+    for K in Ks:
+        x = synth_inputs(torch, lib, _lib.check, M, K, 128, 7, dev, s)[0]
+        scale = torch.empty((M,), dtype=torch.float16, device=dev)
+        blocks = torch.empty((int(lib.vdmq_bf6_bytes(M, K)),), dtype=torch.uint8, device=dev)
+        rows = torch.empty((M, int(lib.vdmq_k_padded(K)) // 2), dtype=torch.uint8, device=dev)
+        forms = {"bf6_blocks": (lambda: _lib.check(lib.vdmq_quantize_act_bf6(x.data_ptr(), M, K, K, 1.0, 0, blocks.data_ptr(), scale.data_ptr(), s)),
+                                M * (2 * K + 3 * K // 4 + 2)),
+                 "int4_rows": (lambda: _lib.check(lib.vdmq_quantize_act(x.data_ptr(), M, K, K, 1.0, rows.data_ptr(), scale.data_ptr(), s)),
+                               M * (2 * K + K // 2 + 2))}
+        for name, (run, nbytes) in forms.items():
+            for _ in range(2):
+                run()
+            a, b = torch.cuda.Event(enable_timing=True), torch.cuda.Event(enable_timing=True)
+            a.record(stream)
+            for _ in range(repeats):
+                run()
+            b.record(stream)
+            torch.cuda.synchronize()
+            out[name][str(K)] = round(nbytes / (a.elapsed_time(b) / repeats) / 1e6, 1)
+        del x, scale, blocks, rows
+        torch.cuda.empty_cache()
+    return out
 
 
 def mfma_ceiling(torch, lib, dev, ms_target=30.0, repeats=3):
@@ -388,7 +420,13 @@ def main():
                     help="skip the int8-path run, the other workloads, the single-linear cases, the config-4 harness and the MFMA probe")
     ap.add_argument("--no-config4", action="store_true", help="skip the end-to-end DiT harness (about 15 s)")
     ap.add_argument("--per-linear", action="store_true", help="add the per-launch table of every workload to the line")
+    ap.add_argument("--details", action="store_true",
+                    help="add the full objects behind the flat figures of `roofline` (int8_path, workloads, cases, stream_ceiling, "
+                         "mfma_ceiling, config4); without it the line stays short")
     ap.add_argument("--ubench", action="store_true", help="only the MFMA-only probe, 200 ms per case (for counter collection)")
+    ap.add_argument("--stream-probe", action="store_true",
+                    help="only the streaming probe (reads and writes in the quantizer's proportion, nothing else) over the byte volumes "
+                         "of the workload's quantizer launches, then the quantizers themselves on the same volumes (for counter collection)")
     ap.add_argument("--calibrate-copy", action="store_true",
                     help="also run the library's plain 1 GiB copy kernel three times first, so that a rocprofv3 --pmc FETCH_SIZE / WRITE_SIZE "
                          "run holds a copy kernel of known size to scale the counters by")
@@ -410,6 +448,16 @@ def main():
     if args.ubench:
         print(json.dumps({"metric": "MFMA-only loop, TOP/s", "unit": "TOP/s", "peaks": {"int8": INT8_PEAK_TOPS, "bf6": FP6_PEAK_TOPS},
                           "mfma_ceiling": mfma_ceiling(torch, lib, dev, ms_target=200.0, repeats=3)}))
+        return
+
+    if args.stream_probe:
+        wl = WORKLOADS[args.workload]
+        Ks = sorted({k for _, k, _ in wl["linears"]})
+        print(json.dumps({"metric": "streaming probe, GB/s of bytes read + written", "unit": "GB/s", "peak": HBM_PEAK_GBS,
+                          "workload": args.workload, "M": wl["M"], "row_lengths": Ks,
+                          "bf6_blocks": stream_ceiling(torch, lib, dev, wl["M"], Ks, True, repeats=20),
+                          "int4_rows": stream_ceiling(torch, lib, dev, wl["M"], Ks, False, repeats=20),
+                          "quantizers_gbs_by_row_length": quantizers_alone(torch, lib, dev, wl["M"], Ks)}))
         return
 
     if args.calibrate_copy:
@@ -514,6 +562,9 @@ def main():
             roof.update({"config4_ms_per_step": c4["ms_per_step"], "config4_w4a4_share": c4["value"], "config4_attention_share": c4["attention_share"],
                          "config4_w4a4_calls_per_forward": c4["w4a4_calls_per_forward"], "config4_unfused_ms_per_step": c4_plain["ms_per_step"],
                          "config4_unfused_w4a4_share": c4_plain["value"]})
+    if not args.details:  # every figure of these objects that matters is a flat key of `roofline`
+        for key in ("int8_path", "workloads", "cases", "stream_ceiling", "mfma_ceiling", "config4"):
+            result.pop(key, None)
     if args.per_linear:
         result["per_linear"] = per_linear
     if not args.no_cpu_baseline:

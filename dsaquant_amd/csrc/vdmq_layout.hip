@@ -148,7 +148,7 @@ __global__ __launch_bounds__(256) void copy_u128_kernel(const u32x4 *__restrict_
 // Streaming probe with another mix of reads and writes than the copy's 1 : 1: a wave loads READS consecutive
 // kilobytes of src (one per instruction, 16 bytes per lane) and stores WRITES consecutive kilobytes of dst derived
 // from all of them -- the quantizers' pattern: a wave reads a contiguous row and writes a shorter contiguous one.
-// With 11 : 4 it moves the A4 quantizer's 2.75 bytes read per byte written (6-bit operand blocks), with 4 : 1 the
+// With 8 : 3 it moves the A4 quantizer's 2 bytes read per 3/4 byte written (6-bit operand blocks), with 4 : 1 the
 // int4 rows' ratio, and does nothing else: what it sustains is what the memory system gives a kernel of that mix.
 template <int READS, int WRITES>
 __global__ __launch_bounds__(256) void stream_mix_kernel(const u32x4 *__restrict__ src, u32x4 *__restrict__ dst, int64_t threads) {
@@ -187,8 +187,8 @@ int launch_stream_mix(const void *src, void *dst, int64_t threads, int reads, in
     if (threads == 0) return VDMQ_OK;
     const u32x4 *in = static_cast<const u32x4 *>(src);
     u32x4 *out = static_cast<u32x4 *>(dst);
-    if (reads == 11 && writes == 4)
-        hipLaunchKernelGGL((stream_mix_kernel<11, 4>), dim3(blocks_for(threads)), dim3(256), 0, s, in, out, threads);
+    if (reads == 8 && writes == 3)
+        hipLaunchKernelGGL((stream_mix_kernel<8, 3>), dim3(blocks_for(threads)), dim3(256), 0, s, in, out, threads);
     else if (reads == 4 && writes == 1)
         hipLaunchKernelGGL((stream_mix_kernel<4, 1>), dim3(blocks_for(threads)), dim3(256), 0, s, in, out, threads);
     else if (reads == 1 && writes == 1)
@@ -196,7 +196,7 @@ int launch_stream_mix(const void *src, void *dst, int64_t threads, int reads, in
     else if (reads == 4 && writes == 0)
         hipLaunchKernelGGL((stream_mix_kernel<4, 0>), dim3(blocks_for(threads)), dim3(256), 0, s, in, out, threads);
     else
-        return fail(VDMQ_EINVAL, "stream probe mixes: 11 : 4, 4 : 1, 1 : 1, 4 : 0 (got %d : %d)", reads, writes);
+        return fail(VDMQ_EINVAL, "stream probe mixes: 8 : 3, 4 : 1, 1 : 1, 4 : 0 (got %d : %d)", reads, writes);
     return check_launch("stream_mix_kernel");
 }
 

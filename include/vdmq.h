@@ -321,8 +321,8 @@ int vdmq_copy_u128(const void *src, void *dst, int64_t bytes, vdmq_stream_t stre
 /* Streaming probe with a given mix of reads and writes (no counterpart in the reference): `threads` threads (a
  * multiple of 64) each load `reads` 16-byte vectors and store `writes` vectors -- a wave reads `reads` consecutive
  * kilobytes of src and writes `writes` consecutive kilobytes of dst, as a quantizer wave reads a row and writes a
- * shorter one -- with non-temporal accesses as the quantizers use, and do nothing else.  Mixes built in: 11 : 4 (the 2.75 bytes read per
- * byte written of the A4 quantizer that writes 6-bit blocks), 4 : 1 (int4 rows), 1 : 1 (a copy), 4 : 0 (reads only;
+ * shorter one -- with non-temporal accesses as the quantizers use, and do nothing else.  Mixes built in: 8 : 3 (the 2 bytes read per
+ * 3/4 byte written of the A4 quantizer that writes 6-bit blocks), 4 : 1 (int4 rows), 1 : 1 (a copy), 4 : 0 (reads only;
  * the loaded values are combined but never stored, dst may be any valid pointer).  src holds threads * reads * 16
  * bytes, dst threads * writes * 16.  What it sustains is the memory system's ceiling for a kernel of that mix, which
  * the quantizers' rates are read against; timed by the caller. */
