@@ -445,14 +445,12 @@ int vdmq_gemm_w4a4_bf6_acc(const void *xblocks, const void *wblocks, int32_t *ac
 
 int vdmq_bf6_pays(int64_t M, int64_t N, int64_t K) {
     if (M <= 0 || N <= 0 || K <= 0) return 0;
-    // Measured, quantizer + GEMM, int8 time / bf6 time (M x K -> N).  K = 1536: 4096 -> 4608 (288 tiles) 1.02, 8192 ->
-    // 4608 (576) 1.04, 4096 -> 1536 (96) 0.91, 12000 -> 1536 (282) 0.99, 512 -> 3072 (24) 0.79.  K >= 3072 with wide N:
-    // 256 x 5120 -> 5120 (20) 1.07, 512 x 5120 -> 10240 (80) 1.37, 256 x 5120 -> 15360 1.41, 1024 x 3072 -> 9216 1.31,
-    // 512 x 3072 -> 6144 1.01, 4096 x 5120 -> 5120 1.05; with narrow N: 1024 x 3072 -> 3072 (48) 0.82, 2048 x 3072 ->
-    // 3072 (96) 1.15, 2048 x 8960 -> 1536 (48) 0.88, 4096 x 8960 -> 1536 (96) 1.05, 6000 x 14336 -> 3072 (288) 1.25.
-    constexpr int64_t kMinTiles = 512, kLongK = 3072, kWideN = 5120, kMinTilesLongK = 96;
-    const int64_t tiles = ((M + 255) / 256) * ((N + 255) / 256);
-    return tiles >= kMinTiles || (K >= kLongK && (N >= kWideN || tiles >= kMinTilesLongK)) ? 1 : 0;
+    // Measured, quantizer + GEMM, int8 time / bf6 time on 180 shapes (M 1 ... 32768, N 128 ... 15360).  K >= 1536: 1.01 ...
+    // 1.97 everywhere but one shape at 0.96 (512 x 5120 -> 10240 1.44, 4096 x 1536 -> 4608 1.01, 8192 x 5120 -> 10240
+    // 1.42, 100 x 5120 -> 15360 1.97).  K = 1280: 1.05 ... 1.36 on 12 of 16 shapes, 0.80 ... 0.98 on four.  K = 1024: 11 : 5,
+    // K = 768: 9 : 7 (0.76 ... 1.27); K <= 512: 0.73 ... 1.03 -- the quantizer that writes blocks is the slower one on short
+    // rows and decides such a linear.  M and N no longer matter since the GEMM has a small-tile configuration.
+    return K >= 1280 ? 1 : 0;
 }
 
 int64_t vdmq_workspace_bytes_bf6(int64_t M, int64_t K) {

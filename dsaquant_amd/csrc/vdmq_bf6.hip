@@ -64,11 +64,12 @@ constexpr int kSideBytes = 512;
 constexpr int kTileTableEntries = 1024, kTileTableBytes = kTileTableEntries * 8;
 
 // Tile configuration.  BM token rows x BN weight rows per workgroup, WAVES_M x WAVES_N waves (a wave owns
-// 128 x 64: 4 x 2 MFMA tiles), STAGES ring slots of (BM + BN) / 32 row-blocks, OCC workgroups per CU.  One
-// configuration is instantiated: one workgroup of eight waves owns the CU, the fewest operand bytes per MAC.
-// (128 x 256 tiles with two workgroups of four waves per CU, so that one's prologue and epilogue run under the
-// other's K loop, measured 2...10 % slower on every shape down to K = 1536, with and without a start offset
-// between the two.)
+// 128 x 64 or 64 x 64: 4 x 2 or 2 x 2 MFMA tiles), STAGES ring slots of (BM + BN) / 32 row-blocks, OCC workgroups
+// per CU.  Two configurations are instantiated.  Big: one workgroup of eight waves owns the CU, the fewest operand
+// bytes per MAC.  (128 x 256 tiles with two workgroups of four waves per CU, so that one's prologue and epilogue run
+// under the other's K loop, measured 2...10 % slower on every shape down to K = 1536, with and without a start
+// offset between the two.)  Small: 128 x 128 tiles, two workgroups of four waves per CU, for problems that cannot
+// give every CU a big tile; only the one-workgroup-per-tile kernel has it.
 template <int BM_, int BN_, int WAVES_M_, int WAVES_N_, int STAGES_, int OCC_>
 struct Bf6Cfg {
     static constexpr int BM = BM_, BN = BN_, kWavesM = WAVES_M_, kWavesN = WAVES_N_, kWaves = WAVES_M_ * WAVES_N_, S = STAGES_, kOcc = OCC_;
@@ -78,18 +79,20 @@ struct Bf6Cfg {
     static constexpr int kRingBytes = S * kStageBytes;
     static constexpr int kTableOffset = kRingBytes + kWaves * kSideBytes;
     static constexpr int kLdsBytes = kTableOffset + kTileTableBytes; /* stage ring + the waves' scale and bias vectors + tile list */
+    static constexpr int kLdsBytesOneTile = kTableOffset;            /* the one-workgroup-per-tile kernel keeps no list */
     static constexpr int kWaveN = NI * 32;
     static constexpr int kStageRowBytes = kWaveN * 2 + 16; /* epilogue staging: fp16 strip rows padded by 16 bytes */
     static constexpr int kStagingBytes = 32 * kStageRowBytes;
     static constexpr int kPiecesPerRow = kWaveN / 8;
     static constexpr int kPerLog2 = BM == 256 ? 5 : 6; /* tiles per super-tile: what an XCD's 32 CUs hold at once */
-    static_assert(MI == 4 && NI == 2, "the schedule below is written for 128 x 64 wave tiles");
+    static_assert((MI == 4 || MI == 2) && NI == 2, "the schedule below is written for 128 x 64 and 64 x 64 wave tiles");
     static_assert(kStagingBytes * kWaves <= kRingBytes, "epilogue staging reuses the stage ring");
     static_assert(kStageBytes % (1024 * kWaves) == 0, "stage splits evenly over the waves");
     static_assert(kLoads * (S - 1) < 64, "vmcnt is a 6-bit counter");
-    static_assert(kLdsBytes * kOcc <= 160 * 1024, "the CU's LDS holds OCC workgroups");
+    static_assert((kOcc == 1 ? kLdsBytes : kLdsBytesOneTile) * kOcc <= 160 * 1024, "the CU's LDS holds OCC workgroups");
 };
 using Bf6Big = Bf6Cfg<256, 256, 2, 4, 3, 1>;
+using Bf6Small = Bf6Cfg<128, 128, 2, 2, 3, 2>;
 
 // workgroup b runs on XCD b % 8; each XCD walks super-tiles (vdmq_bf6_tilemap.h)
 [[maybe_unused]] __device__ __forceinline__ bool map_tile(const Bf6TileMap &tm, int bid, int &tile_m, int &tile_n) {
@@ -126,11 +129,12 @@ using Bf6Big = Bf6Cfg<256, 256, 2, 4, 3, 1>;
 template <class Cfg>
 struct Bf6KLoop {
     static constexpr int NI = Cfg::NI, MI = Cfg::MI, S = Cfg::S, kLoads = Cfg::kLoads, kWaves = Cfg::kWaves, BN = Cfg::BN;
-    static_assert(NI == 2 && MI == 4 && kLoads == 6 && S == 3, "the schedule is written for this shape");
+    static_assert(NI == 2 && (MI == 4 || MI == 2) && kLoads == 6 && S == 3, "the schedule is written for these shapes");
     // MFMAs of a k-block (bit i = behind the i-th) that are followed by a load: behind the 2nd, 4th and 6th in the first
     // k-block, the 3rd, 5th and 7th in the second.  Measured against other triples: a load behind a k-block's first
     // MFMA (right after the barrier, or the loop's head) costs 2 %, the rest lie within 1 %.
-    static constexpr unsigned kLoadSlotsB = 0x2A, kLoadSlotsA = 0x54;
+    // (64 x 64 wave tiles have four MFMAs per k-block: behind the 2nd, 3rd and 4th)
+    static constexpr unsigned kLoadSlotsB = MI == 4 ? 0x2A : 0xE, kLoadSlotsA = MI == 4 ? 0x54 : 0xE;
     uint8_t *lds;
     const __amdgpu_buffer_rsrc_t (&src)[kLoads];
     const uint32_t (&lane_off)[kLoads];
@@ -765,8 +769,14 @@ template <class Cfg>
 int launch_bf6_cfg(const uint8_t *xblocks, const __half *ascale, const uint8_t *wblocks, const __half *wscale, const __half *bias,
                    __half *out, bool out_bf16, int32_t *acc_out, int64_t M, int64_t N, int64_t K, int64_t ldo, const GemmTail &tail,
                    hipStream_t s) {
-    constexpr int per = 1 << Cfg::kPerLog2;
     const int tiles_m = static_cast<int>(ceil_div(M, Cfg::BM)), tiles_n = static_cast<int>(ceil_div(N, Cfg::BN));
+    // Places per super-tile: what an XCD's CUs hold at once.  The small configuration's problems are few such
+    // super-tiles, mostly partly empty ones (M = 512: 4 tile rows in a shape of 16 x 4, so 16 tiles per super-tile);
+    // measured against both alternatives on M = 512, K = 5120, N = 10240 (320 tiles; 25.8 us as it is): the edges
+    // regrouped into five full super-tiles 28.1 us, super-tiles of four dealt over all XCDs 31.7 us (K = 3072, N = 6144:
+    // 11.2 / 18.2 / 13.2 us) -- two workgroups that share a CU keep its matrix pipes busier than one each on two CUs,
+    // and five XCDs are too few.
+    constexpr int per_log2 = Cfg::kPerLog2, per = 1 << per_log2;
     // Super-tile shape.  Candidates in order of preference: 8 x 4 tiles (2048 token rows x 1024 weight rows, the
     // fewest operand bytes per tile and measured best wherever the work is even), the same with the edge super-tiles
     // regrouped (fuller, so fewer of them), 16 x 2, 16 x 2 regrouped.  A later one replaces an earlier one when it
@@ -781,7 +791,7 @@ int launch_bf6_cfg(const uint8_t *xblocks, const __half *ascale, const uint8_t *
     int64_t best_load = -1, best_rounds = 0;
     for (int variant = 0; variant < 4; variant += small ? 2 : 1) {
         Bf6TileMap cand;
-        bf6_tilemap_shape(cand, tiles_m, tiles_n, Cfg::kPerLog2, 2 - variant / 2, variant % 2 != 0);
+        bf6_tilemap_shape(cand, tiles_m, tiles_n, per_log2, 2 - variant / 2, variant % 2 != 0);
         int64_t load[kXcds] = {};
         const bool modelled = cand.total_super <= 4096; /* beyond that the edges no longer matter: the first shape is taken */
         if (modelled)
@@ -824,8 +834,8 @@ int launch_bf6_cfg(const uint8_t *xblocks, const __half *ascale, const uint8_t *
     if (hipGetDevice(&dev) != hipSuccess || dev < 0 || dev >= kMaxDevices) return fail(VDMQ_ELAUNCH, "no current HIP device");
     if (!attr_done[dev][which]) {
         hipError_t e = hipFuncSetAttribute(reinterpret_cast<const void *>(kernels[which]), hipFuncAttributeMaxDynamicSharedMemorySize,
-                                           Cfg::kLdsBytes);
-        if (e != hipSuccess) return fail(VDMQ_ELAUNCH, "hipFuncSetAttribute(%d bytes of LDS): %s", Cfg::kLdsBytes, hipGetErrorString(e));
+                                           Cfg::kLdsBytesOneTile);
+        if (e != hipSuccess) return fail(VDMQ_ELAUNCH, "hipFuncSetAttribute(%d bytes of LDS): %s", Cfg::kLdsBytesOneTile, hipGetErrorString(e));
         attr_done[dev][which] = true;
     }
     // The persistent kernel gives every CU position a fixed share -- its place in each super-tile of the XCD's
@@ -842,8 +852,8 @@ int launch_bf6_cfg(const uint8_t *xblocks, const __half *ascale, const uint8_t *
     if (cu_count[dev] == 0 && hipDeviceGetAttribute(&cu_count[dev], hipDeviceAttributeMultiprocessorCount, dev) != hipSuccess) cu_count[dev] = -1;
     // (its contiguous runs hold equal numbers of super-tiles: a round each, however full)
     const int64_t rounds_p = ceil_div(total_super, kXcds);
-    const bool persistent = which != 2 && cu_count[dev] == kXcds * per && rounds_p * 100 <= ceil_div(busiest, per) * 115;
-    if (persistent) {
+    const bool persistent = Cfg::kOcc == 1 && which != 2 && cu_count[dev] == kXcds * per && rounds_p * 100 <= ceil_div(busiest, per) * 115;
+    if constexpr (Cfg::kOcc == 1) if (persistent) {
         if (contig) bf6_tilemap_runs(tm, false);
         using PKernel = void (*)(const uint8_t *, const uint8_t *, const __half *, const __half *, const __half *, __half *, int, int, int,
                                  int64_t, Bf6TileMap, GemmTail);
@@ -864,7 +874,7 @@ int launch_bf6_cfg(const uint8_t *xblocks, const __half *ascale, const uint8_t *
                                 static_cast<int64_t>(kXcds * per)});
         return rc;
     }
-    hipLaunchKernelGGL(kernels[which], grid, block, Cfg::kLdsBytes, s, xblocks, wblocks, ascale, wscale, bias, out, acc_out,
+    hipLaunchKernelGGL(kernels[which], grid, block, Cfg::kLdsBytesOneTile, s, xblocks, wblocks, ascale, wscale, bias, out, acc_out,
                        static_cast<int>(M), static_cast<int>(N), static_cast<int>(bf6_kblocks(K)), ldo, tm, tail);
     const int rc = check_launch("gemm_bf6_kernel");
     if (rc == VDMQ_OK)
@@ -880,6 +890,13 @@ int launch_gemm_bf6(const uint8_t *xblocks, const __half *ascale, const uint8_t 
                     hipStream_t s) {
     if (M == 0 || N == 0) return VDMQ_OK;
     // (both 16-bit output types go through the same staging and stores; the kernels take the pointer as fp16)
+    // Problems of at most half a 256 x 256 tile per CU take 128 x 128 tiles, two workgroups of four waves per CU: four
+    // times as many workgroups for the same K loop.  Measured on 150 shapes (M 1...32768, N 128...15360, K 64...13824):
+    // up to 128 big tiles the small ones take 0.46...0.9 of the time (512 x 5120 -> 10240: 28 -> 25 us, 512 x 1536 ->
+    // 3072: 13.7 -> 7.3 us), from 160 on 1.0...1.4.
+    if (ceil_div(M, Bf6Big::BM) * ceil_div(N, Bf6Big::BN) <= kXcds * 32 / 2)
+        return launch_bf6_cfg<Bf6Small>(xblocks, ascale, wblocks, wscale, bias, static_cast<__half *>(out), out_dtype == VDMQ_OUT_BF16, acc_out, M,
+                                        N, K, ldo, tail, s);
     return launch_bf6_cfg<Bf6Big>(xblocks, ascale, wblocks, wscale, bias, static_cast<__half *>(out), out_dtype == VDMQ_OUT_BF16, acc_out, M, N,
                                   K, ldo, tail, s);
 }

@@ -242,11 +242,11 @@ int vdmq_linear_w4a4_noalloc(const void *x, int64_t M, int64_t K, int64_t ldx, f
  * build give results off by a power of two without any error.  They must come from this build's vdmq_quantize_act*_bf6
  * / vdmq_native_to_bf6 / vdmq_weight_v1_to_bf6; what is stored on disk is the v1 layout. */
 int64_t vdmq_bf6_bytes(int64_t rows, int64_t K);
-/* 1 when the bf6 path is the faster one for an fp16 linear of this size (quantizer + GEMM, measured on MI355X), 0
- * otherwise: its kernel has one tile shape, 256 x 256, so it wants at least 512 output tiles -- or, when K >= 3072
- * lets the K loop outweigh a tile's prologue and epilogue, N >= 5120 or at least 96 tiles.  A host that keeps both
- * weight forms asks this per call; the results are the same bits either way.  No counterpart in the reference (it
- * has one matrix path). */
+/* 1 when the bf6 path is the faster one for a linear of this size (quantizer + GEMM, measured on MI355X), 0
+ * otherwise.  Its GEMM has 256 x 256 tiles for large problems and 128 x 128 ones for small ones and is the faster
+ * GEMM on every shape measured; what decides is the quantizer, which is slower than the int4 one on short rows: the
+ * path pays from K = 1280 on, whatever M and N.  A host that keeps both weight forms asks this per call; the results
+ * are the same bits either way.  No counterpart in the reference (it has one matrix path). */
 int vdmq_bf6_pays(int64_t M, int64_t N, int64_t K);
 int vdmq_quantize_act_bf6(const void *x, int64_t M, int64_t K, int64_t ldx, float clip, int act, void *xblocks, void *scale_h,
                           vdmq_stream_t stream);

@@ -10,9 +10,9 @@ in seconds, so each case checks
 * rows are independent: the first 4113 rows of the full run equal a run on those rows alone (another launch
   geometry, other tiles, another tile order);
 * which kernel and tile order the library chose, where the choice has special cases: the bf6 path's kernel that walks
-  tiles (also where tile rows or columns are left over and regrouped), the one-workgroup-per-tile kernel it falls back
-  to on small problems, 16 x 2 super-tiles for six tile columns, contiguous runs for wide N; the int8 path's three
-  tile shapes.
+  tiles (also where tile rows or columns are left over and regrouped), the one-workgroup-per-tile kernel with
+  128 x 128 tiles that small problems take, 16 x 2 super-tiles for six tile columns, contiguous runs for wide N; the
+  int8 path's three tile shapes.
 """
 import numpy as np
 import pytest
@@ -32,14 +32,14 @@ CASES = [
     ("cfg1", "o", 32760, 1536, 1536, 1, {"int8": (W4, 256, 128, 4, 0), "bf6": (BF6P, 256, 256, 4, 0)}),       # six tile columns: four as 8 x 4, two as 16 x 2
     ("cfg1", "ffn_up", 32760, 1536, 8960, 1, {"int8": (W4, 256, 256, 4, 0), "bf6": (BF6P, 256, 256, 4, 0)}),
     ("cfg1", "ffn_down", 32760, 8960, 1536, 1, {"int8": (W4, 256, 128, 4, 0), "bf6": (BF6P, 256, 256, 4, 0)}),
-    ("cfg1", "cross_kv", 512, 1536, 3072, 1, {"int8": (W4, 128, 128, 4, 0), "bf6": (BF6P, 256, 256, 2, 0)}),
+    ("cfg1", "cross_kv", 512, 1536, 3072, 1, {"int8": (W4, 128, 128, 4, 0), "bf6": (BF6, 128, 128, 4, 0)}),
     ("cfg2", "qkv", 27280, 3072, 9216, 2, {"int8": (W4, 256, 256, 4, 1), "bf6": (BF6P, 256, 256, 4, 0)}),
     ("cfg2", "o", 27280, 3072, 3072, 2, {"int8": (W4, 256, 256, 4, 1), "bf6": (BF6P, 256, 256, 4, 0)}),
     ("cfg2", "ffn_up", 27280, 3072, 14336, 2, {"int8": (W4, 256, 256, 4, 1), "bf6": (BF6P, 256, 256, 4, 1)}),  # three tile rows left over: regrouped
     ("cfg2", "ffn_down", 27280, 14336, 3072, 2, {"int8": (W4, 256, 256, 4, 1), "bf6": (BF6P, 256, 256, 4, 0)}),
     ("cfg3", "o", 75600, 5120, 5120, 1, {"int8": (W4, 256, 256, 4, 1), "bf6": (BF6P, 256, 256, 4, 0)}),
     ("cfg3", "ffn_up", 75600, 5120, 13824, 1, {"int8": (W4, 256, 256, 4, 1), "bf6": (BF6P, 256, 256, 4, 1)}),
-    ("cfg3", "cross_kv", 512, 5120, 10240, 1, {"int8": (W4, 128, 128, 4, 0), "bf6": (BF6, 256, 256, 2, 0)}),
+    ("cfg3", "cross_kv", 512, 5120, 10240, 1, {"int8": (W4, 128, 128, 4, 0), "bf6": (BF6, 128, 128, 2, 1)}),
 ]
 
 
@@ -170,6 +170,46 @@ def test_bf6_tile_orders_with_regrouped_edges(M, N, K, group_n, contig):
                 assert (info.kernel, info.group_n, info.contiguous_runs) == (_expected_bf6_kernel(BF6P), group_n, contig)
         assert torch.equal(out["bf6"], out["int8"])
         rows = np.r_[0:8, M // 2:M // 2 + 8, M - 8:M]
+        want = O.np_linear(x[rows], qw, ws, bias, 1.0)[0]
+        assert np.array_equal(out["bf6"][torch.from_numpy(rows).to(DEV)].cpu().numpy().view(np.uint16), want.view(np.uint16))
+    finally:
+        v.set_matrix_path(old)
+        torch.cuda.empty_cache()
+
+
+@pytest.mark.parametrize("M,K,N,tile", [
+    (300, 192, 384, 128),       # a handful of tiles, ragged M, K of one and a half steps
+    (512, 6144 - 128, 3072, 128),  # 47 K steps, 24 big tiles
+    (32768, 256, 256, 128),     # exactly 128 big tiles: the last problem that takes small ones; one tile column
+    (33024, 256, 256, 256),     # 129 big tiles
+    (2048 + 9, 1536, 10240, 256),  # 360 big tiles, too uneven for the tile-walking kernel's fixed places or not: either big kernel
+    (128, 64, 128, 128),        # one tile, one k-block
+])
+def test_bf6_tile_size_follows_the_problem_size(M, K, N, tile):
+    """Problems of at most 128 tiles of 256 x 256 (half a tile per CU) run the bf6 GEMM with 128 x 128 tiles, two
+    workgroups of four waves per CU; larger ones with 256 x 256.  Every output element against the int8 path, sampled
+    rows against the oracle, and the tile size the library reports."""
+    from dsaquant_amd import _lib
+    from dsaquant_amd.kernels import vdm_w4a4 as v
+
+    assert v.is_available(), v.load_error()
+    rng = np.random.default_rng(M + N + K)
+    qw = rng.integers(-8, 8, (N, K), dtype=np.int8)
+    x = O.synth_linear(M, K, 128, seed=K)[0]
+    _, _, ws, bias = O.synth_linear(1, 64, N, seed=K + 1)
+    print(f"tile size M={M} K={K} N={N}", flush=True)
+    old = v.matrix_path()
+    try:
+        out = {}
+        for path in ("bf6", "int8"):
+            v.set_matrix_path(path)
+            out[path] = v.linear_vdm_w4a4(_dev(x), _dev(O.np_pack_wgt_v1(qw)), _dev(O.np_pack_wscales_v1(ws, K)), _dev(bias), clip_ratio=1.0)
+            if path == "bf6":
+                info = _lib.last_gemm_launch()
+                assert (info.tile_m, info.tile_n) == (tile, tile), f"launcher chose {info.tile_m} x {info.tile_n}"
+                assert info.kernel == BF6 if tile == 128 else info.kernel in (BF6, BF6P)
+        assert torch.equal(out["bf6"], out["int8"])
+        rows = np.unique(np.r_[0:min(M, 8), M // 2:min(M, M // 2 + 8), max(0, M - 8):M])
         want = O.np_linear(x[rows], qw, ws, bias, 1.0)[0]
         assert np.array_equal(out["bf6"][torch.from_numpy(rows).to(DEV)].cpu().numpy().view(np.uint16), want.view(np.uint16))
     finally:

@@ -500,19 +500,19 @@ def test_cache_keys_work_for_tensors_made_under_inference_mode():
 
 
 def test_library_says_where_the_fp6_path_pays():
-    """vdmq_bf6_pays is a pure function of the sizes (no GPU work): the BASELINE shapes and the measured crossovers."""
+    """vdmq_bf6_pays is a pure function of the sizes (no GPU work): with a small-tile configuration in the GEMM it is
+    the row length alone that decides (the quantizer that writes 6-bit blocks is the slower one on short rows)."""
     from dsaquant_amd import _lib
 
     lib = _lib.load()
     pays = lambda M, N, K: bool(lib.vdmq_bf6_pays(M, N, K))  # noqa: E731
     assert pays(75600, 15360, 5120) and pays(75600, 5120, 13824) and pays(32760, 1536, 1536) and pays(27280, 3072, 14336)
-    assert pays(2048, 5120, 5120)            # 160 tiles, long K
-    assert not pays(4096, 4608, 1536)        # config 0: 288 tiles, short K
-    assert pays(4096, 1536, 8960)            # 96 tiles, long K
-    assert not pays(2048, 1536, 8960)        # 48 tiles, narrow N
-    assert pays(512, 10240, 5120)            # the skinny cross-attention K/V case of the 14B model: wide N, long K
-    assert not pays(512, 3072, 1536)         # the same of the 1.3B model
-    assert not pays(0, 128, 64) and not pays(-1, 128, 64)
+    assert pays(4096, 4608, 1536)            # config 0
+    assert pays(512, 10240, 5120)            # the skinny cross-attention K/V case of the 14B model
+    assert pays(512, 3072, 1536)             # the same of the 1.3B model
+    assert pays(1, 128, 1280) and not pays(1, 128, 1216)
+    assert not pays(32768, 5120, 1024) and not pays(257, 128, 64)
+    assert not pays(0, 128, 5120) and not pays(-1, 128, 5120)
 
 
 def test_bf6_tile_order_takes_every_tile_once(tmp_path):

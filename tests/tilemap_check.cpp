@@ -1,6 +1,8 @@
 // Host-side check of the bf6 GEMM's tile order (dsaquant_amd/csrc/vdmq_bf6_tilemap.h): for every grid of output tiles
 // in a range, both main super-tile shapes, edges regrouped or not, and the three ways the super-tile sequence is dealt to the XCDs, each tile is
-// taken exactly once, by a place inside the grid, and the closed-form tile counts agree with the enumeration.
+// taken exactly once, by a place inside the grid, and the closed-form tile counts agree with the enumeration.  Super-tiles
+// of 32 places (the 256 x 256 tiles' kernels) on the full range; of 1 ... 64 places (what the launcher picks for the
+// few 128 x 128 tiles of a small problem) on a smaller one.
 // Prints "ok <cases>" or the first disagreement; built and run by tests/test_host.py.
 #include <cstdio>
 #include <vector>
@@ -9,8 +11,8 @@
 
 using namespace vdmq;
 
-static int check(int tiles_m, int tiles_n, int gn_log2, int mode, bool regroup) {
-    const int per_log2 = 5, per = 1 << per_log2;
+static int check(int tiles_m, int tiles_n, int gn_log2, int mode, bool regroup, int per_log2 = 5) {
+    const int per = 1 << per_log2;
     Bf6TileMap tm;
     bf6_tilemap_shape(tm, tiles_m, tiles_n, per_log2, gn_log2, regroup);
     tm.contig = 0;
@@ -64,6 +66,22 @@ int main() {
                 if (int e = check(b[0], b[1], gn_log2, mode, regroup)) return std::printf("tiles %d x %d, columns per group %d, regrouped %d, mode %d: check %d failed\n", b[0], b[1], 1 << gn_log2, regroup, mode, e), 1;
             }
         }
+    for (int per_log2 = 0; per_log2 <= 6; ++per_log2) {
+        if (per_log2 == 5) continue;
+        for (int variant = 0; variant < 4; ++variant)
+            for (int mode = 0; mode < 3; ++mode) {
+                const int gn_log2 = 1 + variant % 2 < per_log2 ? 1 + variant % 2 : per_log2;
+                const bool regroup = variant >= 2;
+                for (int m = 1; m <= 40; ++m)
+                    for (int n = 1; n <= 40; ++n, ++cases)
+                        if (int e = check(m, n, gn_log2, mode, regroup, per_log2)) return std::printf("tiles %d x %d, %d places, columns per group %d, regrouped %d, mode %d: check %d failed\n", m, n, 1 << per_log2, 1 << gn_log2, regroup, mode, e), 1;
+                const int small[][2] = {{4, 80}, {2, 120}, {256, 2}, {128, 4}, {1, 512}, {512, 1}, {3, 170}};
+                for (auto &b : small) {
+                    ++cases;
+                    if (int e = check(b[0], b[1], gn_log2, mode, regroup, per_log2)) return std::printf("tiles %d x %d, %d places, columns per group %d, regrouped %d, mode %d: check %d failed\n", b[0], b[1], 1 << per_log2, 1 << gn_log2, regroup, mode, e), 1;
+                }
+            }
+    }
     std::printf("ok %ld\n", cases);
     return 0;
 }
