@@ -130,11 +130,12 @@ def linear_ln_vdm_w4a4(
 
 
 class QuantizedInput:
-    """A linear's input that is already quantized per token (native int4 rows and fp16
-    scales): one quantizer launch serves every linear that reads the same tensor with the
-    same clip ratio.  The cross-attention context is such a tensor -- every block's
-    ``attn2`` K/V projection reads ``encoder_hidden_states`` (dit_block.py:109 of the
-    reference), which the reference quantizes again in each of them."""
+    """A linear's input that is already quantized per token (fp16 scales and the operand form
+    of the matrix path its row length takes: 6-bit blocks or native int4 rows): one quantizer
+    launch serves every linear that reads the same tensor with the same clip ratio.  The
+    cross-attention context is such a tensor -- every block's ``attn2`` K/V projection reads
+    ``encoder_hidden_states`` (dit_block.py:109 of the reference), which the reference
+    quantizes again in each of them."""
 
     def __init__(self, x: torch.Tensor, clip_ratio: float = 1.0):
         self.shape = tuple(x.shape)
@@ -143,8 +144,10 @@ class QuantizedInput:
         _k._require(x_2d.is_cuda, "input must be a CUDA tensor")
         self.M, self.K = x_2d.shape
         self.device = x_2d.device
+        # (the path of a linear depends on its row length alone, so it is known before any weight is)
+        self.bf6 = _k._use_bf6(self.M, 128, self.K)
         if self.M:
-            self.qact, self.scales = _k._quantize_for_gemm(x_2d, self.clip_ratio, _lib.VDMQ_ACT_NONE, False, None)
+            self.qact, self.scales = _k._quantize_for_gemm(x_2d, self.clip_ratio, _lib.VDMQ_ACT_NONE, self.bf6, None)
         else:
             self.qact = self.scales = None
 
@@ -166,7 +169,7 @@ def linear_fused(
 
     ``x`` is a tensor (optionally with ``act="gelu_tanh"`` applied to it inside the
     quantizer), an ``LnInput`` or a ``QuantizedInput`` (whose clip ratio must be the
-    layer's; the int8 matrix path then runs whatever the problem size).  ``gate`` (fp16, one ``[N]`` vector per batch element
+    layer's; the GEMM then runs on the matrix path the input was quantized for).  ``gate`` (fp16, one ``[N]`` vector per batch element
     or per token) and ``residual`` (fp16, shaped like the output) are folded into the
     GEMM epilogue as the two fp16 tensor operations of the reference's
     ``hidden_states + attn_output * gate`` (dit_block.py:102, :107, :112); either may
@@ -230,7 +233,7 @@ def linear_fused(
     with torch.cuda.device(dev):
         out = torch.empty((M, N) if split_cols is None else (N // split_cols, M, split_cols), dtype=torch.float16, device=dev)
         if M and isinstance(pre, QuantizedInput):
-            _k._gemm_dispatch(pre.qact, pre.scales, False, weight, b, out, K, gate=g2, rows_per_gate=rows_per_gate, residual=r2)
+            _k._gemm_dispatch(pre.qact, pre.scales, pre.bf6, weight, b, out, K, gate=g2, rows_per_gate=rows_per_gate, residual=r2)
         elif M:
             bf6 = _k._use_bf6(M, N, K)
             operand, scales = _k._quantize_for_gemm(x_2d, clip_ratio, act_code, bf6, None if pre is None else pre._args())

@@ -208,3 +208,25 @@ def test_forms_kept_on_inference_tensors_are_not_trusted_at_prepare_time():
         yb = v.linear_vdm_w4a4(_dev(x), q, s, _dev(bias), clip_ratio=1.0)
     assert np.array_equal(ya.cpu().numpy().view(np.uint16), O.np_linear(x, qw_a, ws, bias, 1.0)[0].view(np.uint16))
     assert np.array_equal(yb.cpu().numpy().view(np.uint16), O.np_linear(x, qw_b, ws, bias, 1.0)[0].view(np.uint16))
+
+
+@pytest.mark.parametrize("K,bf6", [(1536, True), (256, False)])
+def test_shared_quantized_input_takes_the_path_of_its_row_length(K, bf6):
+    """An input quantized once for several linears (fused_ops.QuantizedInput: the cross-attention context) is held in
+    the operand form of the matrix path the library picks for its row length, and every linear fed by it gives the
+    bits of the linear that quantizes for itself -- and of the oracle."""
+    from dsaquant_amd import fused_ops
+    from dsaquant_amd.kernels import vdm_w4a4 as v
+
+    assert v.is_available(), v.load_error()
+    M = 512
+    x = O.synth_linear(M, K, 128, seed=K)[0]
+    shared = fused_ops.QuantizedInput(_dev(x), 1.0)
+    assert shared.bf6 is bf6 and v.matrix_path() == "auto"
+    for N, seed in ((384, 1), (3072, 2)):
+        _, qw, ws, bias = O.synth_linear(1, K, N, seed=seed)
+        qv1, sv1, b = _dev(O.np_pack_wgt_v1(qw)), _dev(O.np_pack_wscales_v1(ws, K)), _dev(bias)
+        got = fused_ops.linear_fused(shared, qv1, sv1, b, 1.0)
+        assert torch.equal(got, v.linear_vdm_w4a4(_dev(x), qv1, sv1, b, clip_ratio=1.0))
+        want = O.np_linear(x, qw, ws, bias, 1.0)[0]
+        assert np.array_equal(got.cpu().numpy().view(np.uint16), want.view(np.uint16))
