@@ -171,7 +171,7 @@ int vdmq_gemm_w4a4_acc(const void *qact, const void *wq, int32_t *acc, int64_t M
  * and tuning: the choice never changes a result bit.  Returns VDMQ_EINVAL when
  * nothing was launched yet. */
 #define VDMQ_KERNEL_GEMM_W4A4 1           /* int8 matrix path */
-#define VDMQ_KERNEL_GEMM_BF6 2            /* bf6 matrix path, one workgroup per tile */
+#define VDMQ_KERNEL_GEMM_BF6 2            /* bf6 matrix path, one workgroup per tile (256 x 256, or 128 x 128 for small problems) */
 #define VDMQ_KERNEL_GEMM_BF6_PERSISTENT 3 /* bf6 matrix path, one workgroup per CU walking tiles */
 typedef struct vdmq_gemm_launch_info {
     int kernel;                 /* VDMQ_KERNEL_* */
