@@ -312,7 +312,7 @@ __device__ __forceinline__ void bf6_epilogue(const v16f (&acc)[Cfg::NI][Cfg::MI]
 
 // Timing aid, off in the shipped library: a build with -DVDMQ_DBG_TIMELINE stamps the 100 MHz clock at five points of
 // every tile of the tile-walking kernel (thread 0 of each workgroup, first 64 tiles) into a device array that
-// vdmq_debug_timeline copies out: K loop, next tile's requests, epilogue, wait at the barrier.
+// vdmq_debug_timeline copies out: K loop, next tile's requests, epilogue, wait at the barrier (and the kernel's entry).
 #ifdef VDMQ_DBG_TIMELINE
 __device__ uint64_t g_timeline[256][64][6];
 #define VDMQ_STAMP(tile, i) do { if (threadIdx.x == 0 && (tile) < 64) g_timeline[blockIdx.x][tile][i] = wall_clock64(); } while (0)
@@ -455,6 +455,7 @@ __global__ __launch_bounds__(Cfg::kWaves * 64, (Cfg::kWaves * Cfg::kOcc + 3) / 4
     constexpr int kLoads = Cfg::kLoads, kStageBytes = Cfg::kStageBytes;
     static_assert(S == 3, "the prefetch under the epilogue uses ring slots 1 and 2");
     extern __shared__ __attribute__((aligned(1024))) uint8_t lds[];
+    VDMQ_STAMP(0, 5); /* kernel entry */
     const int lane = threadIdx.x & 63, wave = __builtin_amdgcn_readfirstlane(threadIdx.x >> 6);
     const int wn = wave % kWavesN, wm = wave / kWavesN;
     const int wm0 = wm * MI * 32, wn0 = wn * NI * 32;
@@ -469,21 +470,22 @@ __global__ __launch_bounds__(Cfg::kWaves * 64, (Cfg::kWaves * Cfg::kOcc + 3) / 4
         if (!bf6_tilemap_locate(tmap, st, place, tile_m, tile_n)) tile_m = -1;
         return true;
     };
-    // The workgroup's tiles, round by round, are worked out once, 512 rounds at a time by the 512 threads, and kept in
-    // LDS: between two tiles -- matrix pipes idle, every wave running the same scalar code -- finding the next tile
-    // is then one LDS read instead of the map's divisions and case distinctions (150 scalar instructions per wave
-    // and tile).  Entry: tile_m (-1: no tile at this place in that round, -2: no such round), tile_n.  Launches with
-    // more rounds than the table holds work the map out tile by tile as before.
+    // The workgroup's tiles, round by round, are worked out once, a round per thread, and kept in LDS: between two
+    // tiles -- matrix pipes idle, every wave running the same scalar code -- finding the next tile is then one LDS
+    // read instead of the map's divisions and case distinctions (150 scalar instructions per wave and tile).  Entry:
+    // tile_m (-1: no tile at this place in that round, -2: no such round), tile_n.  Launches with more rounds than the
+    // table holds work the map out tile by tile as before.  The table is filled while the first tile's loads are on
+    // their way (below), for the rounds this XCD has and the entry behind them.
     int2 *tile_table = reinterpret_cast<int2 *>(lds + Cfg::kTableOffset);
-    const bool tabled = (tmap.contig ? tmap.start[xcd + 1] - tmap.start[xcd] : (tmap.total_super + kXcds - 1) / kXcds) < kTileTableEntries;
-    if (tabled) {
-        for (int e = threadIdx.x; e < kTileTableEntries; e += Cfg::kWaves * 64) {
+    const int my_rounds = tmap.contig ? tmap.start[xcd + 1] - tmap.start[xcd] : (tmap.total_super + kXcds - 1) / kXcds;
+    const bool tabled = my_rounds < kTileTableEntries;
+    auto fill_tile_table = [&] {
+        for (int e = threadIdx.x; tabled && e <= my_rounds; e += Cfg::kWaves * 64) {
             int2 ent = {-2, 0};
             if (!locate(e, ent.x, ent.y)) ent.x = -2;
             tile_table[e] = ent;
         }
-        __syncthreads();
-    }
+    };
     // Advances seq to the next existing tile; `skipped` counts the super-tiles passed on the way in which this place
     // has no tile (a ragged edge).
     auto next_tile = [&](int &seq, int &tile_m, int &tile_n, int &skipped) -> bool {
@@ -557,8 +559,11 @@ __global__ __launch_bounds__(Cfg::kWaves * 64, (Cfg::kWaves * Cfg::kOcc + 3) / 4
     };
     v16f acc[NI][MI];
 
+    // (the first tile is found the long way: the table does not exist yet)
     int seq = -1, tile_m = -1, tile_n = 0, skipped = 0;
-    if (!next_tile(seq, tile_m, tile_n, skipped)) return;
+    do {
+        if (!locate(++seq, tile_m, tile_n)) return; /* the same for the whole workgroup */
+    } while (tile_m < 0);
     __amdgpu_buffer_rsrc_t src[kLoads];
     sources(src, tile_m, tile_n);
     bool k_reverse = tmap.contig && (seq & 1) != 0;
@@ -567,10 +572,11 @@ __global__ __launch_bounds__(Cfg::kWaves * 64, (Cfg::kWaves * Cfg::kOcc + 3) / 4
 #pragma unroll
         for (int s = 0; s < S; ++s)
             if (s < ksteps) issue(src, k_reverse, s, s);
-        if (ksteps >= S) /* stages 0 and 1, as for every later tile */
-            __builtin_amdgcn_s_waitcnt(waitcnt_imm(kLoads * (S - 2), 15));
+        fill_tile_table();
+        if (ksteps >= S) /* stages 0 and 1, as for every later tile; the table's writes */
+            __builtin_amdgcn_s_waitcnt(waitcnt_imm(kLoads * (S - 2), 0));
         else
-            __builtin_amdgcn_s_waitcnt(waitcnt_imm(0, 15));
+            __builtin_amdgcn_s_waitcnt(waitcnt_imm(0, 0));
         lds_barrier();
         side_publish(sd);
     }
