@@ -71,7 +71,7 @@ FP6_PEAK_TOPS = 10100.0  # MI355X dense FP6 MFMA, published
 TRAFFIC_FROM_PROFILES = {
     ("wan14b_720p_block", "int8"): {"gemm": 4315445555, "quant": 1379725133,
                                     "source": "profiles/gemm_w4a4_kernel+quantize_rows_kernel.wan14b_720p_block.md"},
-    ("wan14b_720p_block", "bf6"): {"gemm": 6469260928, "quant": 1517356237,
+    ("wan14b_720p_block", "bf6"): {"gemm": 6434431309, "quant": 1517356237,
                                    "source": "profiles/gemm_bf6_persistent_kernel+quantize_rows_kernel.wan14b_720p_block.md"},
 }
 TRAFFIC_UNIT = "bytes leaving L2 per launch, mean of the step's 4 launches; from traffic_source, not from this run"
@@ -82,7 +82,7 @@ WAN14B_720P = dict(M=75600, linears=[("qkv", 5120, 15360), ("o", 5120, 5120), ("
 WAN13B_480P = dict(M=32760, linears=[("qkv", 1536, 4608), ("o", 1536, 1536), ("ffn_up", 1536, 8960), ("ffn_down", 8960, 1536)])
 WAN5B = dict(M=27280, linears=[("qkv", 3072, 9216), ("o", 3072, 3072), ("ffn_up", 3072, 14336), ("ffn_down", 14336, 3072)])
 WORKLOADS = {"wan14b_720p_block": WAN14B_720P, "wan1.3b_480p_block": WAN13B_480P, "wan5b_704x1280_block": WAN5B}
-# single linears (BASELINE configs 0 and 3), timed next to the blocks
+# single linears (benchmark configurations 0 and 3), timed next to the blocks
 CASES = {"cfg0_qkv_m4096": dict(M=4096, linears=[("qkv", 1536, 4608)]),
          "cfg3_cross_kv_m512": dict(M=512, linears=[("cross_kv", 5120, 10240)]),
          "cfg3_qkv_ragged_m75637": dict(M=75637, linears=[("qkv", 5120, 15360)])}
