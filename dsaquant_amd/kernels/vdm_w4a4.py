@@ -372,7 +372,8 @@ def _prepared_weight(qweight: torch.Tensor, wscales: torch.Tensor) -> PreparedWe
 
 def prepare_weight(qweight: torch.Tensor, wscales: torch.Tensor, tokens: Optional[int] = None, path: Optional[str] = None) -> PreparedWeight:
     """Relayout a packed weight now (load time, a known stream) instead of at its first call.  ``tokens``: the number
-    of rows its calls will have, which decides the matrix path under "auto" (default: a video-sized sequence)."""
+    of rows its calls will have, passed on to the library's rule for the matrix path under "auto" (which at present
+    looks at the row length only; default: a video-sized sequence)."""
     if qweight.is_inference():
         release_prepared(qweight, concatenations=True)  # written in place since? not visible: see _version_of
     pw = _prepared_weight(qweight, wscales)
@@ -423,8 +424,9 @@ def _native_weights(qweight: torch.Tensor, wscales: torch.Tensor) -> Tuple[torch
 # "int8": v_mfma_i32_32x32x32_i8 on nibbles widened in registers.  "bf6": v_mfma_f32_32x32x64_f8f6f4 on 6-bit
 # floats (twice the rate, no widening work; every int4 value q is held as the E3M2 float q / 16, exactly, and the
 # fp32 accumulation of the products is exact too).
-# Both give bit-identical results.  "auto" asks the library (vdmq_bf6_pays: bf6 for problems with enough 256 x 256
-# output tiles, fewer when K is long, none needed when N is wide too).
+# Both give bit-identical results.  "auto" asks the library (vdmq_bf6_pays: bf6 from a row length of 1280 on, whatever
+# the other sizes -- its GEMM has a tile configuration for small problems, and only its quantizer is the slower one on
+# short rows).
 _MATRIX_PATH = os.environ.get("VDMQ_MATRIX_PATH", "auto")
 
 
