@@ -498,7 +498,18 @@ def main():
     per_linear = {args.workload: r["per_linear"]}
     if not args.no_extras:
         extra_steps, extra_warmup = max(10, args.steps // 4), 3
-        if path != "int8":  # the instruction the path was specified on: the same workload on the int8 matrix path
+
+        # The measurements beside the headline: each in a section of its own, so that a failure in one (out of memory on a
+        # smaller part, a missing package for the harness) is named in the line instead of costing the line.  The
+        # headline above is not guarded: without it there is nothing to report.
+        def section(name, body):
+            try:
+                body()
+            except Exception as e:  # noqa: BLE001 -- reported, not swallowed
+                roof[f"{name}_error"] = f"{type(e).__name__}: {e}"[:300]
+                print(f"bench.py: section {name} failed: {e!r}", file=sys.stderr)
+
+        def int8_section():  # the instruction the path was specified on: the same workload on the int8 matrix path
             r8 = run(args.workload, "int8", extra_steps, extra_warmup)
             result["int8_path"] = {"steps": extra_steps, "warmup": extra_warmup, "step_tops": round(r8["step_tops"], 1),
                                    "ms_per_step": round(r8["ms_per_step"], 4), "roofline": r8["roofline"], "quantizer": r8["quantizer"]}
@@ -506,44 +517,47 @@ def main():
             roof.update({"int8_path_achieved": r8["roofline"]["achieved"], "int8_path_peak": INT8_PEAK_TOPS,
                          "int8_path_frac": r8["roofline"]["frac"], "int8_path_kernel": r8["roofline"]["kernel"],
                          "int8_path_quantizer_frac": r8["quantizer"]["frac"], "int8_path_step_tops": round(r8["step_tops"], 1)})
-        result["workloads"] = {}
-        for other in sorted(WORKLOADS):
-            if other == args.workload:
-                continue
+
+        def workload_section(other):
             ro = run(other, args.matrix_path, extra_steps, extra_warmup)
-            result["workloads"][other] = {"M": WORKLOADS[other]["M"], "steps": extra_steps, "warmup": extra_warmup,
-                                          "step_tops": round(ro["step_tops"], 1), "ms_per_step": round(ro["ms_per_step"], 4),
-                                          "gemm_tops": ro["roofline"]["achieved"], "gemm_frac": ro["roofline"]["frac"],
-                                          "gemm_frac_of_int8_peak": ro["roofline"]["frac_of_int8_peak"],
-                                          "quant_gbs": ro["quantizer"]["achieved"], "quant_gbs_int4_bytes": ro["quantizer"]["achieved_int4_bytes"]}
+            result.setdefault("workloads", {})[other] = {
+                "M": WORKLOADS[other]["M"], "steps": extra_steps, "warmup": extra_warmup,
+                "step_tops": round(ro["step_tops"], 1), "ms_per_step": round(ro["ms_per_step"], 4),
+                "gemm_tops": ro["roofline"]["achieved"], "gemm_frac": ro["roofline"]["frac"],
+                "gemm_frac_of_int8_peak": ro["roofline"]["frac_of_int8_peak"],
+                "quant_gbs": ro["quantizer"]["achieved"], "quant_gbs_int4_bytes": ro["quantizer"]["achieved_int4_bytes"]}
             per_linear[other] = ro["per_linear"]
             k = SHORT[other]
             roof.update({f"{k}_gemm_achieved": ro["roofline"]["achieved"], f"{k}_gemm_frac": ro["roofline"]["frac"],
                          f"{k}_gemm_frac_of_int8_peak": ro["roofline"]["frac_of_int8_peak"], f"{k}_step_tops": round(ro["step_tops"], 1),
                          f"{k}_quantizer_frac_int4_bytes": ro["quantizer"]["frac_int4_bytes"]})
-        # single linears: launches of 15 ... 2400 us, so more repetitions for the short ones
-        result["cases"] = {}
-        for case, spec in CASES.items():
+
+        def case_section(case, spec):  # single linears: launches of 15 ... 2400 us, so more repetitions for the short ones
             steps_c = 200 if spec["M"] <= 4096 else extra_steps
             rc = run(case, args.matrix_path, steps_c, 5)
             lin = next(iter(rc["per_linear"].values()))
-            result["cases"][case] = {"M": spec["M"], "K": lin["K"], "N": lin["N"], "steps": steps_c, "kernel": lin["kernel"],
-                                     "gemm_us": round(lin["gemm_ms"] * 1e3, 2), "gemm_tops": lin["gemm_tops"],
-                                     "quant_us": round(lin["quant_ms"] * 1e3, 2), "quant_gbs_int4_bytes": lin["quant_gbs_int4_bytes"],
-                                     "linear_tops": round(rc["step_tops"], 1), "linear_us": round(rc["ms_per_step"] * 1e3, 2)}
+            result.setdefault("cases", {})[case] = {
+                "M": spec["M"], "K": lin["K"], "N": lin["N"], "steps": steps_c, "kernel": lin["kernel"],
+                "gemm_us": round(lin["gemm_ms"] * 1e3, 2), "gemm_tops": lin["gemm_tops"],
+                "quant_us": round(lin["quant_ms"] * 1e3, 2), "quant_gbs_int4_bytes": lin["quant_gbs_int4_bytes"],
+                "linear_tops": round(rc["step_tops"], 1), "linear_us": round(rc["ms_per_step"] * 1e3, 2)}
             roof.update({f"{case}_gemm_achieved": lin["gemm_tops"], f"{case}_gemm_frac": round(lin["gemm_tops"] / rc["roofline"]["peak"], 4),
                          f"{case}_linear_tops": round(rc["step_tops"], 1), f"{case}_kernel": lin["kernel"]})
-        # the quantizer against a kernel that only streams the same mix of reads and writes over the same volumes
-        sc = stream_ceiling(torch, lib, dev, wl["M"], [k for _, k, _ in wl["linears"]], path != "int8")
-        result["stream_ceiling"] = sc
-        roof.update({"quantizer_stream_ceiling_gbs": sc["gbs"], "quantizer_stream_mix": sc["mix"],
-                     "quantizer_frac_of_stream_ceiling": round(r["quantizer"]["achieved"] / sc["gbs"], 4),
-                     "stream_copy_gbs": sc["copy_gbs"], "stream_read_only_gbs": sc["read_only_gbs"]})
-        ceiling = mfma_ceiling(torch, lib, dev)
-        result["mfma_ceiling"] = ceiling
-        roof.update({"mfma_only_loop_bf6_workload_data": ceiling["bf6"]["workload"]["tops"],
-                     "mfma_only_loop_int8_workload_data": ceiling["int8"]["workload"]["tops"]})
-        if not args.no_config4:
+
+        def stream_section():  # the quantizer against a kernel that only streams the same mix of reads and writes over the same volumes
+            sc = stream_ceiling(torch, lib, dev, wl["M"], [k for _, k, _ in wl["linears"]], path != "int8")
+            result["stream_ceiling"] = sc
+            roof.update({"quantizer_stream_ceiling_gbs": sc["gbs"], "quantizer_stream_mix": sc["mix"],
+                         "quantizer_frac_of_stream_ceiling": round(r["quantizer"]["achieved"] / sc["gbs"], 4),
+                         "stream_copy_gbs": sc["copy_gbs"], "stream_read_only_gbs": sc["read_only_gbs"]})
+
+        def mfma_section():
+            ceiling = mfma_ceiling(torch, lib, dev)
+            result["mfma_ceiling"] = ceiling
+            roof.update({"mfma_only_loop_bf6_workload_data": ceiling["bf6"]["workload"]["tops"],
+                         "mfma_only_loop_int8_workload_data": ceiling["int8"]["workload"]["tops"]})
+
+        def config4_section():
             import contextlib
 
             import bench_dit
@@ -562,6 +576,18 @@ def main():
             roof.update({"config4_ms_per_step": c4["ms_per_step"], "config4_w4a4_share": c4["value"], "config4_attention_share": c4["attention_share"],
                          "config4_w4a4_calls_per_forward": c4["w4a4_calls_per_forward"], "config4_unfused_ms_per_step": c4_plain["ms_per_step"],
                          "config4_unfused_w4a4_share": c4_plain["value"]})
+
+        if path != "int8":
+            section("int8_path", int8_section)
+        for other in sorted(WORKLOADS):
+            if other != args.workload:
+                section(SHORT[other], lambda other=other: workload_section(other))
+        for case, spec in CASES.items():
+            section(case, lambda case=case, spec=spec: case_section(case, spec))
+        section("stream_ceiling", stream_section)
+        section("mfma_only_loop", mfma_section)
+        if not args.no_config4:
+            section("config4", config4_section)
     if not args.details:  # every figure of these objects that matters is a flat key of `roofline`
         for key in ("int8_path", "workloads", "cases", "stream_ceiling", "mfma_ceiling", "config4"):
             result.pop(key, None)
