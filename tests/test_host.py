@@ -530,3 +530,44 @@ def test_bf6_tile_order_takes_every_tile_once(tmp_path):
                     str(root / "tests" / "tilemap_check.cpp"), "-o", str(exe)], check=True)
     res = subprocess.run([str(exe)], stdout=subprocess.PIPE, text=True)
     assert res.returncode == 0 and res.stdout.startswith("ok "), res.stdout
+
+
+def test_header_is_plain_c_and_a_c_host_links_the_library(tmp_path):
+    """include/vdmq.h is what a C or C++ host of the reference's kernels would include: it must compile as C99 with
+    every warning an error, and a C program must link libvdmq.so by its declarations alone.  The program calls the
+    entry points that need no GPU (sizes, the version, the path rule, a rejected shape and its message)."""
+    import shutil
+    import subprocess
+
+    from dsaquant_amd import _lib
+
+    cc = shutil.which("gcc") or shutil.which("cc")
+    if cc is None:
+        pytest.skip("no host C compiler")
+    _lib.load()  # built, or this raises
+    root = Path(__file__).resolve().parent.parent
+    src = tmp_path / "host.c"
+    src.write_text(r'''
+#include <stdio.h>
+#include <string.h>
+#include "vdmq.h"
+int main(void) {
+    vdmq_gemm_launch_info info;
+    if (vdmq_version() != VDMQ_VERSION) return 1;
+    if (vdmq_k_padded(64) != 256 || vdmq_k_padded(5120) != 5120) return 2;
+    if (vdmq_workspace_bytes(0, 64) < 0) return 3;
+    if (vdmq_bf6_bytes(32, 128) != 32 * 128 * 3 / 4) return 4;
+    if (!vdmq_bf6_pays(75600, 15360, 5120) || vdmq_bf6_pays(75600, 15360, 64)) return 5;
+    if (vdmq_gemm_w4a4(NULL, NULL, NULL, NULL, NULL, NULL, VDMQ_OUT_F16, 16, 100, 64, 100, NULL) == VDMQ_OK) return 6; /* N % 128 */
+    if (strlen(vdmq_last_error()) == 0) return 7;
+    if (vdmq_last_gemm_launch(&info) == VDMQ_OK) return 8; /* nothing was launched */
+    printf("ok %d\n", vdmq_version());
+    return 0;
+}
+''')
+    exe = tmp_path / "host"
+    lib_dir = _lib.LIB_PATH.parent
+    subprocess.run([cc, "-std=c99", "-pedantic", "-Wall", "-Wextra", "-Werror", "-I", str(root / "include"), str(src), "-o", str(exe),
+                    "-L", str(lib_dir), "-lvdmq", f"-Wl,-rpath,{lib_dir}", "-L/opt/rocm/lib", "-Wl,-rpath,/opt/rocm/lib"], check=True)
+    res = subprocess.run([str(exe)], stdout=subprocess.PIPE, text=True)
+    assert res.returncode == 0 and res.stdout.startswith("ok "), (res.returncode, res.stdout)
